@@ -1,0 +1,197 @@
+/*
+ * mole_hip.h - C ABI of the MI355X (gfx950) MoE-layer hot path.
+ *
+ * This is the drop-in boundary for MOLE's single-GPU MoE layer.  Every entry point replaces a
+ * piece of what the reference reaches through pybind (MOLE/cpp/core.cpp:1347-1469) or through
+ * the third-party tutel package (MOLE/moe/layer.py:445-458).  Rules of the boundary:
+ *
+ *   - plain C: pointers, sizes, enums.  No C++ types, no torch types, no exceptions, no exit().
+ *   - every function returns 0 on success, a positive hipError_t, or a negative MOLE_E_* code;
+ *     mole_last_error_string() describes the last failure on the calling thread.
+ *   - the caller allocates every buffer (inputs, outputs, saved activations, workspaces).  The
+ *     library owns only what mole_unimem_create() makes: the slot pool, its copy stream and events.
+ *   - all kernels are enqueued on the caller's stream (a hipStream_t passed as void*) and never
+ *     synchronise the host; the only blocking calls are mole_unimem_sync_tran() and the
+ *     create/destroy pair.
+ *   - all tensors are dense row-major.  Row pointers of x/xd/o/h must be 16-byte aligned
+ *     (M and F multiples of 8 for bf16, of 4 for fp32).
+ *
+ * Symbols: S tokens, M model dim (embed_dim), E experts, k top-k, F ffn dim, C capacity.
+ */
+#ifndef MOLE_HIP_H
+#define MOLE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *mole_stream_t; /* a hipStream_t; NULL is the default stream */
+
+enum { MOLE_F32 = 0, MOLE_BF16 = 1 };
+/* where expert e's rows start: PADDED is the reference's [E, C, M] layout (row = e*C + loc),
+ * RAGGED packs the kept rows of the experts back to back (row = offsets[e] + loc). */
+enum { MOLE_LAYOUT_PADDED = 0, MOLE_LAYOUT_RAGGED = 1 };
+/* derivative used for the GELU in the backward pass.  TANH is what the reference compiles
+ * (MOLE/cpp/define.hpp:6 -> MOLE/cpp/gelu.cu:3-14); EXACT is the erf derivative
+ * (at::gelu_backward, MOLE/cpp/core.cpp:396). */
+enum { MOLE_GELU_BWD_TANH = 0, MOLE_GELU_BWD_EXACT = 1 };
+
+enum {
+    MOLE_E_INVALID = -1,   /* bad argument (null pointer, size out of range, misalignment) */
+    MOLE_E_WORKSPACE = -2, /* workspace too small */
+    MOLE_E_STATE = -3,     /* call does not fit the handle's state (e.g. pool exhausted) */
+    MOLE_E_NOMEM = -4
+};
+
+#define MOLE_MAX_TOPK 16
+#define MOLE_MAX_EXPERTS 1024
+
+int mole_version(void);
+const char *mole_last_error_string(void);
+
+/* ------------------------------------------------------------------------------------------
+ * Gate.  Replaces MOLETopk.forward (MOLE/utils/Ugate.py:11-14): scores = softmax(logits).
+ * logits [S,E] fp32 (x . Wg^T, produced by mole_gemm_nt or any GEMM); logit_bias [E] or NULL.
+ * mole_gate_bwd replaces the autograd of the gate normalisation inside tutel's
+ * extract_critical and, with through_softmax != 0, of the softmax as well: from dgates [k,S]
+ * it produces d(scores) [S,E] (through_softmax == 0) or d(logits) [S,E].
+ * ------------------------------------------------------------------------------------------ */
+int mole_softmax_fwd(const float *logits, const float *logit_bias, int S, int E, float *scores,
+                     mole_stream_t stream);
+int mole_gate_bwd(const float *dgates, const float *scores, const int32_t *idx, int S, int E,
+                  int k, int normalize_gate, int through_softmax, float *dout, mole_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Routing.  Replaces tutel.impls.fast_dispatch.extract_critical (call site
+ * MOLE/moe/layer.py:445-446): top-k with ties to the lowest expert index, gate values
+ * (normalised over the k choices when k > 1 and normalize_gate), per-choice per-expert counts,
+ * k-major locations, capacity, and the dispatch permutation.
+ *
+ *   scores   [S,E] fp32 in
+ *   idx      [k,S] int32 out   chosen expert of every (choice, token)
+ *   loc      [k,S] int32 out   location inside the expert (before the capacity test)
+ *   gates    [k,S] fp32  out
+ *   row      [k,S] int32 out   destination row in the dispatched buffer, -1 when dropped
+ *   counts   [k,E] int32 out
+ *   kept_rows[E]   int32 out   n[e] = min(sum_j counts[j,e], C)
+ *   offsets  [E+1] int32 out   first row of expert e (RAGGED: prefix sum of kept_rows,
+ *                              PADDED: e*C); offsets[E] = total rows
+ *   capacity [1]   int32 out   C, on the device (capacity_factor <= 0 makes it data dependent)
+ *   l_aux    [1]   fp32  out   E/S^2 * sum_e (sum_i scores[i,e]) * counts[0,e]; may be NULL
+ *
+ * capacity_factor > 0: C = k*int(cf*ceil(S/E)); == 0: C = max(loc)+1; < 0: the smaller of both;
+ * C is then rounded up to `alignment`.  k is clipped to E by the caller (k <= E required).
+ * ------------------------------------------------------------------------------------------ */
+size_t mole_route_workspace_bytes(int S, int E, int k);
+int mole_route(const float *scores, int S, int E, int k, float capacity_factor, int normalize_gate,
+               int alignment, int layout, int32_t *idx, int32_t *loc, float *gates, int32_t *row,
+               int32_t *counts, int32_t *kept_rows, int32_t *offsets, int32_t *capacity,
+               float *l_aux, void *workspace, size_t workspace_bytes, mole_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Dispatch / combine.  Replace tutel fast_encode / fast_decode and their backward
+ * (call sites MOLE/moe/layer.py:448-449, 457-458).  `row` is mole_route's permutation.
+ *
+ *   dispatch_fwd : xd[row[j,i],:] = x[i,:]                      for kept pairs
+ *   dispatch_bwd : dx[i,:] = sum_j dxd[row[j,i],:]  (+ dlogits[i,:] . Wg  when dlogits != NULL,
+ *                  the gate's contribution to the input gradient, Wg [E,M] fp32)
+ *   combine_fwd  : y[i,:] = sum_j gates[j,i] * o[row[j,i],:]    (zeros for a fully dropped token)
+ *   combine_bwd  : d_o[row[j,i],:] = gates[j,i]*dy[i,:];  dgates[j,i] = <dy[i,:], o[row[j,i],:]>
+ *                  (0 for dropped pairs)
+ *   zero_pad_rows: zero the rows of a [total_rows, M] buffer that no kept pair owns
+ *                  (rows offsets[e]+kept_rows[e] .. offsets[e+1]), which the reference's zeroed
+ *                  [E,C,M] buffers contain.
+ * ------------------------------------------------------------------------------------------ */
+int mole_dispatch_fwd(const void *x, int dtype, const int32_t *row, int S, int M, int k, void *xd,
+                      mole_stream_t stream);
+int mole_dispatch_bwd(const void *dxd, int dtype, const int32_t *row, int S, int M, int k,
+                      const float *dlogits, const float *wg, int E, void *dx, mole_stream_t stream);
+int mole_combine_fwd(const void *o, int dtype, const int32_t *row, const float *gates, int S,
+                     int M, int k, void *y, mole_stream_t stream);
+int mole_combine_bwd(const void *dy, const void *o, int dtype, const int32_t *row,
+                     const float *gates, int S, int M, int k, void *d_o, float *dgates,
+                     mole_stream_t stream);
+int mole_zero_pad_rows(void *buf, int dtype, const int32_t *kept_rows, const int32_t *offsets,
+                       int E, int M, mole_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Grouped expert FFN.  Replaces _BatchRecord::bffn_fwd / bffn_bwd / bffn_bwd_acc
+ * (MOLE/cpp/core.cpp:344-356, 381-414, 457-491) and the GELU-backward kernel
+ * (MOLE/cpp/gelu.cu:16-58), with bias, GELU and GELU' fused into the GEMM epilogues.
+ *
+ * Expert e owns rows offsets[e] .. offsets[e]+kept_rows[e] of every [rows, *] buffer; both
+ * arrays live on the device.  max_rows bounds offsets[e]+kept_rows[e] (it sizes the launch).
+ *   w1 [E,F,M]  b1 [E,F]  w2 [E,F,M] (used as a . w2)  b2 [E,M]         (dtype)
+ *   fwd: h = xd.w1^T + b1 ; a = gelu_erf(h) ; out = a.w2 + b2             h,a [rows,F]  out [rows,M]
+ *   bwd: g_w2 = a^T.go ; t = (go.w2^T) * gelu'(h) ; g_b2 = sum go ; g_w1 = t^T.xd ;
+ *        g_b1 = sum t ; gx = t.w1     (t [rows,F] is caller-provided scratch; gx may be NULL)
+ *        accumulate != 0 adds into g_* instead of overwriting (bffn_bwd_acc).
+ * fp32 accumulation throughout; bf16 buffers are rounded once, on store.
+ * ------------------------------------------------------------------------------------------ */
+int mole_ffn_fwd(const void *xd, int dtype, const int32_t *offsets, const int32_t *kept_rows, int E,
+                 int max_rows, int M, int F, const void *w1, const void *b1, const void *w2,
+                 const void *b2, void *h, void *a, void *out, mole_stream_t stream);
+int mole_ffn_bwd(const void *go, const void *xd, const void *h, const void *a, int dtype,
+                 const int32_t *offsets, const int32_t *kept_rows, int E, int max_rows, int M, int F,
+                 const void *w1, const void *w2, void *t, void *g_w1, void *g_b1, void *g_w2,
+                 void *g_b2, void *gx, int accumulate, int gelu_bwd, mole_stream_t stream);
+
+/* Plain GEMMs on the same tiles, used by the gate: c[rows,N] = a[rows,K] . b[N,K]^T  (fp32 out). */
+int mole_gemm_nt(const void *a, const void *b, int dtype, int rows, int N, int K, float *c,
+                 mole_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Slot pool and pinned-host expert prefetch.  Replaces _UniMem (MOLE/cpp/umemory.cpp,
+ * MOLE/cpp/define.hpp:143-193), _CPUParamCore::prefetch_to (MOLE/cpp/uparameter.cpp:58-63),
+ * _MOLECore::prefetch_fwd/bwd (MOLE/cpp/core.cpp:41-75), _BatchRecord::fetch_para
+ * (MOLE/cpp/core.cpp:110-143), the H2D copies (MOLE/cpp/transfer.cu:9-12) and the stream/event
+ * plumbing (MOLE/cpp/stream.cpp:38-55, 156-205).
+ *
+ * The pool holds pool_size expert slots for each of the four parameter kinds
+ * p_id 0..3 = w1 [F,M], b1 [F], w2 [F,M], b2 [M].  host_src[p] points at expert `0` of the
+ * pinned host array of kind p ([n_d, ...] contiguous); experts [base, base+n) are copied.
+ *
+ *   prefetch(layer, base, n)      reserve n slots at the virtual offset, push (layer, n) on the
+ *                                 prefetch stack, copy on the library's copy stream, record the
+ *                                 "parameters landed" event.
+ *   fetch_top(layer)              pop the stack when its top belongs to `layer`; returns the number
+ *                                 of experts already prefetched (0 if none) in *n_out.
+ *   fetch(view_base, base, n, prefetched)
+ *                                 make experts [base, base+n) resident in slots
+ *                                 view_base+virtual_offset .. : waits for the last compute that
+ *                                 used those slots, copies the part not yet prefetched, records the
+ *                                 event.
+ *   wait_params(stream)           the compute stream waits for the last fetch/prefetch.
+ *   release(view_base, n, stream) records that compute on `stream` has finished with the slots.
+ * ------------------------------------------------------------------------------------------ */
+int mole_unimem_create(int device, int pool_size, int dtype, int64_t F, int64_t M, void **handle);
+int mole_unimem_destroy(void *handle);
+int mole_unimem_clear_virtual_mem(void *handle);
+int mole_unimem_view_pool_size(void *handle, int *out);
+int mole_unimem_virtual_offset(void *handle, int *out);
+int mole_unimem_slot_ptr(void *handle, int p_id, int slot, void **out);
+int mole_unimem_prefetch(void *handle, int layer, const void *const host_src[4], int base, int n);
+int mole_unimem_fetch_top(void *handle, int layer, int *n_out);
+int mole_unimem_fetch(void *handle, const void *const host_src[4], int view_base, int base, int n,
+                      int prefetched, void **slot_ptrs_out /* [4] */);
+int mole_unimem_wait_params(void *handle, mole_stream_t compute_stream);
+int mole_unimem_release(void *handle, int view_base, int n, mole_stream_t compute_stream);
+int mole_unimem_sync_tran(void *handle);
+int mole_unimem_tran_stream(void *handle, mole_stream_t *out);
+/* bytes moved host->device and the copy stream's busy time between the two most recent
+ * mole_unimem_sync_tran() calls, measured with events on the copy stream */
+int mole_unimem_copy_stats(void *handle, uint64_t *bytes, float *busy_ms);
+
+/* Greedy cross-layer prefetch assignment; replaces fast_assign_prefetch
+ * (MOLE/cpp/core.cpp:1302-1345).  lp_out [n]; gp_out holds up to gp_cap triples
+ * (from_layer, for_layer, count), *gp_n the number written. */
+int mole_fast_assign_prefetch(int P, const int *Fv, const int *Ev, int n, int *lp_out, int *gp_out,
+                              int gp_cap, int *gp_n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOLE_HIP_H */

@@ -1,0 +1,104 @@
+"""ctypes binding of libmole_hip.so (the C ABI declared in include/mole_hip.h).
+
+The library is the product path: if it is missing this module raises, it never falls back to
+another implementation.  torch is imported first so that the HIP runtime the process already
+holds is the one the library binds to.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import POINTER, c_char_p, c_float, c_int, c_int32, c_int64, c_size_t, c_uint64, c_void_p
+
+import torch  # noqa: F401  (must precede the dlopen below)
+
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpp", "libmole_hip.so")
+
+MOLE_F32, MOLE_BF16 = 0, 1
+LAYOUT_PADDED, LAYOUT_RAGGED = 0, 1
+GELU_BWD_TANH, GELU_BWD_EXACT = 0, 1
+MAX_TOPK, MAX_EXPERTS = 16, 1024
+
+_P = c_void_p
+_SIGNATURES = {
+    "mole_version": (c_int, []),
+    "mole_last_error_string": (c_char_p, []),
+    "mole_softmax_fwd": (c_int, [_P, _P, c_int, c_int, _P, _P]),
+    "mole_gate_bwd": (c_int, [_P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P, _P]),
+    "mole_route_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "mole_route": (c_int, [_P, c_int, c_int, c_int, c_float, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P,
+                           _P, _P, c_size_t, _P]),
+    "mole_dispatch_fwd": (c_int, [_P, c_int, _P, c_int, c_int, c_int, _P, _P]),
+    "mole_dispatch_bwd": (c_int, [_P, c_int, _P, c_int, c_int, c_int, _P, _P, c_int, _P, _P]),
+    "mole_combine_fwd": (c_int, [_P, c_int, _P, _P, c_int, c_int, c_int, _P, _P]),
+    "mole_combine_bwd": (c_int, [_P, _P, c_int, _P, _P, c_int, c_int, c_int, _P, _P, _P]),
+    "mole_zero_pad_rows": (c_int, [_P, c_int, _P, _P, c_int, c_int, _P]),
+    "mole_ffn_fwd": (c_int, [_P, c_int, _P, _P, c_int, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P]),
+    "mole_ffn_bwd": (c_int, [_P, _P, _P, _P, c_int, _P, _P, c_int, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P,
+                             _P, c_int, c_int, _P]),
+    "mole_gemm_nt": (c_int, [_P, _P, c_int, c_int, c_int, c_int, _P, _P]),
+    "mole_unimem_create": (c_int, [c_int, c_int, c_int, c_int64, c_int64, POINTER(_P)]),
+    "mole_unimem_destroy": (c_int, [_P]),
+    "mole_unimem_clear_virtual_mem": (c_int, [_P]),
+    "mole_unimem_view_pool_size": (c_int, [_P, POINTER(c_int)]),
+    "mole_unimem_virtual_offset": (c_int, [_P, POINTER(c_int)]),
+    "mole_unimem_slot_ptr": (c_int, [_P, c_int, c_int, POINTER(_P)]),
+    "mole_unimem_prefetch": (c_int, [_P, c_int, POINTER(_P), c_int, c_int]),
+    "mole_unimem_fetch_top": (c_int, [_P, c_int, POINTER(c_int)]),
+    "mole_unimem_fetch": (c_int, [_P, POINTER(_P), c_int, c_int, c_int, c_int, POINTER(_P)]),
+    "mole_unimem_wait_params": (c_int, [_P, _P]),
+    "mole_unimem_release": (c_int, [_P, c_int, c_int, _P]),
+    "mole_unimem_sync_tran": (c_int, [_P]),
+    "mole_unimem_tran_stream": (c_int, [_P, POINTER(_P)]),
+    "mole_unimem_copy_stats": (c_int, [_P, POINTER(c_uint64), POINTER(c_float)]),
+    "mole_fast_assign_prefetch": (c_int, [c_int, POINTER(c_int), POINTER(c_int), c_int, POINTER(c_int),
+                                          POINTER(c_int), c_int, POINTER(c_int)]),
+}
+EXPORTS = tuple(_SIGNATURES)
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: the HIP extension is the only implementation of the MoE hot path. "
+                "Build it with `python -m mole_amd.build` (needs hipcc, no GPU).")
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(handle, name)  # AttributeError if the library does not export it
+            fn.restype, fn.argtypes = res, args
+        _lib = handle
+    return _lib
+
+
+def last_error() -> str:
+    return lib().mole_last_error_string().decode()
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        raise RuntimeError(f"{what} failed (code {rc}): {last_error()}")
+
+
+def ptr(t):
+    """Raw device/host pointer of a tensor; integers (addresses from the slot pool) pass through."""
+    if t is None:
+        return None
+    if isinstance(t, int):
+        return c_void_p(t)
+    return c_void_p(t.data_ptr())
+
+
+def stream():
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def dtype_code(dt: torch.dtype) -> int:
+    if dt == torch.float32:
+        return MOLE_F32
+    if dt == torch.bfloat16:
+        return MOLE_BF16
+    raise TypeError(f"mole_amd supports float32 and bfloat16, got {dt}")

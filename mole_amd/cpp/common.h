@@ -1,0 +1,63 @@
+// Shared helpers of the gfx950 kernels: error plumbing, bf16 <-> fp32, wave-level primitives.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "mole_hip.h"
+
+namespace mole {
+
+void set_error(const char *fmt, ...);
+
+#define MOLE_REQUIRE(cond, ...)                 \
+    do {                                        \
+        if (!(cond)) {                          \
+            mole::set_error(__VA_ARGS__);       \
+            return MOLE_E_INVALID;              \
+        }                                       \
+    } while (0)
+
+#define MOLE_HIP(call)                                                                   \
+    do {                                                                                 \
+        hipError_t e_ = (call);                                                          \
+        if (e_ != hipSuccess) {                                                          \
+            mole::set_error("%s failed: %s (%s:%d)", #call, hipGetErrorString(e_), __FILE__, __LINE__); \
+            return (int)e_;                                                              \
+        }                                                                                \
+    } while (0)
+
+// after a kernel launch: report launch-configuration errors without synchronising
+#define MOLE_LAUNCH_CHECK()                                                              \
+    do {                                                                                 \
+        hipError_t e_ = hipGetLastError();                                               \
+        if (e_ != hipSuccess) {                                                          \
+            mole::set_error("kernel launch failed: %s (%s:%d)", hipGetErrorString(e_), __FILE__, __LINE__); \
+            return (int)e_;                                                              \
+        }                                                                                \
+    } while (0)
+
+typedef __bf16 bf16_t;
+
+__device__ __forceinline__ float to_f32(float v) { return v; }
+__device__ __forceinline__ float to_f32(bf16_t v) { return (float)v; }
+template <typename T> __device__ __forceinline__ T from_f32(float v);
+template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) { return (bf16_t)v; }  // round to nearest even
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t lo16) { return __uint_as_float(lo16 << 16); }
+
+constexpr int WAVE = 64;
+
+__device__ __forceinline__ int lane_id() { return threadIdx.x & (WAVE - 1); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int m = WAVE / 2; m >= 1; m >>= 1) v += __shfl_xor(v, m, WAVE);
+    return v;
+}
+
+static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+}  // namespace mole

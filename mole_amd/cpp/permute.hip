@@ -1,0 +1,307 @@
+// Dispatch scatter, combine gather and their backward: HBM-bound row permutes.
+//
+// Replaces tutel's fast_encode / fast_decode (GatingEncoder / GatingDecoder forward and backward;
+// call sites MOLE/moe/layer.py:448-449 and 457-458).  One wave owns one token: it reads the
+// token's k destination rows once (wave-uniform), then streams the row in 16-byte pieces per lane,
+// so every global access is a full 1 KiB wave transaction.  The source row is read once and
+// written k times (dispatch), or k rows are read and one written (combine); all sums are fp32.
+#include "common.h"
+
+namespace mole {
+
+template <typename T> struct Vec;  // 16 bytes of T
+template <> struct Vec<float> {
+    static constexpr int N = 4;
+    float4 raw;
+    __device__ __forceinline__ void load(const float *p) { raw = *reinterpret_cast<const float4 *>(p); }
+    __device__ __forceinline__ void store(float *p) const { *reinterpret_cast<float4 *>(p) = raw; }
+    __device__ __forceinline__ void unpack(float *f) const { f[0] = raw.x; f[1] = raw.y; f[2] = raw.z; f[3] = raw.w; }
+    __device__ __forceinline__ void pack(const float *f) { raw = make_float4(f[0], f[1], f[2], f[3]); }
+    __device__ __forceinline__ void zero() { raw = make_float4(0.f, 0.f, 0.f, 0.f); }
+};
+template <> struct Vec<bf16_t> {
+    static constexpr int N = 8;
+    uint4 raw;
+    __device__ __forceinline__ void load(const bf16_t *p) { raw = *reinterpret_cast<const uint4 *>(p); }
+    __device__ __forceinline__ void store(bf16_t *p) const { *reinterpret_cast<uint4 *>(p) = raw; }
+    __device__ __forceinline__ void unpack(float *f) const {
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f[2 * i] = __uint_as_float(w[i] << 16);
+            f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+        }
+    }
+    __device__ __forceinline__ void pack(const float *f) {
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const bf16_t lo = (bf16_t)f[2 * i], hi = (bf16_t)f[2 * i + 1];
+            w[i] = (uint32_t)__builtin_bit_cast(uint16_t, lo) | ((uint32_t)__builtin_bit_cast(uint16_t, hi) << 16);
+        }
+        raw = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+    __device__ __forceinline__ void zero() { raw = make_uint4(0, 0, 0, 0); }
+};
+
+constexpr int PM_THREADS = 256;  // 4 waves = 4 tokens per block
+
+template <typename T>
+__global__ __launch_bounds__(PM_THREADS) void dispatch_fwd_kernel(const T *__restrict__ x,
+                                                                  const int32_t *__restrict__ row, int S, int M,
+                                                                  int k, T *__restrict__ xd) {
+    const int i = blockIdx.x * (PM_THREADS / WAVE) + (threadIdx.x >> 6);
+    if (i >= S) return;
+    const int lane = lane_id();
+    int r[MOLE_MAX_TOPK];
+#pragma unroll
+    for (int j = 0; j < MOLE_MAX_TOPK; ++j) r[j] = j < k ? row[(size_t)j * S + i] : -1;
+    constexpr int N = Vec<T>::N;
+    const int chunks = M / N;
+    const T *src = x + (size_t)i * M;
+    for (int c = lane; c < chunks; c += WAVE) {
+        Vec<T> v;
+        v.load(src + (size_t)c * N);
+#pragma unroll
+        for (int j = 0; j < MOLE_MAX_TOPK; ++j)
+            if (r[j] >= 0) v.store(xd + (size_t)r[j] * M + (size_t)c * N);
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(PM_THREADS) void dispatch_bwd_kernel(const T *__restrict__ dxd,
+                                                                  const int32_t *__restrict__ row, int S, int M,
+                                                                  int k, const float *__restrict__ dlogits,
+                                                                  const float *__restrict__ wg, int E,
+                                                                  T *__restrict__ dx) {
+    const int i = blockIdx.x * (PM_THREADS / WAVE) + (threadIdx.x >> 6);
+    if (i >= S) return;
+    const int lane = lane_id();
+    int r[MOLE_MAX_TOPK];
+#pragma unroll
+    for (int j = 0; j < MOLE_MAX_TOPK; ++j) r[j] = j < k ? row[(size_t)j * S + i] : -1;
+    constexpr int N = Vec<T>::N;
+    const int chunks = M / N;
+    for (int c = lane; c < chunks; c += WAVE) {
+        float acc[N];
+#pragma unroll
+        for (int q = 0; q < N; ++q) acc[q] = 0.f;
+#pragma unroll
+        for (int j = 0; j < MOLE_MAX_TOPK; ++j) {
+            if (r[j] >= 0) {
+                Vec<T> v;
+                float f[N];
+                v.load(dxd + (size_t)r[j] * M + (size_t)c * N);
+                v.unpack(f);
+#pragma unroll
+                for (int q = 0; q < N; ++q) acc[q] += f[q];
+            }
+        }
+        if (dlogits != nullptr) {
+            for (int e = 0; e < E; ++e) {
+                const float dl = dlogits[(size_t)i * E + e];
+                const float *wrow = wg + (size_t)e * M + (size_t)c * N;
+#pragma unroll
+                for (int q = 0; q < N; q += 4) {
+                    const float4 wv = *reinterpret_cast<const float4 *>(wrow + q);
+                    acc[q] += dl * wv.x;
+                    acc[q + 1] += dl * wv.y;
+                    acc[q + 2] += dl * wv.z;
+                    acc[q + 3] += dl * wv.w;
+                }
+            }
+        }
+        Vec<T> o;
+        o.pack(acc);
+        o.store(dx + (size_t)i * M + (size_t)c * N);
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(PM_THREADS) void combine_fwd_kernel(const T *__restrict__ o,
+                                                                 const int32_t *__restrict__ row,
+                                                                 const float *__restrict__ gates, int S, int M,
+                                                                 int k, T *__restrict__ y) {
+    const int i = blockIdx.x * (PM_THREADS / WAVE) + (threadIdx.x >> 6);
+    if (i >= S) return;
+    const int lane = lane_id();
+    int r[MOLE_MAX_TOPK];
+    float g[MOLE_MAX_TOPK];
+#pragma unroll
+    for (int j = 0; j < MOLE_MAX_TOPK; ++j) {
+        r[j] = j < k ? row[(size_t)j * S + i] : -1;
+        g[j] = j < k ? gates[(size_t)j * S + i] : 0.f;
+    }
+    constexpr int N = Vec<T>::N;
+    const int chunks = M / N;
+    for (int c = lane; c < chunks; c += WAVE) {
+        float acc[N];
+#pragma unroll
+        for (int q = 0; q < N; ++q) acc[q] = 0.f;
+#pragma unroll
+        for (int j = 0; j < MOLE_MAX_TOPK; ++j) {
+            if (r[j] >= 0) {
+                Vec<T> v;
+                float f[N];
+                v.load(o + (size_t)r[j] * M + (size_t)c * N);
+                v.unpack(f);
+#pragma unroll
+                for (int q = 0; q < N; ++q) acc[q] += g[j] * f[q];
+            }
+        }
+        Vec<T> out;
+        out.pack(acc);
+        out.store(y + (size_t)i * M + (size_t)c * N);
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(PM_THREADS) void combine_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ o,
+                                                                 const int32_t *__restrict__ row,
+                                                                 const float *__restrict__ gates, int S, int M,
+                                                                 int k, T *__restrict__ d_o,
+                                                                 float *__restrict__ dgates) {
+    const int i = blockIdx.x * (PM_THREADS / WAVE) + (threadIdx.x >> 6);
+    if (i >= S) return;
+    const int lane = lane_id();
+    constexpr int N = Vec<T>::N;
+    const int chunks = M / N;
+    for (int j = 0; j < k; ++j) {
+        const int r = row[(size_t)j * S + i];
+        float dot = 0.f;
+        if (r >= 0) {
+            const float g = gates[(size_t)j * S + i];
+            for (int c = lane; c < chunks; c += WAVE) {
+                Vec<T> a, b, w;
+                float fa[N], fb[N], fo[N];
+                a.load(dy + (size_t)i * M + (size_t)c * N);
+                b.load(o + (size_t)r * M + (size_t)c * N);
+                a.unpack(fa);
+                b.unpack(fb);
+#pragma unroll
+                for (int q = 0; q < N; ++q) {
+                    dot += fa[q] * fb[q];
+                    fo[q] = g * fa[q];
+                }
+                w.pack(fo);
+                w.store(d_o + (size_t)r * M + (size_t)c * N);
+            }
+            dot = wave_sum(dot);
+        }
+        if (lane == 0) dgates[(size_t)j * S + i] = dot;
+    }
+}
+
+// rows offsets[e]+kept_rows[e] .. offsets[e+1] of expert e are padding: zero them
+template <typename T>
+__global__ __launch_bounds__(PM_THREADS) void zero_pad_rows_kernel(T *__restrict__ buf,
+                                                                   const int32_t *__restrict__ kept_rows,
+                                                                   const int32_t *__restrict__ offsets, int M) {
+    const int e = blockIdx.y;
+    const int lo = offsets[e] + kept_rows[e], hi = offsets[e + 1];
+    const int lane = lane_id();
+    constexpr int N = Vec<T>::N;
+    const int chunks = M / N;
+    Vec<T> z;
+    z.zero();
+    for (int r = lo + blockIdx.x * (PM_THREADS / WAVE) + (threadIdx.x >> 6); r < hi;
+         r += gridDim.x * (PM_THREADS / WAVE))
+        for (int c = lane; c < chunks; c += WAVE) z.store(buf + (size_t)r * M + (size_t)c * N);
+}
+
+static int check_perm(const char *fn, int dtype, int S, int M, int k) {
+    MOLE_REQUIRE(dtype == MOLE_F32 || dtype == MOLE_BF16, "%s: bad dtype %d", fn, dtype);
+    MOLE_REQUIRE(S >= 0 && M > 0 && k >= 1 && k <= MOLE_MAX_TOPK, "%s: bad sizes S=%d M=%d k=%d", fn, S, M, k);
+    MOLE_REQUIRE(M % (dtype == MOLE_BF16 ? 8 : 4) == 0, "%s: M=%d must be a multiple of %d", fn, M,
+                 dtype == MOLE_BF16 ? 8 : 4);
+    return 0;
+}
+static bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+
+}  // namespace mole
+
+using namespace mole;
+
+extern "C" int mole_dispatch_fwd(const void *x, int dtype, const int32_t *row, int S, int M, int k, void *xd,
+                                 mole_stream_t stream) {
+    if (int rc = check_perm("mole_dispatch_fwd", dtype, S, M, k)) return rc;
+    if (S == 0) return 0;
+    MOLE_REQUIRE(x && row && xd && aligned16(x) && aligned16(xd), "mole_dispatch_fwd: null or misaligned pointer");
+    const dim3 grid(ceil_div(S, PM_THREADS / WAVE));
+    if (dtype == MOLE_BF16)
+        hipLaunchKernelGGL(dispatch_fwd_kernel<bf16_t>, grid, dim3(PM_THREADS), 0, (hipStream_t)stream,
+                           (const bf16_t *)x, row, S, M, k, (bf16_t *)xd);
+    else
+        hipLaunchKernelGGL(dispatch_fwd_kernel<float>, grid, dim3(PM_THREADS), 0, (hipStream_t)stream,
+                           (const float *)x, row, S, M, k, (float *)xd);
+    MOLE_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int mole_dispatch_bwd(const void *dxd, int dtype, const int32_t *row, int S, int M, int k,
+                                 const float *dlogits, const float *wg, int E, void *dx, mole_stream_t stream) {
+    if (int rc = check_perm("mole_dispatch_bwd", dtype, S, M, k)) return rc;
+    if (S == 0) return 0;
+    MOLE_REQUIRE(dxd && row && dx && aligned16(dxd) && aligned16(dx), "mole_dispatch_bwd: null or misaligned pointer");
+    MOLE_REQUIRE(dlogits == nullptr || (wg != nullptr && E >= 1 && aligned16(wg) && M % 4 == 0),
+                 "mole_dispatch_bwd: dlogits given without a valid wg/E");
+    const dim3 grid(ceil_div(S, PM_THREADS / WAVE));
+    if (dtype == MOLE_BF16)
+        hipLaunchKernelGGL(dispatch_bwd_kernel<bf16_t>, grid, dim3(PM_THREADS), 0, (hipStream_t)stream,
+                           (const bf16_t *)dxd, row, S, M, k, dlogits, wg, E, (bf16_t *)dx);
+    else
+        hipLaunchKernelGGL(dispatch_bwd_kernel<float>, grid, dim3(PM_THREADS), 0, (hipStream_t)stream,
+                           (const float *)dxd, row, S, M, k, dlogits, wg, E, (float *)dx);
+    MOLE_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int mole_combine_fwd(const void *o, int dtype, const int32_t *row, const float *gates, int S, int M,
+                                int k, void *y, mole_stream_t stream) {
+    if (int rc = check_perm("mole_combine_fwd", dtype, S, M, k)) return rc;
+    if (S == 0) return 0;
+    MOLE_REQUIRE(o && row && gates && y && aligned16(o) && aligned16(y), "mole_combine_fwd: null or misaligned pointer");
+    const dim3 grid(ceil_div(S, PM_THREADS / WAVE));
+    if (dtype == MOLE_BF16)
+        hipLaunchKernelGGL(combine_fwd_kernel<bf16_t>, grid, dim3(PM_THREADS), 0, (hipStream_t)stream,
+                           (const bf16_t *)o, row, gates, S, M, k, (bf16_t *)y);
+    else
+        hipLaunchKernelGGL(combine_fwd_kernel<float>, grid, dim3(PM_THREADS), 0, (hipStream_t)stream,
+                           (const float *)o, row, gates, S, M, k, (float *)y);
+    MOLE_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int mole_combine_bwd(const void *dy, const void *o, int dtype, const int32_t *row, const float *gates,
+                                int S, int M, int k, void *d_o, float *dgates, mole_stream_t stream) {
+    if (int rc = check_perm("mole_combine_bwd", dtype, S, M, k)) return rc;
+    if (S == 0) return 0;
+    MOLE_REQUIRE(dy && o && row && gates && d_o && dgates && aligned16(dy) && aligned16(o) && aligned16(d_o),
+                 "mole_combine_bwd: null or misaligned pointer");
+    const dim3 grid(ceil_div(S, PM_THREADS / WAVE));
+    if (dtype == MOLE_BF16)
+        hipLaunchKernelGGL(combine_bwd_kernel<bf16_t>, grid, dim3(PM_THREADS), 0, (hipStream_t)stream,
+                           (const bf16_t *)dy, (const bf16_t *)o, row, gates, S, M, k, (bf16_t *)d_o, dgates);
+    else
+        hipLaunchKernelGGL(combine_bwd_kernel<float>, grid, dim3(PM_THREADS), 0, (hipStream_t)stream,
+                           (const float *)dy, (const float *)o, row, gates, S, M, k, (float *)d_o, dgates);
+    MOLE_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int mole_zero_pad_rows(void *buf, int dtype, const int32_t *kept_rows, const int32_t *offsets, int E,
+                                  int M, mole_stream_t stream) {
+    MOLE_REQUIRE(dtype == MOLE_F32 || dtype == MOLE_BF16, "mole_zero_pad_rows: bad dtype %d", dtype);
+    MOLE_REQUIRE(E >= 1 && E <= MOLE_MAX_EXPERTS && M > 0 && M % (dtype == MOLE_BF16 ? 8 : 4) == 0,
+                 "mole_zero_pad_rows: bad sizes E=%d M=%d", E, M);
+    MOLE_REQUIRE(buf && kept_rows && offsets && aligned16(buf), "mole_zero_pad_rows: null or misaligned pointer");
+    const dim3 grid(64, E);
+    if (dtype == MOLE_BF16)
+        hipLaunchKernelGGL(zero_pad_rows_kernel<bf16_t>, grid, dim3(PM_THREADS), 0, (hipStream_t)stream,
+                           (bf16_t *)buf, kept_rows, offsets, M);
+    else
+        hipLaunchKernelGGL(zero_pad_rows_kernel<float>, grid, dim3(PM_THREADS), 0, (hipStream_t)stream,
+                           (float *)buf, kept_rows, offsets, M);
+    MOLE_LAUNCH_CHECK();
+    return 0;
+}

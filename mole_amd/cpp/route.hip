@@ -1,0 +1,485 @@
+// Routing: top-k with lowest-index ties, gate values, per-expert counts, k-major locations,
+// capacity and the dispatch permutation.  Deterministic: no atomics, every sum has a fixed order.
+//
+// Replaces tutel's extract_critical (called at MOLE/moe/layer.py:445-446) and the softmax half of
+// MOLETopk.forward (MOLE/utils/Ugate.py:13).
+//
+// Four launches, all on the caller's stream:
+//   route_topk      256 tokens per block.  A group of G lanes (G = pow2 >= E, at most 64) owns one
+//                   token and holds VPL = ceil(E/G) scores per lane; k rounds of a shuffle arg-max
+//                   with the (score desc, index asc) order.  Then, per choice j, the rank of each
+//                   token among the block's earlier tokens with the same expert: wave ballot +
+//                   popcount inside a wave, LDS wave histograms across the four waves.
+//   route_scan      one wave per (choice, expert): exclusive prefix over the blocks' histograms.
+//   route_finish    one block: per-expert totals, capacity, kept rows, row offsets, l_aux.
+//   route_finalize  loc = base(choice, expert) + block prefix + in-block rank; row = offset + loc.
+#include "common.h"
+
+#include <limits.h>
+#include <math.h>
+
+namespace mole {
+
+constexpr int RT_THREADS = 256;
+constexpr int RT_TOKENS = 256;  // tokens per block == threads per block (phase B/C map thread -> token)
+constexpr float FP32_EPS = 1.1920928955078125e-07f;
+
+// strict "a ranks above b" of torch.topk: NaN above everything, NaNs equal among themselves
+__device__ __forceinline__ bool topk_gt(float a, float b) {
+    bool an = a != a, bn = b != b;
+    if (an | bn) return an & !bn;
+    return a > b;
+}
+__device__ __forceinline__ bool topk_better(float va, int ia, float vb, int ib) {
+    return topk_gt(va, vb) || (!topk_gt(vb, va) && ia < ib);
+}
+
+template <int VPL>
+__global__ __launch_bounds__(RT_THREADS) void route_topk_kernel(
+    const float *__restrict__ scores, int S, int E, int k, int logG, int normalize,
+    int32_t *__restrict__ idx, int32_t *__restrict__ lrank, float *__restrict__ gates,
+    int32_t *__restrict__ hist /* [k][E][nb] */, float *__restrict__ colsum /* [nb][E] */, int nb) {
+    extern __shared__ char smem[];
+    int *s_idx = (int *)smem;                        // [k][256]
+    float *s_graw = (float *)(s_idx + k * RT_TOKENS);  // [k][256]
+    int *s_whist = (int *)(s_graw + k * RT_TOKENS);    // [4][E]
+    float *s_col = (float *)(s_whist + 4 * E);         // [4][E]
+
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int b = blockIdx.x, tok0 = b * RT_TOKENS;
+    const int G = 1 << logG;
+    const int tpw = 64 >> logG;  // tokens a wave handles per pass
+    const int g = lane & (G - 1), tg = lane >> logG;
+
+    // ---- phase A: top-k of every token -------------------------------------------------------
+    float colacc[VPL];
+#pragma unroll
+    for (int r = 0; r < VPL; ++r) colacc[r] = 0.f;
+
+    for (int it = 0; it < G; ++it) {
+        const int tl = w * 64 + it * tpw + tg;
+        const int token = tok0 + tl;
+        const bool tv = token < S;
+        float v[VPL];
+        uint64_t taken = 0;
+#pragma unroll
+        for (int r = 0; r < VPL; ++r) {
+            const int e = g + (r << logG);
+            const bool ok = tv && e < E;
+            v[r] = ok ? scores[(size_t)token * E + e] : -INFINITY;
+            if (ok) colacc[r] += v[r];
+            else taken |= 1ull << r;
+        }
+        for (int j = 0; j < k; ++j) {
+            float bv = -INFINITY;
+            int bi = INT_MAX;
+#pragma unroll
+            for (int r = 0; r < VPL; ++r) {
+                const int e = g + (r << logG);
+                if (!((taken >> r) & 1) && topk_better(v[r], e, bv, bi)) { bv = v[r]; bi = e; }
+            }
+            for (int m = G >> 1; m >= 1; m >>= 1) {
+                const float ov = __shfl_xor(bv, m, WAVE);
+                const int oi = __shfl_xor(bi, m, WAVE);
+                if (topk_better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
+            }
+            if (bi != INT_MAX && (bi & (G - 1)) == g) taken |= 1ull << (bi >> logG);
+            if (g == 0 && tv) {
+                s_idx[j * RT_TOKENS + tl] = bi;
+                s_graw[j * RT_TOKENS + tl] = bv;
+            }
+        }
+    }
+    // column sums of the scores (for l_aux): fold the token groups of a wave, then the 4 waves
+#pragma unroll
+    for (int r = 0; r < VPL; ++r) {
+        float c = colacc[r];
+        for (int m = G; m < WAVE; m <<= 1) c += __shfl_xor(c, m, WAVE);
+        const int e = g + (r << logG);
+        if (tg == 0 && e < E) s_col[w * E + e] = c;
+    }
+    __syncthreads();
+    for (int e = tid; e < E; e += RT_THREADS)
+        colsum[(size_t)b * E + e] = ((s_col[e] + s_col[E + e]) + s_col[2 * E + e]) + s_col[3 * E + e];
+
+    // ---- phase B: gate values and indices out --------------------------------------------------
+    const int token = tok0 + tid;
+    const bool tv = token < S;
+    if (tv) {
+        float denom = 0.f;
+        for (int j = 0; j < k; ++j) denom += s_graw[j * RT_TOKENS + tid];  // left to right, fp32
+        const float den = denom < FP32_EPS ? FP32_EPS : denom;
+        for (int j = 0; j < k; ++j) {
+            float gv = s_graw[j * RT_TOKENS + tid];
+            if (k > 1 && normalize) gv = gv / den;
+            gates[(size_t)j * S + token] = gv;
+            idx[(size_t)j * S + token] = s_idx[j * RT_TOKENS + tid];
+        }
+    }
+
+    // ---- phase C: in-block ranks per choice -----------------------------------------------------
+    const uint64_t lt_mask = (1ull << lane) - 1ull;
+    for (int j = 0; j < k; ++j) {
+        for (int e = tid; e < 4 * E; e += RT_THREADS) s_whist[e] = 0;
+        __syncthreads();
+        const int e = tv ? s_idx[j * RT_TOKENS + tid] : -1;
+        int rank = 0;
+        uint64_t remaining = __ballot(tv);
+        while (remaining) {
+            const int leader = __ffsll((unsigned long long)remaining) - 1;
+            const int e0 = __shfl(e, leader, WAVE);
+            const uint64_t m = __ballot(tv && e == e0);
+            if (tv && e == e0) rank = __popcll(m & lt_mask);
+            if (lane == leader) s_whist[w * E + e0] = __popcll(m);
+            remaining &= ~m;
+        }
+        __syncthreads();
+        if (tv) {
+            int base = 0;
+            for (int ww = 0; ww < w; ++ww) base += s_whist[ww * E + e];
+            lrank[(size_t)j * S + token] = base + rank;
+        }
+        for (int e2 = tid; e2 < E; e2 += RT_THREADS)
+            hist[((size_t)j * E + e2) * nb + b] =
+                s_whist[e2] + s_whist[E + e2] + s_whist[2 * E + e2] + s_whist[3 * E + e2];
+        __syncthreads();
+    }
+}
+
+// one wave per (choice, expert) pair: exclusive prefix over blocks, total into counts
+__global__ __launch_bounds__(256) void route_scan_kernel(int32_t *__restrict__ hist, int nb, int npairs,
+                                                         int32_t *__restrict__ counts) {
+    const int lane = threadIdx.x & 63;
+    const int pair = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (pair >= npairs) return;
+    int carry = 0;
+    for (int c0 = 0; c0 < nb; c0 += WAVE) {
+        const int bi = c0 + lane;
+        const int v = bi < nb ? hist[(size_t)pair * nb + bi] : 0;
+        int x = v;
+        for (int d = 1; d < WAVE; d <<= 1) {
+            const int y = __shfl_up(x, d, WAVE);
+            if (lane >= d) x += y;
+        }
+        if (bi < nb) hist[(size_t)pair * nb + bi] = carry + x - v;
+        carry += __shfl(x, WAVE - 1, WAVE);
+    }
+    if (lane == 0) counts[pair] = carry;
+}
+
+constexpr int FIN_THREADS = 1024;
+
+__global__ __launch_bounds__(FIN_THREADS) void route_finish_kernel(
+    const int32_t *__restrict__ counts, const float *__restrict__ colsum, int nb, int S, int E, int k,
+    int cf_sign, int cap_bound, int alignment, int layout, int32_t *__restrict__ basej,
+    int32_t *__restrict__ kept_rows, int32_t *__restrict__ offsets, int32_t *__restrict__ capacity,
+    float *__restrict__ l_aux) {
+    __shared__ int s_n[MOLE_MAX_EXPERTS];
+    __shared__ int s_red[FIN_THREADS];
+    __shared__ float s_fred[FIN_THREADS];
+    const int tid = threadIdx.x;
+    int lmax = 0;
+    for (int e = tid; e < E; e += FIN_THREADS) {
+        int tot = 0;
+        for (int j = 0; j < k; ++j) {
+            basej[j * E + e] = tot;
+            tot += counts[j * E + e];
+        }
+        s_n[e] = tot;
+        lmax = max(lmax, tot);
+    }
+    s_red[tid] = lmax;
+    __syncthreads();
+    for (int d = FIN_THREADS / 2; d >= 1; d >>= 1) {
+        if (tid < d) s_red[tid] = max(s_red[tid], s_red[tid + d]);
+        __syncthreads();
+    }
+    int cap = cf_sign > 0 ? cap_bound : s_red[0];
+    if (cf_sign < 0) cap = min(cap, cap_bound);
+    const int rem = cap % alignment;
+    if (rem > 0) cap += alignment - rem;
+    __syncthreads();
+
+    // kept rows, then their exclusive prefix (chunk per thread + Hillis-Steele over the chunks)
+    const int chunk = (E + FIN_THREADS - 1) / FIN_THREADS;
+    const int lo = min(tid * chunk, E), hi = min(lo + chunk, E);
+    int csum = 0;
+    for (int e = lo; e < hi; ++e) {
+        const int n = min(s_n[e], cap);
+        s_n[e] = n;
+        kept_rows[e] = n;
+        csum += n;
+    }
+    s_red[tid] = csum;
+    __syncthreads();
+    for (int d = 1; d < FIN_THREADS; d <<= 1) {
+        const int y = tid >= d ? s_red[tid - d] : 0;
+        __syncthreads();
+        s_red[tid] += y;
+        __syncthreads();
+    }
+    if (layout == MOLE_LAYOUT_RAGGED) {
+        int run = s_red[tid] - csum;
+        for (int e = lo; e < hi; ++e) {
+            offsets[e] = run;
+            run += s_n[e];
+        }
+        if (tid == FIN_THREADS - 1) offsets[E] = s_red[tid];
+    } else {
+        for (int e = lo; e < hi; ++e) offsets[e] = e * cap;
+        if (tid == 0) offsets[E] = E * cap;
+    }
+    if (tid == 0) capacity[0] = cap;
+
+    if (l_aux != nullptr) {
+        float acc = 0.f;
+        for (int e = tid; e < E; e += FIN_THREADS) {
+            float me = 0.f;
+            for (int b = 0; b < nb; ++b) me += colsum[(size_t)b * E + e];
+            acc += me * (float)counts[e];
+        }
+        s_fred[tid] = acc;
+        __syncthreads();
+        for (int d = FIN_THREADS / 2; d >= 1; d >>= 1) {
+            if (tid < d) s_fred[tid] += s_fred[tid + d];
+            __syncthreads();
+        }
+        if (tid == 0) l_aux[0] = S > 0 ? s_fred[0] * ((float)E / ((float)S * (float)S)) : 0.f;
+    }
+}
+
+__global__ __launch_bounds__(256) void route_finalize_kernel(
+    const int32_t *__restrict__ idx, const int32_t *__restrict__ hist, const int32_t *__restrict__ basej,
+    const int32_t *__restrict__ offsets, const int32_t *__restrict__ capacity, int S, int E, int k, int nb,
+    int32_t *__restrict__ loc /* in: in-block rank, out: location */, int32_t *__restrict__ row) {
+    const size_t p = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (p >= (size_t)k * S) return;
+    const int j = (int)(p / S), i = (int)(p % S);
+    const int e = idx[p];
+    const int b = i / RT_TOKENS;
+    const int l = basej[j * E + e] + hist[((size_t)j * E + e) * nb + b] + loc[p];
+    loc[p] = l;
+    row[p] = l < capacity[0] ? offsets[e] + l : -1;
+}
+
+static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+}  // namespace mole
+
+using namespace mole;
+
+extern "C" size_t mole_route_workspace_bytes(int S, int E, int k) {
+    if (S < 0 || E <= 0 || k <= 0) return 0;
+    const size_t nb = (size_t)ceil_div(S > 0 ? S : 1, RT_TOKENS);
+    return align256(nb * k * E * sizeof(int32_t)) + align256((size_t)k * E * sizeof(int32_t)) +
+           align256(nb * E * sizeof(float));
+}
+
+template <int VPL>
+static void launch_topk(const float *scores, int S, int E, int k, int logG, int normalize, int32_t *idx,
+                        int32_t *loc, float *gates, int32_t *hist, float *colsum, int nb, hipStream_t st) {
+    const size_t lds = (size_t)k * RT_TOKENS * 8 + (size_t)E * 4 * 8;
+    hipLaunchKernelGGL(route_topk_kernel<VPL>, dim3(nb), dim3(RT_THREADS), lds, st, scores, S, E, k, logG,
+                       normalize, idx, loc, gates, hist, colsum, nb);
+}
+
+extern "C" int mole_route(const float *scores, int S, int E, int k, float capacity_factor, int normalize_gate,
+                          int alignment, int layout, int32_t *idx, int32_t *loc, float *gates, int32_t *row,
+                          int32_t *counts, int32_t *kept_rows, int32_t *offsets, int32_t *capacity,
+                          float *l_aux, void *workspace, size_t workspace_bytes, mole_stream_t stream) {
+    MOLE_REQUIRE(S >= 0 && E >= 1 && E <= MOLE_MAX_EXPERTS, "mole_route: need S >= 0 and 1 <= E <= %d (S=%d E=%d)",
+                 MOLE_MAX_EXPERTS, S, E);
+    MOLE_REQUIRE(k >= 1 && k <= MOLE_MAX_TOPK && k <= E, "mole_route: need 1 <= k <= min(E, %d) (k=%d E=%d)",
+                 MOLE_MAX_TOPK, k, E);
+    MOLE_REQUIRE(alignment >= 1, "mole_route: alignment must be >= 1");
+    MOLE_REQUIRE(layout == MOLE_LAYOUT_PADDED || layout == MOLE_LAYOUT_RAGGED, "mole_route: bad layout %d", layout);
+    MOLE_REQUIRE(counts && kept_rows && offsets && capacity && workspace, "mole_route: null output pointer");
+    MOLE_REQUIRE(S == 0 || (scores && idx && loc && gates && row), "mole_route: null token buffer");
+    MOLE_REQUIRE((long long)S * k < INT_MAX && (long long)S * E < (1ll << 40), "mole_route: S*k too large");
+    if (workspace_bytes < mole_route_workspace_bytes(S, E, k)) {
+        set_error("mole_route: workspace of %zu bytes, need %zu", workspace_bytes, mole_route_workspace_bytes(S, E, k));
+        return MOLE_E_WORKSPACE;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    const int nb = ceil_div(S > 0 ? S : 1, RT_TOKENS);
+    char *ws = (char *)workspace;
+    int32_t *hist = (int32_t *)ws;
+    ws += align256((size_t)nb * k * E * sizeof(int32_t));
+    int32_t *basej = (int32_t *)ws;
+    ws += align256((size_t)k * E * sizeof(int32_t));
+    float *colsum = (float *)ws;
+
+    int logG = 0;
+    while ((1 << logG) < E && logG < 6) ++logG;
+    const int vpl = ceil_div(E, 1 << logG);
+    if (vpl <= 1) launch_topk<1>(scores, S, E, k, logG, normalize_gate, idx, loc, gates, hist, colsum, nb, st);
+    else if (vpl <= 2) launch_topk<2>(scores, S, E, k, logG, normalize_gate, idx, loc, gates, hist, colsum, nb, st);
+    else if (vpl <= 4) launch_topk<4>(scores, S, E, k, logG, normalize_gate, idx, loc, gates, hist, colsum, nb, st);
+    else if (vpl <= 8) launch_topk<8>(scores, S, E, k, logG, normalize_gate, idx, loc, gates, hist, colsum, nb, st);
+    else launch_topk<16>(scores, S, E, k, logG, normalize_gate, idx, loc, gates, hist, colsum, nb, st);
+    MOLE_LAUNCH_CHECK();
+
+    const int npairs = k * E;
+    hipLaunchKernelGGL(route_scan_kernel, dim3(ceil_div(npairs, 4)), dim3(256), 0, st, hist, nb, npairs, counts);
+    MOLE_LAUNCH_CHECK();
+
+    const int spe = (S + E - 1) / E;
+    const int cf_sign = capacity_factor > 0.f ? 1 : (capacity_factor < 0.f ? -1 : 0);
+    // int(cf * spe) of the Python reference: the product is taken in double precision
+    const double prod = (double)(capacity_factor < 0.f ? -capacity_factor : capacity_factor) * (double)spe;
+    const int cap_bound = k * (int)prod;
+    hipLaunchKernelGGL(route_finish_kernel, dim3(1), dim3(FIN_THREADS), 0, st, counts, colsum, nb, S, E, k, cf_sign,
+                       cap_bound, alignment, layout, basej, kept_rows, offsets, capacity, l_aux);
+    MOLE_LAUNCH_CHECK();
+
+    if (S > 0) {
+        const size_t n = (size_t)k * S;
+        hipLaunchKernelGGL(route_finalize_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, idx, hist,
+                           basej, offsets, capacity, S, E, k, nb, loc, row);
+        MOLE_LAUNCH_CHECK();
+    }
+    return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// softmax over experts (MOLE/utils/Ugate.py:13) and the backward from dgates to dlogits
+// ---------------------------------------------------------------------------------------------
+namespace mole {
+
+// One group of G lanes per token (same mapping as route_topk), VPL values per lane.
+template <int VPL>
+__global__ __launch_bounds__(256) void softmax_fwd_kernel(const float *__restrict__ logits,
+                                                          const float *__restrict__ bias, int S, int E, int logG,
+                                                          float *__restrict__ scores) {
+    const int lane = threadIdx.x & 63;
+    const int G = 1 << logG;
+    const int g = lane & (G - 1), tg = lane >> logG;
+    const int tpw = 64 >> logG;
+    const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int token = wave * tpw + tg;
+    const bool tv = token < S;
+    float v[VPL];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < VPL; ++r) {
+        const int e = g + (r << logG);
+        const bool ok = tv && e < E;
+        v[r] = ok ? logits[(size_t)token * E + e] + (bias ? bias[e] : 0.f) : -INFINITY;
+        mx = fmaxf(mx, v[r]);
+    }
+    for (int m = G >> 1; m >= 1; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m, WAVE));
+    float sum = 0.f;
+#pragma unroll
+    for (int r = 0; r < VPL; ++r) {
+        const int e = g + (r << logG);
+        v[r] = (tv && e < E) ? expf(v[r] - mx) : 0.f;
+        sum += v[r];
+    }
+    for (int m = G >> 1; m >= 1; m >>= 1) sum += __shfl_xor(sum, m, WAVE);
+#pragma unroll
+    for (int r = 0; r < VPL; ++r) {
+        const int e = g + (r << logG);
+        if (tv && e < E) scores[(size_t)token * E + e] = v[r] / sum;
+    }
+}
+
+// dlogits[i,e] = s[i,e] * (dscore[i,e] - sum_e' dscore[i,e'] s[i,e']), dscore scattered from dgates
+// through gate_j = graw_j / max(sum graw, eps).  One thread per token for the k-sized part, then the
+// group of lanes writes the row.
+template <int VPL>
+__global__ __launch_bounds__(256) void gate_bwd_kernel(const float *__restrict__ dgates,
+                                                       const float *__restrict__ scores,
+                                                       const int32_t *__restrict__ idx, int S, int E, int k,
+                                                       int logG, int normalize, int through_softmax,
+                                                       float *__restrict__ dlogits) {
+    const int lane = threadIdx.x & 63;
+    const int G = 1 << logG;
+    const int g = lane & (G - 1), tg = lane >> logG;
+    const int tpw = 64 >> logG;
+    const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int token = wave * tpw + tg;
+    const bool tv = token < S;
+    float s[VPL], ds[VPL];
+#pragma unroll
+    for (int r = 0; r < VPL; ++r) {
+        const int e = g + (r << logG);
+        s[r] = (tv && e < E) ? scores[(size_t)token * E + e] : 0.f;
+        ds[r] = 0.f;
+    }
+    if (tv) {
+        float denom = 0.f, dotg = 0.f;
+        for (int j = 0; j < k; ++j) {
+            const int e = idx[(size_t)j * S + token];
+            const float gr = scores[(size_t)token * E + e];
+            denom += gr;
+            dotg += dgates[(size_t)j * S + token] * gr;
+        }
+        const bool norm = k > 1 && normalize;
+        const bool clamped = denom < FP32_EPS;
+        const float den = clamped ? FP32_EPS : denom;
+        const float sub = (norm && !clamped) ? dotg / (den * den) : 0.f;
+        for (int j = 0; j < k; ++j) {
+            const int e = idx[(size_t)j * S + token];
+            const float dg = dgates[(size_t)j * S + token];
+            const float dgraw = norm ? dg / den - sub : dg;
+            if ((e & (G - 1)) == g) {
+                const int rr = e >> logG;
+#pragma unroll
+                for (int r = 0; r < VPL; ++r)
+                    if (r == rr) ds[r] += dgraw;
+            }
+        }
+    }
+    float dot = 0.f;
+#pragma unroll
+    for (int r = 0; r < VPL; ++r) dot += ds[r] * s[r];
+    for (int m = G >> 1; m >= 1; m >>= 1) dot += __shfl_xor(dot, m, WAVE);
+#pragma unroll
+    for (int r = 0; r < VPL; ++r) {
+        const int e = g + (r << logG);
+        if (tv && e < E) dlogits[(size_t)token * E + e] = through_softmax ? s[r] * (ds[r] - dot) : ds[r];
+    }
+}
+
+}  // namespace mole
+
+#define MOLE_VPL_DISPATCH(vpl, KERNEL, grid, st, ...)                                              \
+    do {                                                                                           \
+        if ((vpl) <= 1) hipLaunchKernelGGL(KERNEL<1>, grid, dim3(256), 0, st, __VA_ARGS__);         \
+        else if ((vpl) <= 2) hipLaunchKernelGGL(KERNEL<2>, grid, dim3(256), 0, st, __VA_ARGS__);    \
+        else if ((vpl) <= 4) hipLaunchKernelGGL(KERNEL<4>, grid, dim3(256), 0, st, __VA_ARGS__);    \
+        else if ((vpl) <= 8) hipLaunchKernelGGL(KERNEL<8>, grid, dim3(256), 0, st, __VA_ARGS__);    \
+        else hipLaunchKernelGGL(KERNEL<16>, grid, dim3(256), 0, st, __VA_ARGS__);                   \
+    } while (0)
+
+extern "C" int mole_softmax_fwd(const float *logits, const float *logit_bias, int S, int E, float *scores,
+                                mole_stream_t stream) {
+    MOLE_REQUIRE(S >= 0 && E >= 1 && E <= MOLE_MAX_EXPERTS, "mole_softmax_fwd: bad sizes S=%d E=%d", S, E);
+    if (S == 0) return 0;
+    MOLE_REQUIRE(logits && scores, "mole_softmax_fwd: null pointer");
+    int logG = 0;
+    while ((1 << logG) < E && logG < 6) ++logG;
+    const int vpl = ceil_div(E, 1 << logG);
+    const int tpw = 64 >> logG;
+    const dim3 grid(ceil_div(S, 4 * tpw));
+    MOLE_VPL_DISPATCH(vpl, softmax_fwd_kernel, grid, (hipStream_t)stream, logits, logit_bias, S, E, logG, scores);
+    MOLE_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int mole_gate_bwd(const float *dgates, const float *scores, const int32_t *idx, int S, int E, int k,
+                             int normalize_gate, int through_softmax, float *dlogits, mole_stream_t stream) {
+    MOLE_REQUIRE(S >= 0 && E >= 1 && E <= MOLE_MAX_EXPERTS && k >= 1 && k <= MOLE_MAX_TOPK && k <= E,
+                 "mole_gate_bwd: bad sizes S=%d E=%d k=%d", S, E, k);
+    if (S == 0) return 0;
+    MOLE_REQUIRE(dgates && scores && idx && dlogits, "mole_gate_bwd: null pointer");
+    int logG = 0;
+    while ((1 << logG) < E && logG < 6) ++logG;
+    const int vpl = ceil_div(E, 1 << logG);
+    const int tpw = 64 >> logG;
+    const dim3 grid(ceil_div(S, 4 * tpw));
+    MOLE_VPL_DISPATCH(vpl, gate_bwd_kernel, grid, (hipStream_t)stream, dgates, scores, idx, S, E, k, logG,
+                      normalize_gate, through_softmax, dlogits);
+    MOLE_LAUNCH_CHECK();
+    return 0;
+}

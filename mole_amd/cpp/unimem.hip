@@ -1,0 +1,276 @@
+// Slot pool for offloaded experts and the pinned-host -> HBM prefetch that feeds it.
+//
+// Replaces _UniMem (MOLE/cpp/umemory.cpp:92-183, MOLE/cpp/define.hpp:143-193),
+// _CPUParamCore::prefetch_to (MOLE/cpp/uparameter.cpp:58-63), _ParamProxy::fetch
+// (MOLE/cpp/umemory.cpp:189-205), _MOLECore::prefetch_fwd/bwd (MOLE/cpp/core.cpp:41-75),
+// _BatchRecord::fetch_para (MOLE/cpp/core.cpp:110-143), the copy wrappers
+// (MOLE/cpp/transfer.cu:9-12) and the "tran" stream with its events (MOLE/cpp/stream.cpp).
+//
+// The pool is four device arrays of pool_size slots (w1, b1, w2, b2).  Copies run on one
+// library-owned stream at default priority; ordering against the caller's compute stream is by
+// events only: a "parameters landed" event the compute stream waits on, and one "slot released"
+// event per slot that the copy stream waits on before overwriting the slot.
+#include "common.h"
+
+#include <array>
+#include <vector>
+
+namespace mole {
+
+struct UniMem {
+    int device = 0, pool_size = 0, dtype = 0;
+    size_t slot_bytes[4] = {0, 0, 0, 0};
+    char *pool[4] = {nullptr, nullptr, nullptr, nullptr};
+    hipStream_t tran = nullptr;
+    hipEvent_t para_event = nullptr;
+    bool para_recorded = false;
+    std::vector<hipEvent_t> slot_event;
+    std::vector<char> slot_pending;  // slot_event[s] was recorded and not yet waited on
+    std::vector<std::array<int, 2>> stk;  // (layer, n)
+    int virtual_offset = 0, view_pool_size = 0;
+    // copy statistics
+    std::vector<std::array<hipEvent_t, 2>> timers;
+    size_t timers_used = 0;
+    uint64_t bytes_open = 0, bytes_last = 0;
+    float ms_last = 0.f;
+};
+
+static int copy_experts(UniMem *u, const void *const host_src[4], int slot0, int base, int n) {
+    if (n <= 0) return 0;
+    for (int s = slot0; s < slot0 + n; ++s)
+        if (u->slot_pending[s]) {
+            MOLE_HIP(hipStreamWaitEvent(u->tran, u->slot_event[s], 0));
+            u->slot_pending[s] = 0;
+        }
+    if (u->timers_used == u->timers.size()) {
+        std::array<hipEvent_t, 2> p;
+        MOLE_HIP(hipEventCreate(&p[0]));
+        MOLE_HIP(hipEventCreate(&p[1]));
+        u->timers.push_back(p);
+    }
+    auto &tm = u->timers[u->timers_used++];
+    MOLE_HIP(hipEventRecord(tm[0], u->tran));
+    for (int p = 0; p < 4; ++p) {
+        const size_t sb = u->slot_bytes[p];
+        MOLE_HIP(hipMemcpyAsync(u->pool[p] + (size_t)slot0 * sb, (const char *)host_src[p] + (size_t)base * sb,
+                                (size_t)n * sb, hipMemcpyHostToDevice, u->tran));
+        u->bytes_open += (uint64_t)n * sb;
+    }
+    MOLE_HIP(hipEventRecord(tm[1], u->tran));
+    MOLE_HIP(hipEventRecord(u->para_event, u->tran));
+    u->para_recorded = true;
+    return 0;
+}
+
+}  // namespace mole
+
+using namespace mole;
+
+#define UM(handle)                                                        \
+    UniMem *u = (UniMem *)(handle);                                        \
+    MOLE_REQUIRE(u != nullptr, "%s: null handle", __func__)
+
+extern "C" int mole_unimem_create(int device, int pool_size, int dtype, int64_t F, int64_t M, void **handle) {
+    MOLE_REQUIRE(handle != nullptr, "mole_unimem_create: null handle pointer");
+    MOLE_REQUIRE(pool_size >= 0 && F > 0 && M > 0, "mole_unimem_create: bad sizes pool=%d F=%lld M=%lld", pool_size,
+                 (long long)F, (long long)M);
+    MOLE_REQUIRE(dtype == MOLE_F32 || dtype == MOLE_BF16, "mole_unimem_create: bad dtype %d", dtype);
+    MOLE_HIP(hipSetDevice(device));
+    UniMem *u = new UniMem();
+    u->device = device;
+    u->pool_size = pool_size;
+    u->dtype = dtype;
+    const size_t es = dtype == MOLE_BF16 ? 2 : 4;
+    u->slot_bytes[0] = (size_t)F * M * es;
+    u->slot_bytes[1] = (size_t)F * es;
+    u->slot_bytes[2] = (size_t)F * M * es;
+    u->slot_bytes[3] = (size_t)M * es;
+    u->view_pool_size = pool_size;
+    for (int p = 0; p < 4 && pool_size > 0; ++p) {
+        hipError_t e = hipMalloc((void **)&u->pool[p], u->slot_bytes[p] * pool_size);
+        if (e != hipSuccess) {
+            set_error("mole_unimem_create: hipMalloc of %zu bytes failed: %s", u->slot_bytes[p] * pool_size,
+                      hipGetErrorString(e));
+            for (int q = 0; q < p; ++q) (void)hipFree(u->pool[q]);
+            delete u;
+            return MOLE_E_NOMEM;
+        }
+    }
+    MOLE_HIP(hipStreamCreateWithFlags(&u->tran, hipStreamNonBlocking));
+    MOLE_HIP(hipEventCreateWithFlags(&u->para_event, hipEventDisableTiming));
+    u->slot_event.resize(pool_size);
+    u->slot_pending.assign(pool_size, 0);
+    for (int s = 0; s < pool_size; ++s) MOLE_HIP(hipEventCreateWithFlags(&u->slot_event[s], hipEventDisableTiming));
+    *handle = u;
+    return 0;
+}
+
+extern "C" int mole_unimem_destroy(void *handle) {
+    UM(handle);
+    (void)hipSetDevice(u->device);
+    (void)hipStreamSynchronize(u->tran);
+    for (auto &e : u->slot_event) (void)hipEventDestroy(e);
+    for (auto &t : u->timers) { (void)hipEventDestroy(t[0]); (void)hipEventDestroy(t[1]); }
+    (void)hipEventDestroy(u->para_event);
+    (void)hipStreamDestroy(u->tran);
+    for (int p = 0; p < 4; ++p)
+        if (u->pool[p]) (void)hipFree(u->pool[p]);
+    delete u;
+    return 0;
+}
+
+extern "C" int mole_unimem_clear_virtual_mem(void *handle) {
+    UM(handle);
+    u->stk.clear();
+    u->virtual_offset = 0;
+    u->view_pool_size = u->pool_size;
+    return 0;
+}
+
+extern "C" int mole_unimem_view_pool_size(void *handle, int *out) {
+    UM(handle);
+    *out = u->view_pool_size;
+    return 0;
+}
+
+extern "C" int mole_unimem_virtual_offset(void *handle, int *out) {
+    UM(handle);
+    *out = u->virtual_offset;
+    return 0;
+}
+
+extern "C" int mole_unimem_slot_ptr(void *handle, int p_id, int slot, void **out) {
+    UM(handle);
+    MOLE_REQUIRE(p_id >= 0 && p_id < 4 && slot >= 0 && slot < u->pool_size && out, "mole_unimem_slot_ptr: bad p_id %d / slot %d", p_id, slot);
+    *out = u->pool[p_id] + (size_t)slot * u->slot_bytes[p_id];
+    return 0;
+}
+
+extern "C" int mole_unimem_prefetch(void *handle, int layer, const void *const host_src[4], int base, int n) {
+    UM(handle);
+    if (n == 0) return 0;
+    MOLE_REQUIRE(n > 0 && base >= 0 && host_src && host_src[0] && host_src[1] && host_src[2] && host_src[3],
+                 "mole_unimem_prefetch: bad arguments (base=%d n=%d)", base, n);
+    if (n > u->view_pool_size) {
+        set_error("mole_unimem_prefetch: %d experts do not fit the %d free pool slots", n, u->view_pool_size);
+        return MOLE_E_STATE;
+    }
+    if (int rc = copy_experts(u, host_src, u->virtual_offset, base, n)) return rc;
+    if (!u->stk.empty() && u->stk.back()[0] == layer) u->stk.back()[1] += n;
+    else u->stk.push_back({layer, n});
+    u->virtual_offset += n;
+    u->view_pool_size -= n;
+    return 0;
+}
+
+extern "C" int mole_unimem_fetch_top(void *handle, int layer, int *n_out) {
+    UM(handle);
+    MOLE_REQUIRE(n_out != nullptr, "mole_unimem_fetch_top: null output");
+    *n_out = 0;
+    if (!u->stk.empty() && u->stk.back()[0] == layer) {
+        const int n = u->stk.back()[1];
+        u->stk.pop_back();
+        u->virtual_offset -= n;
+        u->view_pool_size += n;
+        *n_out = n;
+    }
+    return 0;
+}
+
+extern "C" int mole_unimem_fetch(void *handle, const void *const host_src[4], int view_base, int base, int n,
+                                 int prefetched, void **slot_ptrs_out) {
+    UM(handle);
+    const int slot0 = view_base + u->virtual_offset;
+    MOLE_REQUIRE(n > 0 && view_base >= 0 && base >= 0 && prefetched >= 0 && prefetched <= n && host_src && slot_ptrs_out,
+                 "mole_unimem_fetch: bad arguments (view_base=%d base=%d n=%d prefetched=%d)", view_base, base, n, prefetched);
+    if (slot0 + n > u->pool_size) {
+        set_error("mole_unimem_fetch: slots %d..%d exceed the pool of %d", slot0, slot0 + n, u->pool_size);
+        return MOLE_E_STATE;
+    }
+    if (int rc = copy_experts(u, host_src, slot0 + prefetched, base + prefetched, n - prefetched)) return rc;
+    for (int p = 0; p < 4; ++p) slot_ptrs_out[p] = u->pool[p] + (size_t)slot0 * u->slot_bytes[p];
+    return 0;
+}
+
+extern "C" int mole_unimem_wait_params(void *handle, mole_stream_t compute_stream) {
+    UM(handle);
+    if (u->para_recorded) MOLE_HIP(hipStreamWaitEvent((hipStream_t)compute_stream, u->para_event, 0));
+    return 0;
+}
+
+extern "C" int mole_unimem_release(void *handle, int view_base, int n, mole_stream_t compute_stream) {
+    UM(handle);
+    const int slot0 = view_base + u->virtual_offset;
+    MOLE_REQUIRE(n >= 0 && slot0 >= 0 && slot0 + n <= u->pool_size, "mole_unimem_release: slots %d..%d outside the pool", slot0, slot0 + n);
+    for (int s = slot0; s < slot0 + n; ++s) {
+        MOLE_HIP(hipEventRecord(u->slot_event[s], (hipStream_t)compute_stream));
+        u->slot_pending[s] = 1;
+    }
+    return 0;
+}
+
+extern "C" int mole_unimem_sync_tran(void *handle) {
+    UM(handle);
+    MOLE_HIP(hipStreamSynchronize(u->tran));
+    float total = 0.f;
+    for (size_t i = 0; i < u->timers_used; ++i) {
+        float ms = 0.f;
+        MOLE_HIP(hipEventElapsedTime(&ms, u->timers[i][0], u->timers[i][1]));
+        total += ms;
+    }
+    u->ms_last = total;
+    u->bytes_last = u->bytes_open;
+    u->bytes_open = 0;
+    u->timers_used = 0;
+    return 0;
+}
+
+extern "C" int mole_unimem_tran_stream(void *handle, mole_stream_t *out) {
+    UM(handle);
+    *out = (mole_stream_t)u->tran;
+    return 0;
+}
+
+extern "C" int mole_unimem_copy_stats(void *handle, uint64_t *bytes, float *busy_ms) {
+    UM(handle);
+    if (bytes) *bytes = u->bytes_last;
+    if (busy_ms) *busy_ms = u->ms_last;
+    return 0;
+}
+
+extern "C" int mole_fast_assign_prefetch(int P, const int *Fv, const int *Ev, int n, int *lp_out, int *gp_out,
+                                         int gp_cap, int *gp_n) {
+    MOLE_REQUIRE(n >= 0 && Fv && Ev && lp_out && gp_out && gp_n, "mole_fast_assign_prefetch: null pointer");
+    // Layers with spare fetch time lend it to later layers that cannot hide their own fetches.
+    // `lenders` is a stack of (layer, spare experts it may still fetch for others); `pool_free`
+    // is the number of pool slots not yet promised.
+    std::vector<std::array<int, 2>> lenders;
+    int pool_free = P, written = 0;
+    auto emit = [&](int from, int to, int cnt) -> bool {
+        if (written >= gp_cap) return false;
+        gp_out[3 * written] = from; gp_out[3 * written + 1] = to; gp_out[3 * written + 2] = cnt;
+        ++written;
+        return true;
+    };
+    for (int i = 0; i < n; ++i) {
+        const int can = pool_free < Fv[i] ? pool_free : Fv[i];
+        if (can > Ev[i]) {                 // spare capacity: lend it
+            lp_out[i] = Ev[i];
+            lenders.push_back({i, can - Ev[i]});
+            pool_free -= can - Ev[i];
+            continue;
+        }
+        lp_out[i] = can;
+        int need = Ev[i] - can;
+        while (need > 0 && !lenders.empty()) {
+            auto &top = lenders.back();
+            const int take = top[1] > need ? need : top[1];
+            if (!emit(top[0], i, take)) { set_error("mole_fast_assign_prefetch: gp_out too small"); return MOLE_E_WORKSPACE; }
+            pool_free += take;
+            need -= take;
+            if (top[1] > take) top[1] -= take; else lenders.pop_back();
+        }
+    }
+    *gp_n = written;
+    return 0;
+}

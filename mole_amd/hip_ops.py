@@ -1,0 +1,185 @@
+"""Tensor-level wrappers of the C ABI: allocate outputs with torch, pass raw pointers, run on
+torch's current HIP stream.  No math happens here."""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+from . import _lib as L
+
+
+def _dev(t: torch.Tensor) -> torch.Tensor:
+    if not t.is_cuda:
+        raise RuntimeError("mole_amd: tensors must live on the GPU (there is no CPU path)")
+    if not t.is_contiguous():
+        raise RuntimeError("mole_amd: tensors must be contiguous")
+    return t
+
+
+def gemm_nt(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """c[rows,N] = a[rows,K] @ b[N,K].T in fp32 (gate logits)."""
+    _dev(a), _dev(b)
+    rows, K = a.shape
+    N = b.shape[0]
+    c = torch.empty(rows, N, dtype=torch.float32, device=a.device)
+    L.check(L.lib().mole_gemm_nt(L.ptr(a), L.ptr(b), L.dtype_code(a.dtype), rows, N, K, L.ptr(c), L.stream()), "mole_gemm_nt")
+    return c
+
+
+def softmax_fwd(logits: torch.Tensor, logit_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _dev(logits)
+    S, E = logits.shape
+    scores = torch.empty_like(logits)
+    L.check(L.lib().mole_softmax_fwd(L.ptr(logits), L.ptr(logit_bias), S, E, L.ptr(scores), L.stream()), "mole_softmax_fwd")
+    return scores
+
+
+def gate_bwd(dgates: torch.Tensor, scores: torch.Tensor, idx: torch.Tensor, normalize_gate: bool,
+             through_softmax: bool = True) -> torch.Tensor:
+    """d(logits) (through_softmax) or d(scores) from d(gates)."""
+    _dev(dgates), _dev(scores), _dev(idx)
+    S, E = scores.shape
+    k = idx.shape[0]
+    dlogits = torch.empty_like(scores)
+    L.check(L.lib().mole_gate_bwd(L.ptr(dgates), L.ptr(scores), L.ptr(idx), S, E, k, int(normalize_gate), int(through_softmax), L.ptr(dlogits),
+                                  L.stream()), "mole_gate_bwd")
+    return dlogits
+
+
+@dataclass
+class Route:
+    """Device-side result of mole_route (what tutel's extract_critical returns, plus the ragged
+    bookkeeping).  Nothing here forces a host synchronisation."""
+    S: int
+    E: int
+    k: int
+    layout: int
+    idx: torch.Tensor        # [k,S] int32
+    loc: torch.Tensor        # [k,S] int32
+    gates: torch.Tensor      # [k,S] fp32
+    row: torch.Tensor        # [k,S] int32
+    counts: torch.Tensor     # [k,E] int32
+    kept_rows: torch.Tensor  # [E] int32
+    offsets: torch.Tensor    # [E+1] int32
+    capacity: torch.Tensor   # [1] int32
+    l_aux: torch.Tensor      # [1] fp32
+    normalize_gate: bool = True
+
+
+def route(scores: torch.Tensor, top_k: int, capacity_factor: float = 1.0, normalize_gate: bool = True,
+          alignment: int = 1, layout: int = L.LAYOUT_RAGGED) -> Route:
+    _dev(scores)
+    if scores.dtype != torch.float32:
+        raise TypeError("mole_route takes fp32 scores")
+    S, E = scores.shape
+    k = min(int(top_k), E)
+    dev = scores.device
+    i32 = dict(dtype=torch.int32, device=dev)
+    idx, loc, row = (torch.empty(k, S, **i32) for _ in range(3))
+    gates = torch.empty(k, S, dtype=torch.float32, device=dev)
+    meta = torch.empty(k * E + E + (E + 1) + 1, **i32)
+    counts = meta[:k * E].view(k, E)
+    kept = meta[k * E:k * E + E]
+    offsets = meta[k * E + E:k * E + 2 * E + 1]
+    cap = meta[k * E + 2 * E + 1:]
+    l_aux = torch.empty(1, dtype=torch.float32, device=dev)
+    nbytes = L.lib().mole_route_workspace_bytes(S, E, k)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    L.check(L.lib().mole_route(L.ptr(scores), S, E, k, float(capacity_factor), int(normalize_gate), int(alignment),
+                               int(layout), L.ptr(idx), L.ptr(loc), L.ptr(gates), L.ptr(row), L.ptr(counts),
+                               L.ptr(kept), L.ptr(offsets), L.ptr(cap), L.ptr(l_aux), L.ptr(ws), nbytes, L.stream()),
+            "mole_route")
+    return Route(S, E, k, layout, idx, loc, gates, row, counts, kept, offsets, cap, l_aux, normalize_gate)
+
+
+def dispatch_fwd(x: torch.Tensor, row: torch.Tensor, total_rows: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _dev(x), _dev(row)
+    S, M = x.shape
+    k = row.shape[0]
+    xd = out if out is not None else torch.empty(total_rows, M, dtype=x.dtype, device=x.device)
+    L.check(L.lib().mole_dispatch_fwd(L.ptr(x), L.dtype_code(x.dtype), L.ptr(row), S, M, k, L.ptr(xd), L.stream()),
+            "mole_dispatch_fwd")
+    return xd
+
+
+def dispatch_bwd(dxd: torch.Tensor, row: torch.Tensor, dlogits: Optional[torch.Tensor] = None,
+                 wg: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _dev(dxd), _dev(row)
+    k, S = row.shape
+    M = dxd.shape[-1]
+    dx = torch.empty(S, M, dtype=dxd.dtype, device=dxd.device)
+    E = 0
+    if dlogits is not None:
+        _dev(dlogits), _dev(wg)
+        E = wg.shape[0]
+        if wg.dtype != torch.float32 or dlogits.dtype != torch.float32:
+            raise TypeError("gate tensors are fp32")
+    L.check(L.lib().mole_dispatch_bwd(L.ptr(dxd), L.dtype_code(dxd.dtype), L.ptr(row), S, M, k, L.ptr(dlogits), L.ptr(wg),
+                                      E, L.ptr(dx), L.stream()), "mole_dispatch_bwd")
+    return dx
+
+
+def combine_fwd(o: torch.Tensor, row: torch.Tensor, gates: torch.Tensor) -> torch.Tensor:
+    _dev(o), _dev(row), _dev(gates)
+    k, S = row.shape
+    M = o.shape[-1]
+    y = torch.empty(S, M, dtype=o.dtype, device=o.device)
+    L.check(L.lib().mole_combine_fwd(L.ptr(o), L.dtype_code(o.dtype), L.ptr(row), L.ptr(gates), S, M, k, L.ptr(y), L.stream()),
+            "mole_combine_fwd")
+    return y
+
+
+def combine_bwd(dy: torch.Tensor, o: torch.Tensor, row: torch.Tensor, gates: torch.Tensor,
+                d_o: Optional[torch.Tensor] = None):
+    _dev(dy), _dev(o), _dev(row), _dev(gates)
+    k, S = row.shape
+    M = o.shape[-1]
+    if d_o is None:
+        d_o = torch.empty_like(o)
+    dgates = torch.empty(k, S, dtype=torch.float32, device=o.device)
+    L.check(L.lib().mole_combine_bwd(L.ptr(dy), L.ptr(o), L.dtype_code(o.dtype), L.ptr(row), L.ptr(gates), S, M, k,
+                                     L.ptr(d_o), L.ptr(dgates), L.stream()), "mole_combine_bwd")
+    return d_o, dgates
+
+
+def zero_pad_rows(buf: torch.Tensor, kept_rows: torch.Tensor, offsets: torch.Tensor) -> None:
+    _dev(buf)
+    E = kept_rows.shape[0]
+    M = buf.shape[-1]
+    L.check(L.lib().mole_zero_pad_rows(L.ptr(buf), L.dtype_code(buf.dtype), L.ptr(kept_rows), L.ptr(offsets), E, M, L.stream()),
+            "mole_zero_pad_rows")
+
+
+def ffn_fwd(xd, offsets, kept_rows, w1, b1, w2, b2, max_rows: Optional[int] = None):
+    """Returns (out [rows,M], h [rows,F], a [rows,F])."""
+    for t in (xd, offsets, kept_rows, w1, b1, w2, b2):
+        _dev(t)
+    rows, M = xd.shape
+    E, F, _ = w1.shape
+    max_rows = rows if max_rows is None else max_rows
+    h = torch.empty(rows, F, dtype=xd.dtype, device=xd.device)
+    a = torch.empty(rows, F, dtype=xd.dtype, device=xd.device)
+    out = torch.empty(rows, M, dtype=xd.dtype, device=xd.device)
+    L.check(L.lib().mole_ffn_fwd(L.ptr(xd), L.dtype_code(xd.dtype), L.ptr(offsets), L.ptr(kept_rows), E, max_rows, M, F,
+                                 L.ptr(w1), L.ptr(b1), L.ptr(w2), L.ptr(b2), L.ptr(h), L.ptr(a), L.ptr(out), L.stream()),
+            "mole_ffn_fwd")
+    return out, h, a
+
+
+def ffn_bwd(go, xd, h, a, offsets, kept_rows, w1, w2, g_w1, g_b1, g_w2, g_b2, need_gx: bool = True,
+            accumulate: bool = False, gelu_bwd: int = L.GELU_BWD_TANH, max_rows: Optional[int] = None):
+    """Writes (or accumulates into) g_w1, g_b1, g_w2, g_b2; returns gx [rows,M] or None."""
+    for t in (go, xd, h, a, offsets, kept_rows, w1, w2, g_w1, g_b1, g_w2, g_b2):
+        _dev(t)
+    rows, M = xd.shape
+    E, F, _ = w1.shape
+    max_rows = rows if max_rows is None else max_rows
+    t = torch.empty(rows, F, dtype=xd.dtype, device=xd.device)
+    gx = torch.empty(rows, M, dtype=xd.dtype, device=xd.device) if need_gx else None
+    L.check(L.lib().mole_ffn_bwd(L.ptr(go), L.ptr(xd), L.ptr(h), L.ptr(a), L.dtype_code(xd.dtype), L.ptr(offsets),
+                                 L.ptr(kept_rows), E, max_rows, M, F, L.ptr(w1), L.ptr(w2), L.ptr(t), L.ptr(g_w1),
+                                 L.ptr(g_b1), L.ptr(g_w2), L.ptr(g_b2), L.ptr(gx), int(accumulate), int(gelu_bwd),
+                                 L.stream()), "mole_ffn_bwd")
+    return gx

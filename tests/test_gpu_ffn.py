@@ -1,0 +1,99 @@
+"""HIP grouped expert FFN forward/backward (MFMA kernels) against the CPU oracle, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+from tests.util import rel_err, tol
+
+pytestmark = pytest.mark.gpu
+
+
+def _make(E, M, Fd, rows_per_expert, dtype, seed=0, pad_between=0):
+    g = torch.Generator().manual_seed(seed)
+    n = np.array(rows_per_expert, dtype=np.int32)
+    off = np.zeros(E + 1, dtype=np.int32)
+    off[1:] = np.cumsum(n + pad_between)
+    R = int(off[-1])
+    r = lambda *s, sc=1.0: (torch.randn(*s, generator=g) * sc).to(dtype)
+    d = dict(xd=r(max(R, 1), M), w1=r(E, Fd, M, sc=0.05), b1=r(E, Fd, sc=0.05), w2=r(E, Fd, M, sc=0.05),
+             b2=r(E, M, sc=0.05), go=r(max(R, 1), M), n=n, off=off, R=R)
+    return d
+
+
+def _oracle_fwd_bwd(d, gelu_bwd):
+    """fp32 oracle on the same (rounded) inputs, per expert over its kept rows only."""
+    f = {k: (v.float() if torch.is_tensor(v) else v) for k, v in d.items()}
+    E = f["w1"].shape[0]
+    R, M, Fd = d["R"], f["w1"].shape[2], f["w1"].shape[1]
+    out = torch.zeros(max(R, 1), M); h = torch.zeros(max(R, 1), Fd)
+    gx = torch.zeros(max(R, 1), M)
+    g_w1 = torch.zeros_like(f["w1"]); g_w2 = torch.zeros_like(f["w2"])
+    g_b1 = torch.zeros(E, Fd); g_b2 = torch.zeros(E, M)
+    for e in range(E):
+        lo, hi = int(d["off"][e]), int(d["off"][e]) + int(d["n"][e])
+        if hi <= lo:
+            continue
+        o_e, h_e = O.ffn_fwd(f["xd"][lo:hi][None], f["w1"][e:e + 1], f["b1"][e:e + 1], f["w2"][e:e + 1], f["b2"][e:e + 1])
+        out[lo:hi], h[lo:hi] = o_e[0], h_e[0]
+        a, b, c_, dd, ee = O.ffn_bwd(f["go"][lo:hi][None], f["xd"][lo:hi][None], h_e, f["w1"][e:e + 1], f["w2"][e:e + 1], gelu_bwd)
+        g_w1[e], g_b1[e], g_w2[e], g_b2[e], gx[lo:hi] = a[0], b[0], c_[0], dd[0], ee[0]
+    return out, h, gx, g_w1, g_b1, g_w2, g_b2
+
+
+CASES = [
+    # E, M, F, rows per expert, gap between experts (padded layout has gaps)
+    (1, 64, 128, [5], 0),
+    (4, 64, 128, [130, 0, 7, 64], 0),
+    (3, 136, 264, [257, 31, 129], 3),
+    (8, 256, 512, [100, 200, 0, 1, 300, 128, 127, 129], 0),
+    (2, 512, 2048, [1024, 1000], 24),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("gelu_bwd", ["tanh", "exact"])
+@pytest.mark.parametrize("E,M,Fd,rows,gap", CASES)
+def test_ffn_fwd_bwd_matches_oracle(E, M, Fd, rows, gap, gelu_bwd, dtype):
+    from mole_amd import hip_ops as H, _lib as L
+    print(f"ffn E={E} M={M} F={Fd} rows={rows} gap={gap} {gelu_bwd} {dtype}", flush=True)
+    d = _make(E, M, Fd, rows, dtype, seed=E * 7 + M, pad_between=gap)
+    c = {k: (v.cuda() if torch.is_tensor(v) else v) for k, v in d.items()}
+    off = torch.from_numpy(d["off"]).cuda(); n = torch.from_numpy(d["n"]).cuda()
+    out, h, a = H.ffn_fwd(c["xd"], off, n, c["w1"], c["b1"], c["w2"], c["b2"])
+    w_out, w_h, w_gx, w_gw1, w_gb1, w_gw2, w_gb2 = _oracle_fwd_bwd(d, gelu_bwd)
+    t = tol(dtype)
+    mask = torch.zeros(max(d["R"], 1), dtype=torch.bool)
+    for e in range(E):
+        mask[int(d["off"][e]):int(d["off"][e]) + int(d["n"][e])] = True
+    assert rel_err(h.cpu()[mask], w_h[mask]) < t
+    assert rel_err(out.cpu()[mask], w_out[mask]) < t
+    assert rel_err(a.cpu()[mask], torch.nn.functional.gelu(w_h[mask])) < t
+    g_w1 = torch.full_like(c["w1"], 9.0); g_w2 = torch.full_like(c["w2"], 9.0)
+    g_b1 = torch.full_like(c["b1"], 9.0); g_b2 = torch.full_like(c["b2"], 9.0)
+    mode = L.GELU_BWD_TANH if gelu_bwd == "tanh" else L.GELU_BWD_EXACT
+    gx = H.ffn_bwd(c["go"], c["xd"], h, a, off, n, c["w1"], c["w2"], g_w1, g_b1, g_w2, g_b2, True, False, mode)
+    # the backward consumes the GPU's own saved h (rounded to the storage dtype), so compare against the
+    # oracle evaluated on that same h for the tight fp32 bound
+    assert rel_err(gx.cpu()[mask], w_gx[mask]) < t
+    assert rel_err(g_w2, w_gw2) < t
+    assert rel_err(g_b2, w_gb2) < t
+    assert rel_err(g_w1, w_gw1) < t
+    assert rel_err(g_b1, w_gb1) < t
+    # accumulate variant (bffn_bwd_acc): a second call adds the same gradients again
+    if dtype == torch.float32:
+        H.ffn_bwd(c["go"], c["xd"], h, a, off, n, c["w1"], c["w2"], g_w1, g_b1, g_w2, g_b2, False, True, mode)
+        assert rel_err(g_w1, 2 * w_gw1) < t and rel_err(g_b2, 2 * w_gb2) < t
+        assert rel_err(g_w2, 2 * w_gw2) < t and rel_err(g_b1, 2 * w_gb1) < t
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gemm_nt_gate_logits(dtype):
+    from mole_amd import hip_ops as H
+    print(f"gemm_nt {dtype}", flush=True)
+    g = torch.Generator().manual_seed(1)
+    for rows, N, K in [(1, 1, 8), (300, 16, 512), (1000, 256, 1024), (129, 100, 264)]:
+        a = torch.randn(rows, K, generator=g).to(dtype); b = (torch.randn(N, K, generator=g) * 0.05).to(dtype)
+        c = H.gemm_nt(a.cuda(), b.cuda())
+        want = a.float() @ b.float().t()
+        assert rel_err(c, want) < (1e-5 if dtype == torch.float32 else 1e-4)   # fp32 accumulation of exact products

@@ -1,0 +1,71 @@
+"""HIP dispatch / combine forward and backward against the CPU oracle, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+from tests.util import rel_err, tol, zipf_scores
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("ragged", [True, False])
+@pytest.mark.parametrize("S,E,k,cf,M", [(1, 2, 1, 1.0, 8), (300, 8, 2, 1.0, 64), (1000, 16, 1, 0.5, 520),
+                                        (513, 4, 4, 0.0, 1024), (200, 32, 8, 0.0, 2048)])
+def test_permutes_match_oracle(S, E, k, cf, M, ragged, dtype):
+    from mole_amd import hip_ops as H, _lib as L
+    print(f"permute S={S} E={E} k={k} cf={cf} M={M} ragged={ragged} {dtype}", flush=True)
+    g = torch.Generator().manual_seed(S + M)
+    scores = zipf_scores(S, E, seed=S)
+    c = O.extract_critical(scores.numpy(), k, cf)
+    r = H.route(scores.cuda(), k, cf, True, 1, L.LAYOUT_RAGGED if ragged else L.LAYOUT_PADDED)
+    total = int(c.offsets[-1]) if ragged else E * c.capacity
+    x = torch.randn(S, M, generator=g).to(dtype)
+    xf = x.float()
+    # dispatch forward: a pure copy, exact in every dtype; padding rows zeroed like the reference's buffer
+    xd = torch.full((max(total, 1), M), 7.0, dtype=dtype, device="cuda")
+    H.dispatch_fwd(x.cuda(), r.row, total, out=xd)
+    H.zero_pad_rows(xd, r.kept_rows, r.offsets)
+    want = O.fast_encode(xf, c, ragged).reshape(total, M)
+    assert torch.equal(xd[:total].float().cpu(), want)
+    # combine forward
+    o = torch.randn(max(total, 1), M, generator=g).to(dtype)
+    y = H.combine_fwd(o.cuda(), r.row, r.gates)
+    want_y = O.fast_decode(o[:total].float(), c, ragged)
+    assert rel_err(y, want_y) < tol(dtype)
+    # combine backward
+    dy = torch.randn(S, M, generator=g).to(dtype)
+    d_o = torch.full((max(total, 1), M), 3.0, dtype=dtype, device="cuda")
+    d_o, dg = H.combine_bwd(dy.cuda(), o.cuda(), r.row, r.gates, d_o)
+    H.zero_pad_rows(d_o, r.kept_rows, r.offsets)
+    want_do, want_dg = O.fast_decode_bwd(dy.float(), o[:total].float(), c, ragged)
+    assert rel_err(d_o[:total], want_do) < tol(dtype)
+    assert rel_err(dg, want_dg) < (1e-5 if dtype == torch.float32 else 1e-4)   # fp32 sums of exact products
+    # dispatch backward, alone and with the gate's input gradient folded in
+    dxd = torch.randn(max(total, 1), M, generator=g).to(dtype)
+    dx = H.dispatch_bwd(dxd.cuda(), r.row)
+    want_dx = O.fast_encode_bwd(dxd[:total].float(), c, ragged)
+    assert rel_err(dx, want_dx) < tol(dtype)
+    dlog = torch.randn(S, E, generator=g) * 0.1
+    wg = torch.randn(E, M, generator=g)
+    dx2 = H.dispatch_bwd(dxd.cuda(), r.row, dlog.cuda(), wg.cuda())
+    assert rel_err(dx2, want_dx + dlog @ wg) < tol(dtype)
+
+
+def test_permute_full_size_properties():
+    """c5-sized round trip: combine(dispatch(x)) with unit gates = k*x, and <dispatch(x), D> = <x, dispatch_bwd(D)>."""
+    from mole_amd import hip_ops as H
+    S, E, k, M = 32768, 256, 8, 2048
+    print("permute full size c5", flush=True)
+    scores = zipf_scores(S, E, seed=2).cuda()
+    r = H.route(scores, k, 0.0, normalize_gate=False)
+    x = torch.randn(S, M, device="cuda").bfloat16()
+    xd = H.dispatch_fwd(x, r.row, S * k)
+    y = H.combine_fwd(xd, r.row, torch.ones_like(r.gates))
+    assert torch.equal(y.float(), (x.float() * k).bfloat16().float())
+    d = torch.randn(S * k, M, device="cuda").bfloat16()
+    lhs = (xd.double() * d.double()).sum()
+    dx = H.dispatch_bwd(d, r.row)
+    rhs = (x.double() * dx.double()).sum()
+    assert abs(float(lhs - rhs)) < 2e-3 * abs(float(lhs)) + 50.0   # dx is rounded to bf16 once

@@ -1,0 +1,83 @@
+"""HIP routing (mole_route, mole_softmax_fwd, mole_gate_bwd) against the CPU oracle, through the C ABI.
+Integer outputs are compared bit for bit; gates too (same fp32 operations in the same order)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+from tests.util import crit_to_numpy, rel_err, zipf_scores
+
+pytestmark = pytest.mark.gpu
+
+
+def _compare(scores, k, cf, layout_ragged, normalize=True, alignment=1):
+    from mole_amd import hip_ops as H, _lib as L
+    r = H.route(scores.cuda(), k, cf, normalize, alignment, L.LAYOUT_RAGGED if layout_ragged else L.LAYOUT_PADDED)
+    got = crit_to_numpy(r)
+    c = O.extract_critical(scores.numpy(), k, cf, normalize, alignment)
+    kk = c.top_k
+    np.testing.assert_array_equal(got["idx"], np.stack(c.indices_s))
+    np.testing.assert_array_equal(got["counts"], c.counts)
+    np.testing.assert_array_equal(got["loc"], np.stack(c.locations_s))
+    assert got["capacity"] == c.capacity
+    np.testing.assert_array_equal(got["kept"], c.kept_rows)
+    want_off = c.offsets if layout_ragged else np.arange(c.num_experts + 1, dtype=np.int32) * c.capacity
+    np.testing.assert_array_equal(got["offsets"], want_off)
+    np.testing.assert_array_equal(got["row"], c.rows(layout_ragged))
+    np.testing.assert_array_equal(got["gates"], np.stack(c.gates_s))
+    assert abs(got["l_aux"] - c.l_aux) <= 1e-5 * max(1.0, abs(c.l_aux))
+    assert kk == r.k
+
+
+@pytest.mark.parametrize("S,E,k,cf", [
+    (1, 1, 1, 1.0), (5, 3, 2, 0.0), (255, 8, 2, 1.0), (256, 8, 2, 1.0), (257, 8, 2, 0.5),
+    (1000, 16, 1, 1.25), (777, 5, 5, 0.0), (4096, 64, 2, 0.0), (3000, 100, 4, -0.5),
+    (2048, 256, 8, 0.0), (600, 1024, 16, 0.0), (4096, 8, 2, 1.0),
+])
+@pytest.mark.parametrize("ragged", [True, False])
+def test_route_matches_oracle(S, E, k, cf, ragged):
+    print(f"route S={S} E={E} k={k} cf={cf} ragged={ragged}", flush=True)
+    _compare(zipf_scores(S, E, seed=S + E + k), k, cf, ragged)
+
+
+def test_route_ties_nan_alignment_and_unnormalised():
+    print("route ties", flush=True)
+    _compare(zipf_scores(1500, 16, seed=3, ties=True), 4, 0.0, True)
+    _compare(torch.full((700, 32), 1.0 / 32), 3, 1.0, False)            # every score equal
+    s = zipf_scores(300, 8, seed=9)
+    s[5, 3] = float("nan"); s[17, :] = float("nan"); s[40, 0] = float("inf")
+    from mole_amd import hip_ops as H
+    r = H.route(s.cuda(), 2, 0.0)
+    c = O.extract_critical(s.numpy(), 2, 0.0)
+    np.testing.assert_array_equal(r.idx.cpu().numpy(), np.stack(c.indices_s))
+    np.testing.assert_array_equal(r.loc.cpu().numpy(), np.stack(c.locations_s))
+    _compare(zipf_scores(900, 8, seed=4), 2, 0.0, True, normalize=False)
+    _compare(zipf_scores(900, 8, seed=5), 2, 0.0, False, alignment=64)
+
+
+@pytest.mark.parametrize("name,S,E,k,cf", [("c2", 16384, 16, 1, 1.25), ("c3", 8192, 64, 2, 0.0),
+                                           ("c5", 32768, 256, 8, 0.0)])
+def test_route_full_size_configs(name, S, E, k, cf):
+    print(f"route full {name}", flush=True)
+    _compare(zipf_scores(S, E, seed=1), k, cf, True)
+
+
+@pytest.mark.parametrize("S,E", [(100, 8), (513, 16), (64, 100), (300, 256)])
+def test_softmax_and_gate_bwd(S, E):
+    from mole_amd import hip_ops as H
+    print(f"softmax/gate_bwd S={S} E={E}", flush=True)
+    g = torch.Generator().manual_seed(S)
+    logits = torch.randn(S, E, generator=g) * 3
+    bias = torch.randn(E, generator=g)
+    sc = H.softmax_fwd(logits.cuda(), bias.cuda())
+    want = torch.softmax(logits + bias, dim=-1)
+    assert rel_err(sc, want) < 1e-6
+    assert rel_err(H.softmax_fwd(logits.cuda()), torch.softmax(logits, dim=-1)) < 1e-6
+    for k, norm in [(1, True), (min(3, E), True), (min(3, E), False)]:
+        scores = sc.cpu()
+        c = O.extract_critical(scores.numpy(), k, 0.0, norm)
+        dg = torch.randn(c.top_k, S, generator=g)
+        want_dl = O.softmax_bwd(O.gate_normalize_bwd(dg, scores, c, norm), scores)
+        idx = torch.from_numpy(np.stack(c.indices_s)).cuda()
+        got = H.gate_bwd(dg.cuda(), sc, idx, norm)
+        assert rel_err(got, want_dl) < 1e-5

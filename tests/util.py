@@ -1,0 +1,40 @@
+"""Shared helpers of the GPU parity tests."""
+import numpy as np
+import torch
+
+
+def rel_err(got: torch.Tensor, want: torch.Tensor) -> float:
+    """max |got - want| / max |want|: the relative error the 1e-5 (fp32) and 2e-2 (bf16)
+    tolerances of the parity tests are stated in."""
+    got = got.detach().double().cpu()
+    want = want.detach().double().cpu()
+    denom = float(want.abs().max())
+    if denom == 0.0:
+        return float(got.abs().max())
+    return float((got - want).abs().max()) / denom
+
+
+FP32_TOL = 1e-5
+BF16_TOL = 2e-2
+
+
+def tol(dtype) -> float:
+    return FP32_TOL if dtype == torch.float32 else BF16_TOL
+
+
+def zipf_scores(S, E, seed, ties=False):
+    g = torch.Generator().manual_seed(seed)
+    logits = torch.randn(S, E, generator=g)
+    logits += torch.log(torch.arange(1, E + 1, dtype=torch.float32) ** -1.2)[torch.randperm(E, generator=g)]
+    s = torch.softmax(logits, dim=-1)
+    if ties and E >= 4:
+        s[:, E - 1] = s[:, 0]          # whole duplicated columns: exact ties in every row
+        s[::3, 1] = s[::3, 2]
+    return s.contiguous()
+
+
+def crit_to_numpy(r):
+    """mole_amd.hip_ops.Route -> dict of numpy arrays (one host copy for the whole comparison)."""
+    return dict(idx=r.idx.cpu().numpy(), loc=r.loc.cpu().numpy(), gates=r.gates.cpu().numpy(),
+                row=r.row.cpu().numpy(), counts=r.counts.cpu().numpy(), kept=r.kept_rows.cpu().numpy(),
+                offsets=r.offsets.cpu().numpy(), capacity=int(r.capacity.cpu()), l_aux=float(r.l_aux.cpu()))
