@@ -52,6 +52,29 @@ enum {
 int mole_version(void);
 const char *mole_last_error_string(void);
 
+/* Optional per-kernel timing for benchmarks (no counterpart in the reference, whose timers wrap
+ * whole layers: MOLE/utils/Utimer.py:5-70).  While enabled, each kernel below is bracketed by two
+ * events on the stream it runs on; mole_kernel_timing_read() waits for them and returns, for ids
+ * 0..n_ids-1, the number of launches and their summed duration in ms, then forgets them. */
+enum {
+    MOLE_K_FFN_FWD1 = 0,  /* h = xd.w1^T + b1, a = gelu(h) */
+    MOLE_K_FFN_FWD2 = 1,  /* out = a.w2 + b2 */
+    MOLE_K_FFN_GW2 = 2,   /* g_w2 = a^T.go */
+    MOLE_K_FFN_DA = 3,    /* t = (go.w2^T) * gelu'(h) */
+    MOLE_K_FFN_GW1 = 4,   /* g_w1 = t^T.xd */
+    MOLE_K_FFN_GX = 5,    /* gx = t.w1 */
+    MOLE_K_FFN_GB = 6,    /* bias gradients */
+    MOLE_K_DISPATCH_FWD = 7,
+    MOLE_K_DISPATCH_BWD = 8,
+    MOLE_K_COMBINE_FWD = 9,
+    MOLE_K_COMBINE_BWD = 10,
+    MOLE_K_ROUTE = 11,    /* the four routing kernels together */
+    MOLE_K_GEMM_NT = 12,
+    MOLE_K_COUNT = 13
+};
+int mole_kernel_timing_enable(int on);
+int mole_kernel_timing_read(int n_ids, int *counts, float *ms_total);
+
 /* ------------------------------------------------------------------------------------------
  * Gate.  Replaces MOLETopk.forward (MOLE/utils/Ugate.py:11-14): scores = softmax(logits).
  * logits [S,E] fp32 (x . Wg^T, produced by mole_gemm_nt or any GEMM); logit_bias [E] or NULL.

@@ -18,11 +18,15 @@ MOLE_F32, MOLE_BF16 = 0, 1
 LAYOUT_PADDED, LAYOUT_RAGGED = 0, 1
 GELU_BWD_TANH, GELU_BWD_EXACT = 0, 1
 MAX_TOPK, MAX_EXPERTS = 16, 1024
+KERNEL_IDS = ("ffn_fwd1", "ffn_fwd2", "ffn_gw2", "ffn_da", "ffn_gw1", "ffn_gx", "ffn_gb", "dispatch_fwd", "dispatch_bwd",
+              "combine_fwd", "combine_bwd", "route", "gemm_nt")
 
 _P = c_void_p
 _SIGNATURES = {
     "mole_version": (c_int, []),
     "mole_last_error_string": (c_char_p, []),
+    "mole_kernel_timing_enable": (c_int, [c_int]),
+    "mole_kernel_timing_read": (c_int, [c_int, POINTER(c_int), POINTER(c_float)]),
     "mole_softmax_fwd": (c_int, [_P, _P, c_int, c_int, _P, _P]),
     "mole_gate_bwd": (c_int, [_P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P, _P]),
     "mole_route_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
@@ -81,6 +85,18 @@ def last_error() -> str:
 def check(rc: int, what: str) -> None:
     if rc != 0:
         raise RuntimeError(f"{what} failed (code {rc}): {last_error()}")
+
+
+def kernel_timing_enable(on: bool) -> None:
+    check(lib().mole_kernel_timing_enable(int(on)), "mole_kernel_timing_enable")
+
+
+def kernel_timing_read() -> dict:
+    """{kernel name: (launches, total ms)} since the last read; waits for the recorded events."""
+    n = len(KERNEL_IDS)
+    counts, ms = (c_int * n)(), (c_float * n)()
+    check(lib().mole_kernel_timing_read(n, counts, ms), "mole_kernel_timing_read")
+    return {KERNEL_IDS[i]: (counts[i], ms[i]) for i in range(n)}
 
 
 def ptr(t):

@@ -1,0 +1,360 @@
+"""Host side of the expert pipeline: the module the reference reaches as `UniMoE.core` (pybind,
+MOLE/cpp/core.cpp:1347-1469), re-hosted in Python over the C ABI of libmole_hip.so.
+
+What is mirrored (same names, same argument meaning):
+  create_UniMem / clear_virtual_mem / view_pool_size / fetch_top_prefetched_batch /
+  synchronize_tran / default_wait_tran / fast_assign_prefetch       core.cpp:1397-1432
+  MOLECore(...).forward / .backward / .prefetch_fwd / .prefetch_bwd / .dummy_fetch /
+  .set_GPUParamCore / .set_CPUParamCore                               core.cpp:1356-1388
+  BatchFusedFWD  - the autograd.Function MOLE/moe/layer.py:453 calls but the reference snapshot
+                   never defines; it forwards to MOLECore.forward / MOLECore.backward
+                   (define.hpp:594-606).
+
+The expert math itself (two grouped GEMMs forward, four backward, bias/GELU/GELU' epilogues) is
+mole_ffn_fwd / mole_ffn_bwd; this file only decides which experts run from which memory:
+GPU-resident ("static") experts in one grouped launch, offloaded ("dynamic") experts in chunks that
+fit the free part of the slot pool (core.cpp:1020-1051), each chunk fetched on the copy stream and
+handed to the compute stream through events (core.cpp:110-143, 212-249).
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_uint64, c_void_p
+from typing import List, Optional
+
+import torch
+
+from . import _lib as L
+from . import hip_ops as H
+
+_DTYPES = {"torch.float32": torch.float32, "torch.bfloat16": torch.bfloat16}
+
+
+# ---------------------------------------------------------------------------------------------
+# slot pool (process-global, first caller wins: umemory.cpp:77-86)
+# ---------------------------------------------------------------------------------------------
+class UniMem:
+    def __init__(self, device: int, pool_size: int, dtype: torch.dtype, F: int, M: int):
+        self.device, self.pool_size, self.dtype, self.F, self.M = device, pool_size, dtype, F, M
+        self._h = c_void_p()
+        L.check(L.lib().mole_unimem_create(device, max(pool_size, 0), L.dtype_code(dtype), F, M, ctypes.byref(self._h)),
+                "mole_unimem_create")
+
+    def close(self):
+        if self._h:
+            L.check(L.lib().mole_unimem_destroy(self._h), "mole_unimem_destroy")
+            self._h = c_void_p()
+
+    def _int(self, fn) -> int:
+        out = c_int()
+        L.check(fn(self._h, ctypes.byref(out)), fn.__name__)
+        return out.value
+
+    def view_pool_size(self) -> int:
+        return self._int(L.lib().mole_unimem_view_pool_size)
+
+    def virtual_offset(self) -> int:
+        return self._int(L.lib().mole_unimem_virtual_offset)
+
+    def clear_virtual_mem(self):
+        L.check(L.lib().mole_unimem_clear_virtual_mem(self._h), "mole_unimem_clear_virtual_mem")
+
+    @staticmethod
+    def _src(host_tensors):
+        arr = (c_void_p * 4)()
+        for i, t in enumerate(host_tensors):
+            arr[i] = t.data_ptr()
+        return arr
+
+    def prefetch(self, layer: int, host_tensors, base: int, n: int):
+        L.check(L.lib().mole_unimem_prefetch(self._h, layer, self._src(host_tensors), base, n), "mole_unimem_prefetch")
+
+    def fetch_top(self, layer: int) -> int:
+        out = c_int()
+        L.check(L.lib().mole_unimem_fetch_top(self._h, layer, ctypes.byref(out)), "mole_unimem_fetch_top")
+        return out.value
+
+    def fetch(self, host_tensors, view_base: int, base: int, n: int, prefetched: int) -> List[int]:
+        ptrs = (c_void_p * 4)()
+        L.check(L.lib().mole_unimem_fetch(self._h, self._src(host_tensors), view_base, base, n, prefetched, ptrs),
+                "mole_unimem_fetch")
+        return [int(p) for p in ptrs]
+
+    def wait_params(self):
+        L.check(L.lib().mole_unimem_wait_params(self._h, L.stream()), "mole_unimem_wait_params")
+
+    def release(self, view_base: int, n: int):
+        L.check(L.lib().mole_unimem_release(self._h, view_base, n, L.stream()), "mole_unimem_release")
+
+    def sync_tran(self):
+        L.check(L.lib().mole_unimem_sync_tran(self._h), "mole_unimem_sync_tran")
+
+    def tran_stream_handle(self) -> int:
+        out = c_void_p()
+        L.check(L.lib().mole_unimem_tran_stream(self._h, ctypes.byref(out)), "mole_unimem_tran_stream")
+        return int(out.value or 0)
+
+    def copy_stats(self):
+        b, ms = c_uint64(), c_float()
+        L.check(L.lib().mole_unimem_copy_stats(self._h, ctypes.byref(b), ctypes.byref(ms)), "mole_unimem_copy_stats")
+        return b.value, ms.value
+
+    def slot_tensor(self, p_id: int, slot: int, n: int) -> torch.Tensor:
+        """Device pointer of `slot` for parameter kind p_id (debug / tests)."""
+        out = c_void_p()
+        L.check(L.lib().mole_unimem_slot_ptr(self._h, p_id, slot, ctypes.byref(out)), "mole_unimem_slot_ptr")
+        return int(out.value)
+
+
+_UniMemInst: List[UniMem] = []
+
+
+def create_UniMem(device, pool_size, dtype, sizes) -> UniMem:
+    """create_UniMem(local_rank, pool_size, "torch.float32", [[F,M],[F],[F,M],[M]]) - layer.py:43-47."""
+    if _UniMemInst:
+        return _UniMemInst[0]
+    dt = _DTYPES[dtype] if isinstance(dtype, str) else dtype
+    F, M = int(sizes[0][0]), int(sizes[0][1])
+    um = UniMem(int(device), int(pool_size), dt, F, M)
+    _UniMemInst.append(um)
+    return um
+
+
+def get_UniMem() -> Optional[UniMem]:
+    return _UniMemInst[0] if _UniMemInst else None
+
+
+def destroy_UniMem():
+    while _UniMemInst:
+        _UniMemInst.pop().close()
+
+
+def clear_virtual_mem():
+    _UniMemInst[0].clear_virtual_mem()
+
+
+def view_pool_size() -> int:
+    return _UniMemInst[0].view_pool_size()
+
+
+def fetch_top_prefetched_batch(moe_id: int) -> int:
+    return _UniMemInst[0].fetch_top(moe_id)
+
+
+def synchronize_tran():
+    if _UniMemInst:
+        _UniMemInst[0].sync_tran()
+
+
+def default_wait_tran():
+    if _UniMemInst:
+        _UniMemInst[0].wait_params()
+
+
+def fast_assign_prefetch(P: int, Fv, Ev):
+    """(GPscheme, LPscheme) as core.cpp:1302-1345: GPscheme[i] = [[later_layer, count], ...]."""
+    n = len(Ev)
+    IntN = c_int * max(n, 1)
+    lp = IntN()
+    cap = 4 * n + 4
+    gp = (c_int * (3 * cap))()
+    gpn = c_int()
+    L.check(L.lib().mole_fast_assign_prefetch(int(P), IntN(*[int(v) for v in Fv]), IntN(*[int(v) for v in Ev]), n, lp, gp,
+                                              cap, ctypes.byref(gpn)), "mole_fast_assign_prefetch")
+    scheme = [[] for _ in range(n)]
+    for i in range(gpn.value):
+        scheme[gp[3 * i]].append([gp[3 * i + 1], gp[3 * i + 2]])
+    return scheme, [lp[i] for i in range(n)]
+
+
+# ---------------------------------------------------------------------------------------------
+# per-layer core
+# ---------------------------------------------------------------------------------------------
+class MOLECore:
+    """Per-layer state and the expert-batch pipeline (define.hpp:338-607, core.cpp:991-1300)."""
+
+    def __init__(self, use_pool, mome_use_pool, vari_use_pool, grad_use_pool, s_experts, d_experts, ebatch_size,
+                 world_size, act_name, adv_adam, acc_step, step, device, moe_id, total_experts,
+                 gelu_bwd: str = "tanh"):
+        if world_size != 1:
+            raise NotImplementedError("this build covers the single-GPU hot path (world_size == 1)")
+        if act_name != "gelu":
+            raise NotImplementedError("only act='gelu' is on the hot path")
+        if adv_adam:
+            raise NotImplementedError("in-pipeline Adam (adv_adam) is outside the hot path")
+        self.use_pool, self.acc_step, self.step = bool(use_pool), int(acc_step), int(step)
+        self.device, self.moe_id, self.total_experts = device, moe_id, total_experts
+        self.s_experts, self.d_experts, self.ebatch_size = s_experts, d_experts, max(int(ebatch_size), 1)
+        self.world_size, self.act_name = world_size, act_name
+        self.fwd_base = self.bwd_base = 0
+        self.gelu_bwd = L.GELU_BWD_TANH if gelu_bwd == "tanh" else L.GELU_BWD_EXACT
+        self.gpu = [None] * 4       # (all_tensors, grad_tensors)
+        self.cpu = [None] * 4       # (all_tensors, grad_)
+        self._saved = None
+
+    # parameter stores -------------------------------------------------------------------------
+    def set_GPUParamCore(self, p_id, all_tensors, grad_tensors, bias):
+        self.gpu[p_id] = (all_tensors, grad_tensors)
+
+    def set_CPUParamCore(self, p_id, all_tensors, grad_, momentum, variance, bias, p_id2=None):
+        self.cpu[p_id] = (all_tensors, grad_)
+
+    def _host(self):
+        return [c[0] for c in self.cpu]
+
+    # prefetch -----------------------------------------------------------------------------------
+    def prefetch_fwd(self, batch_size: int):
+        if batch_size == 0:
+            return
+        get_UniMem().prefetch(self.moe_id, self._host(), self.fwd_base, batch_size)
+        self.fwd_base += batch_size
+
+    def prefetch_bwd(self, batch_size: int):
+        if batch_size == 0:
+            return
+        get_UniMem().prefetch(self.moe_id, self._host(), self.bwd_base, batch_size)
+        self.bwd_base += batch_size
+
+    def dummy_fetch(self, batch_size: int):
+        """Copy `batch_size` experts into slots 0.. without reserving them (core.cpp:25-39)."""
+        if batch_size == 0:
+            return
+        um = get_UniMem()
+        um.fetch(self._host(), -um.virtual_offset(), 0, batch_size, 0)
+
+    # pipeline -----------------------------------------------------------------------------------
+    def _chunks(self, prefetched: int):
+        """Offloaded experts -> [(base, size, already_prefetched, view_base)] (core.cpp:1020-1051)."""
+        um = get_UniMem()
+        if self.d_experts == 0:
+            return []
+        if not self.use_pool or um is None or um.pool_size <= 0:
+            raise RuntimeError("offloaded experts need the slot pool (pool_size >= 1, use_pool=True)")
+        vps = um.view_pool_size()
+        if vps <= 0:
+            raise RuntimeError("slot pool exhausted by prefetches: no slot left to run offloaded experts")
+        d_batch = min(self.ebatch_size, vps)
+        out, view_base, i = [], 0, 0
+        while i < self.d_experts:
+            size = min(d_batch, self.d_experts - i)
+            if vps - view_base < size:
+                view_base = 0
+            out.append((i, size, max(0, min(size, prefetched - i)), view_base))
+            view_base += size
+            i += d_batch
+        return out
+
+    def forward(self, dispatched_input: torch.Tensor, requires_grad: bool, offsets=None, kept_rows=None,
+                return_saved: bool = False):
+        """dispatched_input: [E, C, M] (reference layout; every row is computed, like the reference)
+        or, with offsets/kept_rows from mole_route, any [rows, M] expert-contiguous buffer of which
+        only the kept rows are computed.  Returns a tensor of the same shape."""
+        x = dispatched_input
+        shape = x.shape
+        M = shape[-1]
+        E = self.s_experts + self.d_experts
+        if offsets is None:
+            assert x.dim() == 3 and shape[0] == E, f"expected [E={E}, C, M], got {tuple(shape)}"
+            C = shape[1]
+            offsets = torch.arange(E + 1, dtype=torch.int32, device=x.device) * C
+            kept_rows = torch.full((E,), C, dtype=torch.int32, device=x.device)
+        x2 = x.reshape(-1, M)
+        if not x2.is_contiguous():
+            x2 = x2.contiguous()
+        rows = x2.shape[0]
+        F = (self.gpu[0][0] if self.s_experts else self.cpu[0][0]).shape[1]
+        h = torch.empty(rows, F, dtype=x.dtype, device=x.device)
+        a = torch.empty(rows, F, dtype=x.dtype, device=x.device)
+        out = torch.empty(rows, M, dtype=x.dtype, device=x.device)
+        if self.s_experts:
+            w1, b1, w2, b2 = (g[0] for g in self.gpu)
+            H.ffn_fwd_into(x2, offsets, kept_rows, self.s_experts, rows, M, F, w1, b1, w2, b2, h, a, out)
+        if self.d_experts:
+            um = get_UniMem()
+            prefetched = um.fetch_top(self.moe_id)
+            if prefetched != self.fwd_base:
+                raise RuntimeError(f"prefetch stack out of order: top holds {prefetched}, layer expects {self.fwd_base}")
+            self.fwd_base = 0
+            for (base, size, pref, view_base) in self._chunks(prefetched):
+                p = um.fetch(self._host(), view_base, base, size, pref)
+                um.wait_params()
+                e0 = self.s_experts + base
+                H.ffn_fwd_into(x2, offsets[e0:], kept_rows[e0:], size, rows, M, F, p[0], p[1], p[2], p[3], h, a, out)
+                um.release(view_base, size)
+        saved = (x2, h, a, offsets, kept_rows, requires_grad, shape)
+        if return_saved:          # the caller (an autograd node) keeps the activations itself
+            return out.view(shape), saved
+        self._saved = saved       # reference behaviour: the core holds them until backward (define.hpp:594-606)
+        return out.view(shape)
+
+    def backward(self, all_output_grad: torch.Tensor, saved=None):
+        if saved is None:
+            saved, self._saved = self._saved, None
+        if saved is None:
+            raise RuntimeError("MOLECore.backward without a preceding forward")
+        x2, h, a, offsets, kept_rows, need_gx, shape = saved
+        M = shape[-1]
+        go = all_output_grad.reshape(-1, M)
+        if not go.is_contiguous():
+            go = go.contiguous()
+        rows = x2.shape[0]
+        F = h.shape[1]
+        t = torch.empty(rows, F, dtype=x2.dtype, device=x2.device)
+        gx = torch.empty(rows, M, dtype=x2.dtype, device=x2.device) if need_gx else None
+        acc = self.acc_step > 1
+        if self.s_experts:
+            w1, _, w2, _ = (g[0] for g in self.gpu)
+            gw1, gb1, gw2, gb2 = (g[1] for g in self.gpu)
+            H.ffn_bwd_into(go, x2, h, a, offsets, kept_rows, self.s_experts, rows, M, F, w1, w2, t, gw1, gb1, gw2, gb2,
+                           gx, acc, self.gelu_bwd)
+        if self.d_experts:
+            um = get_UniMem()
+            prefetched = um.fetch_top(self.moe_id)
+            if prefetched != self.bwd_base:
+                raise RuntimeError(f"prefetch stack out of order: top holds {prefetched}, layer expects {self.bwd_base}")
+            self.bwd_base = 0
+            host_grads = [c[1] for c in self.cpu]
+            for (base, size, pref, view_base) in self._chunks(prefetched):
+                p = um.fetch(self._host(), view_base, base, size, pref)   # weights are fetched again (core.cpp:1203)
+                um.wait_params()
+                e0 = self.s_experts + base
+                g = [torch.empty((size, *hg.shape[1:]), dtype=hg.dtype, device=x2.device) for hg in host_grads]
+                H.ffn_bwd_into(go, x2, h, a, offsets[e0:], kept_rows[e0:], size, rows, M, F, p[0], p[2], t, g[0], g[1],
+                               g[2], g[3], gx, False, self.gelu_bwd)
+                um.release(view_base, size)
+                self._store_grad(host_grads, g, base, size)
+        self.step += 1
+        for c in self.cpu:
+            if c is not None and hasattr(c[1], "lazy_zero"):
+                c[1].lazy_zero = False
+        return gx.view(shape) if need_gx else None
+
+    def _store_grad(self, host_grads, g, base, size):
+        """Gradients of offloaded experts go back to their pinned host buffers (core.cpp:77-103,
+        uparameter.cpp:68-83): overwrite, or add when accumulating and the buffer is not lazily zero."""
+        for hg, gg in zip(host_grads, g):
+            dst = hg[base:base + size]
+            if self.acc_step > 1 and not getattr(hg, "lazy_zero", True):
+                dst += gg.to("cpu")
+            else:
+                dst.copy_(gg, non_blocking=True)
+
+
+class BatchFusedFWD(torch.autograd.Function):
+    """experts_output = BatchFusedFWD.apply(dispatched_input, module, dummy_param, time_it, prefetch)
+    (MOLE/moe/layer.py:453-454).  `dummy_param` makes autograd record the node even when the input
+    does not require grad (layer.py:80-81); expert gradients are written straight into the
+    parameter stores' gradient buffers, as in the reference."""
+
+    @staticmethod
+    def forward(ctx, dispatched_input, module, dummy_param, time_it=False, prefetch=False, offsets=None, kept_rows=None):
+        ctx.module = module
+        ctx.prefetch = prefetch
+        out = module.MOLECore.forward(dispatched_input, dispatched_input.requires_grad, offsets, kept_rows)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        gx = ctx.module.MOLECore.backward(grad_out)
+        dummy = torch.zeros_like(ctx.module.dummy_param) if ctx.module.dummy_param is not None else None
+        return gx, None, dummy, None, None, None, None

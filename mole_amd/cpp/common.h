@@ -60,4 +60,15 @@ __device__ __forceinline__ float wave_sum(float v) {
 
 static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
+// optional per-kernel timing (see error.cpp); ids are the MOLE_K_* of mole_hip.h
+bool timing_enabled();
+void timing_begin(int id, hipStream_t st);
+void timing_end(hipStream_t st);
+struct ScopedTiming {
+    hipStream_t st;
+    bool on;
+    ScopedTiming(int id, hipStream_t s) : st(s), on(timing_enabled()) { if (on) timing_begin(id, st); }
+    ~ScopedTiming() { if (on) timing_end(st); }
+};
+
 }  // namespace mole

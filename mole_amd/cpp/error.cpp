@@ -1,5 +1,13 @@
-// Error string plumbing and version of the C ABI.
+// Library-wide plumbing of the C ABI: error string, version, and optional per-kernel timing.
+//
+// Timing: when enabled, every instrumented launch is bracketed by two events recorded on the
+// stream the kernel runs on; mole_kernel_timing_read() synchronises those events and returns, per
+// kernel id, the number of launches and their summed duration.  Disabled (the default) it costs
+// one predictable branch per launch.
 #include "common.h"
+
+#include <mutex>
+#include <vector>
 
 namespace mole {
 static thread_local char g_err[512] = "";
@@ -9,7 +17,61 @@ void set_error(const char *fmt, ...) {
     vsnprintf(g_err, sizeof(g_err), fmt, ap);
     va_end(ap);
 }
+
+struct TimedLaunch { int id; hipEvent_t a, b; };
+static bool g_timing = false;
+static std::mutex g_tmu;
+static std::vector<TimedLaunch> g_launches;
+static std::vector<hipEvent_t> g_free_events;
+
+bool timing_enabled() { return g_timing; }
+
+static hipEvent_t get_event() {
+    if (!g_free_events.empty()) {
+        hipEvent_t e = g_free_events.back();
+        g_free_events.pop_back();
+        return e;
+    }
+    hipEvent_t e = nullptr;
+    (void)hipEventCreate(&e);
+    return e;
+}
+
+void timing_begin(int id, hipStream_t st) {
+    std::lock_guard<std::mutex> lk(g_tmu);
+    TimedLaunch t{id, get_event(), get_event()};
+    (void)hipEventRecord(t.a, st);
+    g_launches.push_back(t);
+}
+void timing_end(hipStream_t st) {
+    std::lock_guard<std::mutex> lk(g_tmu);
+    if (!g_launches.empty()) (void)hipEventRecord(g_launches.back().b, st);
+}
 }  // namespace mole
 
+using namespace mole;
+
 extern "C" int mole_version(void) { return 100; }
-extern "C" const char *mole_last_error_string(void) { return mole::g_err; }
+extern "C" const char *mole_last_error_string(void) { return g_err; }
+
+extern "C" int mole_kernel_timing_enable(int on) {
+    std::lock_guard<std::mutex> lk(g_tmu);
+    g_timing = on != 0;
+    return 0;
+}
+
+extern "C" int mole_kernel_timing_read(int n_ids, int *counts, float *ms_total) {
+    MOLE_REQUIRE(n_ids >= 0 && counts && ms_total, "mole_kernel_timing_read: null pointer");
+    std::lock_guard<std::mutex> lk(g_tmu);
+    for (int i = 0; i < n_ids; ++i) { counts[i] = 0; ms_total[i] = 0.f; }
+    for (auto &t : g_launches) {
+        MOLE_HIP(hipEventSynchronize(t.b));
+        float ms = 0.f;
+        MOLE_HIP(hipEventElapsedTime(&ms, t.a, t.b));
+        if (t.id >= 0 && t.id < n_ids) { counts[t.id] += 1; ms_total[t.id] += ms; }
+        g_free_events.push_back(t.a);
+        g_free_events.push_back(t.b);
+    }
+    g_launches.clear();
+    return 0;
+}

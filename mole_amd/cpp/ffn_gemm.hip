@@ -389,8 +389,9 @@ __global__ __launch_bounds__(256) void bias_grad_kernel(const T *__restrict__ in
 }
 
 template <typename T, bool A_KS, bool B_KS, bool WG, int BM, int BN, int EPI>
-static int launch_gemm(GemmArgs g, int tiles, hipStream_t st) {
+static int launch_gemm(GemmArgs g, int tiles, hipStream_t st, int kid) {
     if (tiles <= 0) return 0;
+    ScopedTiming timing(kid, st);
     g.n_blocks = tiles;
     const int grid = (tiles + 7) & ~7;
     const size_t lds = 2 * (size_t)(BM + BN) * 128;
@@ -417,11 +418,11 @@ static int ffn_fwd_t(const void *xd, const int32_t *offsets, const int32_t *kept
     // h = xd . w1^T + b1, a = gelu(h)
     g.A = xd; g.lda = M; g.B = w1; g.ldb = M; g.strideB = (long)F * M; g.N = F; g.K = M;
     g.C = h; g.C2 = a; g.ldc = F; g.bias = b1;
-    if (int rc = launch_gemm<T, false, false, false, TBM, TBN, EPI_BIAS_GELU>(g, m_tiles * ceil_div(F, TBN), st)) return rc;
+    if (int rc = launch_gemm<T, false, false, false, TBM, TBN, EPI_BIAS_GELU>(g, m_tiles * ceil_div(F, TBN), st, MOLE_K_FFN_FWD1)) return rc;
     // out = a . w2 + b2   (w2 [F,M]: K-strided)
     g.A = a; g.lda = F; g.B = w2; g.ldb = M; g.strideB = (long)F * M; g.N = M; g.K = F;
     g.C = out; g.C2 = nullptr; g.ldc = M; g.bias = b2;
-    return launch_gemm<T, false, true, false, TBM, TBN, EPI_BIAS>(g, m_tiles * ceil_div(M, TBN), st);
+    return launch_gemm<T, false, true, false, TBM, TBN, EPI_BIAS>(g, m_tiles * ceil_div(M, TBN), st, MOLE_K_FFN_FWD2);
 }
 
 template <typename T>
@@ -436,24 +437,27 @@ static int ffn_bwd_t(const void *go, const void *xd, const void *h, const void *
     const int wg_tiles = E * ceil_div(F, TBM) * ceil_div(M, TBN);
     // g_w2[e] = a^T . go          (contract over the expert's rows)
     g.A = a; g.lda = F; g.B = go; g.ldb = M; g.M = F; g.N = M; g.C = g_w2; g.ldc = M; g.strideC = (long)F * M;
-    if (int rc = launch_gemm<T, true, true, true, TBM, TBN, EPI_WGRAD>(g, wg_tiles, st)) return rc;
+    if (int rc = launch_gemm<T, true, true, true, TBM, TBN, EPI_WGRAD>(g, wg_tiles, st, MOLE_K_FFN_GW2)) return rc;
     // t = (go . w2^T) * gelu'(h)   (w2 [F,M]: K = M contiguous)
     g.A = go; g.lda = M; g.B = w2; g.ldb = M; g.strideB = (long)F * M; g.N = F; g.K = M; g.C = t; g.ldc = F; g.H = h;
-    if (int rc = launch_gemm<T, false, false, false, TBM, TBN, EPI_DGELU>(g, m_tiles * ceil_div(F, TBN), st)) return rc;
+    if (int rc = launch_gemm<T, false, false, false, TBM, TBN, EPI_DGELU>(g, m_tiles * ceil_div(F, TBN), st, MOLE_K_FFN_DA)) return rc;
     // g_b2 = sum go ; g_b1 = sum t
+    {
+    ScopedTiming timing(MOLE_K_FFN_GB, st);
     hipLaunchKernelGGL(bias_grad_kernel<T>, dim3(ceil_div(M, 64), E), dim3(256), 0, st, (const T *)go, offsets, kept, M,
                        accumulate, (T *)g_b2);
     MOLE_LAUNCH_CHECK();
     hipLaunchKernelGGL(bias_grad_kernel<T>, dim3(ceil_div(F, 64), E), dim3(256), 0, st, (const T *)t, offsets, kept, F,
                        accumulate, (T *)g_b1);
     MOLE_LAUNCH_CHECK();
+    }
     // g_w1[e] = t^T . xd
     g.A = t; g.lda = F; g.B = xd; g.ldb = M; g.M = F; g.N = M; g.C = g_w1; g.ldc = M; g.strideC = (long)F * M;
-    if (int rc = launch_gemm<T, true, true, true, TBM, TBN, EPI_WGRAD>(g, wg_tiles, st)) return rc;
+    if (int rc = launch_gemm<T, true, true, true, TBM, TBN, EPI_WGRAD>(g, wg_tiles, st, MOLE_K_FFN_GW1)) return rc;
     // gx = t . w1                  (w1 [F,M]: K = F strided)
     if (gx != nullptr) {
         g.A = t; g.lda = F; g.B = w1; g.ldb = M; g.strideB = (long)F * M; g.N = M; g.K = F; g.C = gx; g.ldc = M;
-        if (int rc = launch_gemm<T, false, true, false, TBM, TBN, EPI_STORE>(g, m_tiles * ceil_div(M, TBN), st)) return rc;
+        if (int rc = launch_gemm<T, false, true, false, TBM, TBN, EPI_STORE>(g, m_tiles * ceil_div(M, TBN), st, MOLE_K_FFN_GX)) return rc;
     }
     return 0;
 }
@@ -510,6 +514,6 @@ extern "C" int mole_gemm_nt(const void *a, const void *b, int dtype, int rows, i
     g.single_rows = rows; g.E = 1;
     g.A = a; g.lda = K; g.B = b; g.ldb = K; g.N = N; g.K = K; g.C = c; g.ldc = N;
     const int tiles = ceil_div(rows, TBM) * ceil_div(N, TBN);
-    if (dtype == MOLE_BF16) return launch_gemm<bf16_t, false, false, false, TBM, TBN, EPI_F32>(g, tiles, (hipStream_t)stream);
-    return launch_gemm<float, false, false, false, TBM, TBN, EPI_F32>(g, tiles, (hipStream_t)stream);
+    if (dtype == MOLE_BF16) return launch_gemm<bf16_t, false, false, false, TBM, TBN, EPI_F32>(g, tiles, (hipStream_t)stream, MOLE_K_GEMM_NT);
+    return launch_gemm<float, false, false, false, TBM, TBN, EPI_F32>(g, tiles, (hipStream_t)stream, MOLE_K_GEMM_NT);
 }

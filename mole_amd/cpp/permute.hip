@@ -228,6 +228,7 @@ extern "C" int mole_dispatch_fwd(const void *x, int dtype, const int32_t *row, i
     if (S == 0) return 0;
     MOLE_REQUIRE(x && row && xd && aligned16(x) && aligned16(xd), "mole_dispatch_fwd: null or misaligned pointer");
     const dim3 grid(ceil_div(S, PM_THREADS / WAVE));
+    ScopedTiming timing(MOLE_K_DISPATCH_FWD, (hipStream_t)stream);
     if (dtype == MOLE_BF16)
         hipLaunchKernelGGL(dispatch_fwd_kernel<bf16_t>, grid, dim3(PM_THREADS), 0, (hipStream_t)stream,
                            (const bf16_t *)x, row, S, M, k, (bf16_t *)xd);
@@ -246,6 +247,7 @@ extern "C" int mole_dispatch_bwd(const void *dxd, int dtype, const int32_t *row,
     MOLE_REQUIRE(dlogits == nullptr || (wg != nullptr && E >= 1 && aligned16(wg) && M % 4 == 0),
                  "mole_dispatch_bwd: dlogits given without a valid wg/E");
     const dim3 grid(ceil_div(S, PM_THREADS / WAVE));
+    ScopedTiming timing(MOLE_K_DISPATCH_BWD, (hipStream_t)stream);
     if (dtype == MOLE_BF16)
         hipLaunchKernelGGL(dispatch_bwd_kernel<bf16_t>, grid, dim3(PM_THREADS), 0, (hipStream_t)stream,
                            (const bf16_t *)dxd, row, S, M, k, dlogits, wg, E, (bf16_t *)dx);
@@ -262,6 +264,7 @@ extern "C" int mole_combine_fwd(const void *o, int dtype, const int32_t *row, co
     if (S == 0) return 0;
     MOLE_REQUIRE(o && row && gates && y && aligned16(o) && aligned16(y), "mole_combine_fwd: null or misaligned pointer");
     const dim3 grid(ceil_div(S, PM_THREADS / WAVE));
+    ScopedTiming timing(MOLE_K_COMBINE_FWD, (hipStream_t)stream);
     if (dtype == MOLE_BF16)
         hipLaunchKernelGGL(combine_fwd_kernel<bf16_t>, grid, dim3(PM_THREADS), 0, (hipStream_t)stream,
                            (const bf16_t *)o, row, gates, S, M, k, (bf16_t *)y);
@@ -279,6 +282,7 @@ extern "C" int mole_combine_bwd(const void *dy, const void *o, int dtype, const 
     MOLE_REQUIRE(dy && o && row && gates && d_o && dgates && aligned16(dy) && aligned16(o) && aligned16(d_o),
                  "mole_combine_bwd: null or misaligned pointer");
     const dim3 grid(ceil_div(S, PM_THREADS / WAVE));
+    ScopedTiming timing(MOLE_K_COMBINE_BWD, (hipStream_t)stream);
     if (dtype == MOLE_BF16)
         hipLaunchKernelGGL(combine_bwd_kernel<bf16_t>, grid, dim3(PM_THREADS), 0, (hipStream_t)stream,
                            (const bf16_t *)dy, (const bf16_t *)o, row, gates, S, M, k, (bf16_t *)d_o, dgates);

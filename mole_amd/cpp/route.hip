@@ -301,6 +301,7 @@ extern "C" int mole_route(const float *scores, int S, int E, int k, float capaci
         return MOLE_E_WORKSPACE;
     }
     hipStream_t st = (hipStream_t)stream;
+    ScopedTiming timing(MOLE_K_ROUTE, st);
     const int nb = ceil_div(S > 0 ? S : 1, RT_TOKENS);
     char *ws = (char *)workspace;
     int32_t *hist = (int32_t *)ws;

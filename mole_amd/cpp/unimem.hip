@@ -181,7 +181,7 @@ extern "C" int mole_unimem_fetch(void *handle, const void *const host_src[4], in
                                  int prefetched, void **slot_ptrs_out) {
     UM(handle);
     const int slot0 = view_base + u->virtual_offset;
-    MOLE_REQUIRE(n > 0 && view_base >= 0 && base >= 0 && prefetched >= 0 && prefetched <= n && host_src && slot_ptrs_out,
+    MOLE_REQUIRE(n > 0 && slot0 >= 0 && base >= 0 && prefetched >= 0 && prefetched <= n && host_src && slot_ptrs_out,
                  "mole_unimem_fetch: bad arguments (view_base=%d base=%d n=%d prefetched=%d)", view_base, base, n, prefetched);
     if (slot0 + n > u->pool_size) {
         set_error("mole_unimem_fetch: slots %d..%d exceed the pool of %d", slot0, slot0 + n, u->pool_size);

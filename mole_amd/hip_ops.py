@@ -152,6 +152,22 @@ def zero_pad_rows(buf: torch.Tensor, kept_rows: torch.Tensor, offsets: torch.Ten
             "mole_zero_pad_rows")
 
 
+def ffn_fwd_into(xd, offsets, kept_rows, E, max_rows, M, F, w1, b1, w2, b2, h, a, out) -> None:
+    """mole_ffn_fwd on caller-provided buffers.  Weights may be tensors or raw device addresses
+    (slot-pool pointers); offsets/kept_rows may be views starting at the first expert of a chunk."""
+    L.check(L.lib().mole_ffn_fwd(L.ptr(xd), L.dtype_code(xd.dtype), L.ptr(offsets), L.ptr(kept_rows), int(E), int(max_rows),
+                                 int(M), int(F), L.ptr(w1), L.ptr(b1), L.ptr(w2), L.ptr(b2), L.ptr(h), L.ptr(a), L.ptr(out),
+                                 L.stream()), "mole_ffn_fwd")
+
+
+def ffn_bwd_into(go, xd, h, a, offsets, kept_rows, E, max_rows, M, F, w1, w2, t, g_w1, g_b1, g_w2, g_b2, gx,
+                 accumulate: bool, gelu_bwd: int) -> None:
+    L.check(L.lib().mole_ffn_bwd(L.ptr(go), L.ptr(xd), L.ptr(h), L.ptr(a), L.dtype_code(xd.dtype), L.ptr(offsets),
+                                 L.ptr(kept_rows), int(E), int(max_rows), int(M), int(F), L.ptr(w1), L.ptr(w2), L.ptr(t),
+                                 L.ptr(g_w1), L.ptr(g_b1), L.ptr(g_w2), L.ptr(g_b2), L.ptr(gx), int(accumulate),
+                                 int(gelu_bwd), L.stream()), "mole_ffn_bwd")
+
+
 def ffn_fwd(xd, offsets, kept_rows, w1, b1, w2, b2, max_rows: Optional[int] = None):
     """Returns (out [rows,M], h [rows,F], a [rows,F])."""
     for t in (xd, offsets, kept_rows, w1, b1, w2, b2):
@@ -162,9 +178,7 @@ def ffn_fwd(xd, offsets, kept_rows, w1, b1, w2, b2, max_rows: Optional[int] = No
     h = torch.empty(rows, F, dtype=xd.dtype, device=xd.device)
     a = torch.empty(rows, F, dtype=xd.dtype, device=xd.device)
     out = torch.empty(rows, M, dtype=xd.dtype, device=xd.device)
-    L.check(L.lib().mole_ffn_fwd(L.ptr(xd), L.dtype_code(xd.dtype), L.ptr(offsets), L.ptr(kept_rows), E, max_rows, M, F,
-                                 L.ptr(w1), L.ptr(b1), L.ptr(w2), L.ptr(b2), L.ptr(h), L.ptr(a), L.ptr(out), L.stream()),
-            "mole_ffn_fwd")
+    ffn_fwd_into(xd, offsets, kept_rows, E, max_rows, M, F, w1, b1, w2, b2, h, a, out)
     return out, h, a
 
 
@@ -178,8 +192,6 @@ def ffn_bwd(go, xd, h, a, offsets, kept_rows, w1, w2, g_w1, g_b1, g_w2, g_b2, ne
     max_rows = rows if max_rows is None else max_rows
     t = torch.empty(rows, F, dtype=xd.dtype, device=xd.device)
     gx = torch.empty(rows, M, dtype=xd.dtype, device=xd.device) if need_gx else None
-    L.check(L.lib().mole_ffn_bwd(L.ptr(go), L.ptr(xd), L.ptr(h), L.ptr(a), L.dtype_code(xd.dtype), L.ptr(offsets),
-                                 L.ptr(kept_rows), E, max_rows, M, F, L.ptr(w1), L.ptr(w2), L.ptr(t), L.ptr(g_w1),
-                                 L.ptr(g_b1), L.ptr(g_w2), L.ptr(g_b2), L.ptr(gx), int(accumulate), int(gelu_bwd),
-                                 L.stream()), "mole_ffn_bwd")
+    ffn_bwd_into(go, xd, h, a, offsets, kept_rows, E, max_rows, M, F, w1, w2, t, g_w1, g_b1, g_w2, g_b2, gx, accumulate,
+                 gelu_bwd)
     return gx

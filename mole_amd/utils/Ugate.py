@@ -1,0 +1,46 @@
+"""Gate of the MoE layer: Linear without bias, softmax over experts.
+
+Mirror of MOLE/utils/Ugate.py:5-14 (same class name, same `linear` attribute).  The logits come from
+the MFMA NT GEMM of the C ABI (mole_gemm_nt), the softmax from mole_softmax_fwd; the backward is the
+textbook softmax/linear backward on device tensors.  `logit_bias` ([E], optional, not trained) is
+added to the logits before the softmax - the reference gate has none.
+"""
+import torch
+
+from .. import hip_ops as H
+
+
+class _GateFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, weight, logit_bias):
+        scores = gate_scores(x, weight, logit_bias)
+        ctx.save_for_backward(x, weight, scores)
+        return scores
+
+    @staticmethod
+    def backward(ctx, dscores):
+        x, weight, scores = ctx.saved_tensors
+        dlogits = scores * (dscores - (dscores * scores).sum(dim=-1, keepdim=True))
+        dx = (dlogits @ weight).to(x.dtype) if ctx.needs_input_grad[0] else None
+        dw = (dlogits.t().to(x.dtype) @ x).to(weight.dtype) if ctx.needs_input_grad[1] else None
+        return dx, dw, None
+
+
+def gate_scores(x: torch.Tensor, weight: torch.Tensor, logit_bias=None) -> torch.Tensor:
+    """softmax(x @ weight.T + logit_bias) in fp32; x [S,M] fp32 or bf16, weight [E,M] fp32."""
+    w = weight.detach()
+    if w.dtype != x.dtype:
+        w = w.to(x.dtype)
+    logits = H.gemm_nt(x.detach().contiguous(), w.contiguous())
+    return H.softmax_fwd(logits, logit_bias)
+
+
+class MOLETopk(torch.nn.Module):
+    def __init__(self, model_dim, total_experts) -> None:
+        super().__init__()
+        self.total_experts = total_experts
+        self.linear = torch.nn.Linear(model_dim, total_experts, bias=False)
+        self.logit_bias = None
+
+    def forward(self, input):
+        return _GateFn.apply(input, self.linear.weight, self.logit_bias)
