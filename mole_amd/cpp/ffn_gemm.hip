@@ -18,37 +18,11 @@
 // offsets/kept_rows on the device; a block finds its (expert, m-tile) with a wave-parallel prefix
 // search, so no host synchronisation is needed to launch.  Weight gradients contract over the
 // expert's rows instead (K extent ragged).
-#include "common.h"
+#include "gemm.h"
 
-#include <math.h>
+#include <stdlib.h>
 
 namespace mole {
-
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-
-// ---------------------------------------------------------------------------------------------
-// activation math (fp32)
-// ---------------------------------------------------------------------------------------------
-__device__ __forceinline__ float gelu_erf(float x) { return 0.5f * x * (1.0f + erff(x * 0.70710678118654752f)); }
-
-// derivative of the tanh-approximate GELU, term by term as MOLE/cpp/gelu.cu:3-14
-__device__ __forceinline__ float d_gelu_tanh(float x) {
-    const float sqrt_param = 0.79788456080286535587989211986876f;
-    const float mul_param = 0.044715f;
-    const float x2mul = x * x * mul_param;
-    const float tan_h = tanhf(sqrt_param * (x + x * x2mul));
-    const float dg1 = 0.5f * (1.0f + tan_h);
-    const float dg2 = x * 0.5f * sqrt_param * (1.0f - tan_h * tan_h);
-    const float dg3 = dg2 * 3.0f * x2mul;
-    return dg1 + dg2 + dg3;
-}
-// derivative of the erf GELU (at::gelu_backward): Phi(x) + x*phi(x)
-__device__ __forceinline__ float d_gelu_exact(float x) {
-    const float cdf = 0.5f * (1.0f + erff(x * 0.70710678118654752f));
-    const float pdf = expf(-0.5f * x * x) * 0.39894228040143267794f;
-    return cdf + x * pdf;
-}
 
 // ---------------------------------------------------------------------------------------------
 // tile geometry shared by both element types: a row of a staged tile is 128 bytes = 8 chunks
@@ -192,28 +166,6 @@ __device__ __forceinline__ void mma_step(const char *ldsA, const char *ldsB, int
     }
 }
 
-enum { EPI_STORE = 0, EPI_BIAS = 1, EPI_BIAS_GELU = 2, EPI_DGELU = 3, EPI_WGRAD = 4, EPI_F32 = 5 };
-
-struct GemmArgs {
-    const void *A, *B;      // operands (see A_KS / B_KS for their layout)
-    void *C, *C2;           // outputs; C2 = gelu(h) for EPI_BIAS_GELU
-    const void *bias;       // [E][N] for EPI_BIAS*, else unused
-    const void *H;          // [rows][N] pre-activation for EPI_DGELU
-    const int32_t *offsets; // [E] first row of every expert (NULL: one group starting at row 0)
-    const int32_t *kept;    // [E] rows of every expert (NULL: single_rows)
-    int single_rows;
-    int E;
-    int M;                  // output rows per expert for weight gradients (F), unused for row-ragged
-    int N, K;               // N output columns; K contraction length (row-ragged products)
-    long lda, ldb, ldc;
-    long strideB;           // elements between experts in B (row-ragged) -- weights
-    long strideC;           // elements between experts in C (weight gradients)
-    int m_tiles_bound;      // upper bound of the number of m-tiles over all experts (row-ragged)
-    int accumulate;         // EPI_WGRAD: add into C
-    int gelu_bwd;           // EPI_DGELU: MOLE_GELU_BWD_*
-    int n_blocks;           // real number of tiles in the launch (grid is rounded up to 8)
-};
-
 // Row-ragged: C[rows_e, N] = A[rows_e, K] . B_e   (A K-contiguous; B_e [N,K] or, B_KS, [K,N])
 // Weight gradient (WG): C_e[M, N] = sum_{r in rows_e} A[r, M]^T . B[r, N]  (both K-strided)
 template <typename T, bool A_KS, bool B_KS, bool WG, int BM, int BN, int EPI>
@@ -223,22 +175,33 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kernel(const GemmArgs g) {
     extern __shared__ __align__(16) char smem[];
     constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
 
-    // ---- which tile am I?  (blocks are dealt round-robin to the 8 XCDs: give each XCD a
-    //      contiguous range of tiles so that neighbours share operands in its L2)
-    const int nblk = gridDim.x;
-    const int t = (blockIdx.x & 7) * (nblk >> 3) + (blockIdx.x >> 3);
-    if (t >= g.n_blocks) return;
+    // ---- which tile am I?  Blocks are dealt round-robin to the 8 XCDs (block b runs on XCD b mod 8):
+    //      give each XCD a contiguous range of the REAL tiles, so that neighbours share operands in
+    //      its L2 and every XCD gets the same share.  For row-ragged products the number of real
+    //      tiles is only known here (the grid is sized for the worst case), hence the device-side sum.
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n_tiles = (g.N + BN - 1) / BN;
-
     int e, mt, nt, m_ext, k_ext;
     long row0;  // first row of the expert
     if constexpr (!WG) {
+        int total_m_tiles;
+        if (g.offsets == nullptr) {
+            total_m_tiles = (g.single_rows + BM - 1) / BM;
+        } else {
+            int part = 0;
+            for (int ee = lane; ee < g.E; ee += WAVE) part += (g.kept[ee] + BM - 1) / BM;
+            for (int d = WAVE / 2; d >= 1; d >>= 1) part += __shfl_xor(part, d, WAVE);
+            total_m_tiles = part;
+        }
+        const int total = total_m_tiles * n_tiles;
+        const int per_xcd = (total + 7) >> 3;
+        const int slot = blockIdx.x >> 3;
+        const int t = (blockIdx.x & 7) * per_xcd + slot;
+        if (slot >= per_xcd || t >= total) return;
         const int mtg = t / n_tiles;
         nt = t % n_tiles;
         if (g.offsets == nullptr) {
             e = 0; mt = mtg; m_ext = g.single_rows; row0 = 0;
-            if (mt * BM >= m_ext) return;
         } else {
             int run = 0, found = -1, fmt = 0;
             for (int base = 0; base < g.E && found < 0; base += WAVE) {
@@ -264,6 +227,9 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kernel(const GemmArgs g) {
         }
         k_ext = g.K;
     } else {
+        const int nblk = gridDim.x;
+        const int t = (blockIdx.x & 7) * (nblk >> 3) + (blockIdx.x >> 3);
+        if (t >= g.n_blocks) return;
         const int m_tiles = (g.M + BM - 1) / BM;
         e = t / (m_tiles * n_tiles);
         const int rem = t % (m_tiles * n_tiles);
@@ -365,26 +331,63 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kernel(const GemmArgs g) {
 }
 
 // column sums over an expert's rows: out[e, n] (+)= sum_{r in rows_e} in[r, n]
-// (torch::sum_out(g_b2, go, {1}) / (g_b1, t, {1}), MOLE/cpp/core.cpp:399, 408)
+// (torch::sum_out(g_b2, go, {1}) / (g_b1, t, {1}), MOLE/cpp/core.cpp:399, 408).
+// A block of 16 waves owns 64*VEC columns of one expert; wave w sums rows w, w+16, ... with 8-byte
+// loads per lane (4 rows in flight), then the 16 partial rows are folded through LDS in a fixed order.
+constexpr int BG_WAVES = 16;
 template <typename T>
-__global__ __launch_bounds__(256) void bias_grad_kernel(const T *__restrict__ in, const int32_t *__restrict__ offsets,
-                                                        const int32_t *__restrict__ kept, int N, int accumulate,
-                                                        T *__restrict__ out) {
-    __shared__ float s_part[4][64];
+__global__ __launch_bounds__(BG_WAVES * 64) void bias_grad_kernel(const T *__restrict__ in,
+                                                                   const int32_t *__restrict__ offsets,
+                                                                   const int32_t *__restrict__ kept, int N,
+                                                                   int accumulate, T *__restrict__ out) {
+    constexpr int VEC = 8 / sizeof(T);   // elements per 8-byte load: 4 bf16 or 2 fp32
+    __shared__ float s_part[BG_WAVES][64 * VEC];
     const int e = blockIdx.y;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    const int n = blockIdx.x * 64 + lane;
+    const int n = (blockIdx.x * 64 + lane) * VEC;
     const long r0 = offsets[e];
     const int rows = kept[e];
-    float acc = 0.f;
-    if (n < N)
-        for (int r = w; r < rows; r += 4) acc += to_f32(in[(r0 + r) * (long)N + n]);
-    s_part[w][lane] = acc;
+    float acc[VEC];
+#pragma unroll
+    for (int q = 0; q < VEC; ++q) acc[q] = 0.f;
+    if (n < N) {
+        const T *p = in + r0 * (long)N + n;
+        int r = w;
+        for (; r + 3 * BG_WAVES < rows; r += 4 * BG_WAVES) {
+            uint2 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const uint2 *>(p + (long)(r + u * BG_WAVES) * N);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if constexpr (sizeof(T) == 2) {
+                    acc[0] += __uint_as_float(v[u].x << 16); acc[1] += __uint_as_float(v[u].x & 0xffff0000u);
+                    acc[2] += __uint_as_float(v[u].y << 16); acc[3] += __uint_as_float(v[u].y & 0xffff0000u);
+                } else {
+                    acc[0] += __uint_as_float(v[u].x); acc[1] += __uint_as_float(v[u].y);
+                }
+            }
+        }
+        for (; r < rows; r += BG_WAVES) {
+            const uint2 v = *reinterpret_cast<const uint2 *>(p + (long)r * N);
+            if constexpr (sizeof(T) == 2) {
+                acc[0] += __uint_as_float(v.x << 16); acc[1] += __uint_as_float(v.x & 0xffff0000u);
+                acc[2] += __uint_as_float(v.y << 16); acc[3] += __uint_as_float(v.y & 0xffff0000u);
+            } else {
+                acc[0] += __uint_as_float(v.x); acc[1] += __uint_as_float(v.y);
+            }
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < VEC; ++q) s_part[w][lane * VEC + q] = acc[q];
     __syncthreads();
-    if (w == 0 && n < N) {
-        float v = (s_part[0][lane] + s_part[1][lane]) + (s_part[2][lane] + s_part[3][lane]);
-        if (accumulate) v += to_f32(out[(long)e * N + n]);
-        out[(long)e * N + n] = from_f32<T>(v);
+    for (int c = threadIdx.x; c < 64 * VEC; c += BG_WAVES * 64) {
+        const int nn = blockIdx.x * 64 * VEC + c;
+        if (nn >= N) continue;
+        float v = 0.f;
+#pragma unroll
+        for (int ww = 0; ww < BG_WAVES; ++ww) v += s_part[ww][c];
+        if (accumulate) v += to_f32(out[(long)e * N + nn]);
+        out[(long)e * N + nn] = from_f32<T>(v);
     }
 }
 
@@ -406,7 +409,29 @@ static int launch_gemm(GemmArgs g, int tiles, hipStream_t st, int kid) {
     return 0;
 }
 
-constexpr int TBM = 128, TBN = 128;  // tile of every product
+constexpr int TBM = 128, TBN = 128;  // tile of the generic kernel
+
+// MOLE_GEMM=generic in the environment forces the generic kernel (tests compare both paths)
+static bool fast_path_enabled() {
+    static const bool on = [] {
+        const char *v = getenv("MOLE_GEMM");
+        return !(v && v[0] == 'g');
+    }();
+    return on;
+}
+
+// bf16 products go to the 256x256 direct-to-LDS kernel when their shape allows it
+template <typename T, bool A_KS, bool B_KS, bool WG, int EPI>
+static int run_gemm(const GemmArgs &g, int max_rows, int tiles_generic, hipStream_t st, int kid) {
+    if constexpr (sizeof(T) == 2) {
+        if (fast_path_enabled()) {
+            const int rc = launch_gemm256(g, A_KS, B_KS, WG, EPI, max_rows, st, kid);
+            if (rc != -100) return rc;
+        }
+    }
+    return launch_gemm<T, A_KS, B_KS, WG, TBM, TBN, EPI>(g, tiles_generic, st, kid);
+}
+
 
 template <typename T>
 static int ffn_fwd_t(const void *xd, const int32_t *offsets, const int32_t *kept, int E, int max_rows, int M, int F,
@@ -418,11 +443,11 @@ static int ffn_fwd_t(const void *xd, const int32_t *offsets, const int32_t *kept
     // h = xd . w1^T + b1, a = gelu(h)
     g.A = xd; g.lda = M; g.B = w1; g.ldb = M; g.strideB = (long)F * M; g.N = F; g.K = M;
     g.C = h; g.C2 = a; g.ldc = F; g.bias = b1;
-    if (int rc = launch_gemm<T, false, false, false, TBM, TBN, EPI_BIAS_GELU>(g, m_tiles * ceil_div(F, TBN), st, MOLE_K_FFN_FWD1)) return rc;
+    if (int rc = run_gemm<T, false, false, false, EPI_BIAS_GELU>(g, max_rows, m_tiles * ceil_div(F, TBN), st, MOLE_K_FFN_FWD1)) return rc;
     // out = a . w2 + b2   (w2 [F,M]: K-strided)
     g.A = a; g.lda = F; g.B = w2; g.ldb = M; g.strideB = (long)F * M; g.N = M; g.K = F;
     g.C = out; g.C2 = nullptr; g.ldc = M; g.bias = b2;
-    return launch_gemm<T, false, true, false, TBM, TBN, EPI_BIAS>(g, m_tiles * ceil_div(M, TBN), st, MOLE_K_FFN_FWD2);
+    return run_gemm<T, false, true, false, EPI_BIAS>(g, max_rows, m_tiles * ceil_div(M, TBN), st, MOLE_K_FFN_FWD2);
 }
 
 template <typename T>
@@ -437,27 +462,27 @@ static int ffn_bwd_t(const void *go, const void *xd, const void *h, const void *
     const int wg_tiles = E * ceil_div(F, TBM) * ceil_div(M, TBN);
     // g_w2[e] = a^T . go          (contract over the expert's rows)
     g.A = a; g.lda = F; g.B = go; g.ldb = M; g.M = F; g.N = M; g.C = g_w2; g.ldc = M; g.strideC = (long)F * M;
-    if (int rc = launch_gemm<T, true, true, true, TBM, TBN, EPI_WGRAD>(g, wg_tiles, st, MOLE_K_FFN_GW2)) return rc;
+    if (int rc = run_gemm<T, true, true, true, EPI_WGRAD>(g, max_rows, wg_tiles, st, MOLE_K_FFN_GW2)) return rc;
     // t = (go . w2^T) * gelu'(h)   (w2 [F,M]: K = M contiguous)
     g.A = go; g.lda = M; g.B = w2; g.ldb = M; g.strideB = (long)F * M; g.N = F; g.K = M; g.C = t; g.ldc = F; g.H = h;
-    if (int rc = launch_gemm<T, false, false, false, TBM, TBN, EPI_DGELU>(g, m_tiles * ceil_div(F, TBN), st, MOLE_K_FFN_DA)) return rc;
+    if (int rc = run_gemm<T, false, false, false, EPI_DGELU>(g, max_rows, m_tiles * ceil_div(F, TBN), st, MOLE_K_FFN_DA)) return rc;
     // g_b2 = sum go ; g_b1 = sum t
     {
     ScopedTiming timing(MOLE_K_FFN_GB, st);
-    hipLaunchKernelGGL(bias_grad_kernel<T>, dim3(ceil_div(M, 64), E), dim3(256), 0, st, (const T *)go, offsets, kept, M,
+    hipLaunchKernelGGL(bias_grad_kernel<T>, dim3(ceil_div(M, 512 / (int)sizeof(T)), E), dim3(BG_WAVES * 64), 0, st, (const T *)go, offsets, kept, M,
                        accumulate, (T *)g_b2);
     MOLE_LAUNCH_CHECK();
-    hipLaunchKernelGGL(bias_grad_kernel<T>, dim3(ceil_div(F, 64), E), dim3(256), 0, st, (const T *)t, offsets, kept, F,
+    hipLaunchKernelGGL(bias_grad_kernel<T>, dim3(ceil_div(F, 512 / (int)sizeof(T)), E), dim3(BG_WAVES * 64), 0, st, (const T *)t, offsets, kept, F,
                        accumulate, (T *)g_b1);
     MOLE_LAUNCH_CHECK();
     }
     // g_w1[e] = t^T . xd
     g.A = t; g.lda = F; g.B = xd; g.ldb = M; g.M = F; g.N = M; g.C = g_w1; g.ldc = M; g.strideC = (long)F * M;
-    if (int rc = launch_gemm<T, true, true, true, TBM, TBN, EPI_WGRAD>(g, wg_tiles, st, MOLE_K_FFN_GW1)) return rc;
+    if (int rc = run_gemm<T, true, true, true, EPI_WGRAD>(g, max_rows, wg_tiles, st, MOLE_K_FFN_GW1)) return rc;
     // gx = t . w1                  (w1 [F,M]: K = F strided)
     if (gx != nullptr) {
         g.A = t; g.lda = F; g.B = w1; g.ldb = M; g.strideB = (long)F * M; g.N = M; g.K = F; g.C = gx; g.ldc = M;
-        if (int rc = launch_gemm<T, false, true, false, TBM, TBN, EPI_STORE>(g, m_tiles * ceil_div(M, TBN), st, MOLE_K_FFN_GX)) return rc;
+        if (int rc = run_gemm<T, false, true, false, EPI_STORE>(g, max_rows, m_tiles * ceil_div(M, TBN), st, MOLE_K_FFN_GX)) return rc;
     }
     return 0;
 }
@@ -514,6 +539,6 @@ extern "C" int mole_gemm_nt(const void *a, const void *b, int dtype, int rows, i
     g.single_rows = rows; g.E = 1;
     g.A = a; g.lda = K; g.B = b; g.ldb = K; g.N = N; g.K = K; g.C = c; g.ldc = N;
     const int tiles = ceil_div(rows, TBM) * ceil_div(N, TBN);
-    if (dtype == MOLE_BF16) return launch_gemm<bf16_t, false, false, false, TBM, TBN, EPI_F32>(g, tiles, (hipStream_t)stream, MOLE_K_GEMM_NT);
+    if (dtype == MOLE_BF16) return run_gemm<bf16_t, false, false, false, EPI_F32>(g, rows, tiles, (hipStream_t)stream, MOLE_K_GEMM_NT);
     return launch_gemm<float, false, false, false, TBM, TBN, EPI_F32>(g, tiles, (hipStream_t)stream, MOLE_K_GEMM_NT);
 }

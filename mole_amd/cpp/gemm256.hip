@@ -1,0 +1,488 @@
+// bf16 grouped GEMM on 256 x 256 tiles for gfx950: the fast path of the six expert-FFN products.
+//
+// A block of 4 waves owns a 256 (m) x 256 (n) output tile; every wave covers all 256 m and 64 n
+// (8 x 2 MFMA 32x32x16 blocks, 256 fp32 accumulators in AGPRs).  Operand tiles go from HBM/L2
+// straight into LDS (global_load_lds_dwordx4, no staging registers) through a ring of four stages of
+// 32 of K, so that three stages of loads are in flight while one is consumed: with a single stage
+// of look-ahead the loop ran at the memory latency, not at the MFMA rate.  One barrier per stage.
+// Each 16-byte piece is placed at a swizzled LDS position by choosing which global address the lane
+// that owns the slot fetches:
+//   * K-contiguous operand  -> LDS [row][4 x 16 B]; fragments read with ds_read_b128
+//   * K-strided operand     -> LDS [k][256 x 2 B] as it lies in HBM; fragments read with
+//                              ds_read_b64_tr_b16, the LDS transpose read
+// The MFMA "A" slot is fed with the n-side operand and the "B" slot with the m-side operand, so the
+// four consecutive accumulator rows a lane holds are four consecutive n: the epilogue stores (and
+// the bias / pre-activation loads) are 8 bytes per lane.
+// A ragged m-tile runs only the 32-row blocks it has rows for (2, 4 or 8 of 8).
+#include "gemm.h"
+
+namespace mole {
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+
+constexpr int Q_BM = 256, Q_BN = 256, Q_BK = 32;
+constexpr int Q_OPERAND = 16 * 1024;        // one operand tile of one stage
+constexpr int Q_STAGE = 2 * Q_OPERAND;
+constexpr int Q_NSTAGE = 4;                 // ring of LDS stages: one consumed, up to three in flight
+constexpr int Q_THREADS = 256;
+constexpr int Q_LOADS_PER_STAGE = 8;        // asynchronous loads a wave issues per stage
+
+// s_waitcnt immediate that waits for vmcnt <= n and nothing else (gfx9 encoding: vmcnt in bits 3:0
+// and 15:14, expcnt 6:4, lgkmcnt 11:8)
+constexpr int waitcnt_vm(int n) { return (n & 0xf) | ((n >> 4) << 14) | 0x0070 | 0x0f00; }
+
+// 16 bytes per lane from global memory straight into LDS: lane i of the wave writes LDS bytes
+// [lds_off + 16 i, +16).  Issued as inline assembly on purpose: the compiler makes every LDS read
+// that follows a global_load_lds it knows about wait for vmcnt(0), which would serialise the ring of
+// stages; here the K loop does its own vmcnt accounting (s_waitcnt before each barrier).  M0 is
+// reserved by the compiler and nothing else in these kernels uses it.
+__device__ __forceinline__ void dma16(const void *gptr, uint32_t lds_off) {
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_off) : "memory");
+}
+__device__ __forceinline__ uint32_t lds_offset_of(const char *p) {
+    return (uint32_t)(size_t)(__attribute__((address_space(3))) const char *)p;
+}
+
+// ---- cheap, accurate-enough activation math for a bf16 result --------------------------------
+// erf by Abramowitz-Stegun 7.1.26 (|error| < 1.5e-7) on the hardware reciprocal and exp2
+__device__ __forceinline__ float fast_erf_abs(float z) {  // erf(z) for z >= 0
+    const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, z, 1.0f));
+    float p = fmaf(1.061405429f, t, -1.453152027f);
+    p = fmaf(p, t, 1.421413741f);
+    p = fmaf(p, t, -0.284496736f);
+    p = fmaf(p, t, 0.254829592f);
+    p *= t;
+    const float e = __builtin_amdgcn_exp2f(-1.4426950408889634f * z * z);
+    return fmaf(-p, e, 1.0f);
+}
+__device__ __forceinline__ float fast_gelu_erf(float x) {
+    const float er = fast_erf_abs(fabsf(x) * 0.70710678118654752f);
+    return 0.5f * x * (1.0f + copysignf(er, x));
+}
+__device__ __forceinline__ float fast_tanh(float u) {  // 1 - 2/(1+e^{2u}), saturates cleanly
+    const float e = __builtin_amdgcn_exp2f(2.0f * 1.4426950408889634f * u);
+    return 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
+}
+__device__ __forceinline__ float fast_d_gelu_tanh(float x) {  // MOLE/cpp/gelu.cu:3-14
+    const float sqrt_param = 0.79788456080286535587989211986876f;
+    const float x2mul = x * x * 0.044715f;
+    const float th = fast_tanh(sqrt_param * (x + x * x2mul));
+    const float dg1 = 0.5f * (1.0f + th);
+    const float dg2 = x * 0.5f * sqrt_param * (1.0f - th * th);
+    return dg1 + dg2 + dg2 * 3.0f * x2mul;
+}
+__device__ __forceinline__ float fast_d_gelu_exact(float x) {
+    const float er = fast_erf_abs(fabsf(x) * 0.70710678118654752f);
+    const float cdf = 0.5f * (1.0f + copysignf(er, x));
+    const float pdf = __builtin_amdgcn_exp2f(-0.5f * 1.4426950408889634f * x * x) * 0.39894228040143267794f;
+    return cdf + x * pdf;
+}
+
+// ---- operand tiles in LDS -------------------------------------------------------------------------
+// A stage holds 32 of K.  Every lane always issues its load (no divergent branches in the K loop):
+// rows past the operand's extent are clamped to the last valid row / 16-byte piece.  What lands in
+// LDS for them is real, finite data that only contributes to output rows or columns the epilogue
+// does not store - except along a ragged contraction length, which zero_k_tail() repairs.
+//
+// K-contiguous operand, element (r, k) at p[r*ld + k]: LDS [256 rows][4 x 16 B], the chunk index
+// XORed with (row >> 1) & 3 so that 16 consecutive rows of one chunk column cover all 64 banks.
+// Wave w, load i fills LDS bytes [(4i+w)*1024, +1024) = rows 16(4i+w) .. +16.
+__device__ __forceinline__ void load_kc(const bf16_t *p, long ld, int r0, int r_ext, int k0, uint32_t lds) {
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int blk = 4 * i + w;
+        const int row = blk * 16 + (lane >> 2);
+        const int c = (lane & 3) ^ ((row >> 1) & 3);
+        const int r = min(r0 + row, r_ext - 1);
+        dma16(p + (long)r * ld + k0 + c * 8, __builtin_amdgcn_readfirstlane(lds + blk * 1024));
+    }
+}
+// K-strided operand, element (r, k) at p[k*ld + r]: LDS [32 k][256 x 2 B] as it lies in HBM, the
+// 32-byte granule index XORed with (k & 3) << 1 (conflict-free transpose reads, see frag_ks).
+// Wave w, load i fills k-rows 2(4i+w), 2(4i+w)+1.
+__device__ __forceinline__ void load_ks(const bf16_t *p, long ld, int r0, int r_ext, int k0, int k_ext, uint32_t lds) {
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int blk = 4 * i + w;
+        const int kr = blk * 2 + (lane >> 5);
+        const int pc = lane & 31;                                        // physical 16-byte slot in the k-row
+        const int c = ((((pc >> 1) ^ ((kr & 3) << 1)) << 1) | (pc & 1));  // logical 16-byte chunk
+        const int k = min(k0 + kr, k_ext - 1);
+        const int r = min(r0 + c * 8, r_ext - 8);
+        dma16(p + (long)k * ld + r, __builtin_amdgcn_readfirstlane(lds + blk * 1024));
+    }
+}
+// zero the k-rows [k_valid, 32) of a K-strided tile (the last, partial stage of a weight gradient)
+__device__ __forceinline__ void zero_k_tail(char *lds, int k_valid) {
+    for (int idx = threadIdx.x; idx < (Q_BK - k_valid) * 32; idx += Q_THREADS)
+        *reinterpret_cast<uint4 *>(lds + k_valid * 512 + idx * 16) = make_uint4(0, 0, 0, 0);
+}
+
+// ---- MFMA fragments: 8 bf16 of k for row (lane % 32) of 32-row block tb, k-sub-step kk (16 of k) --
+__device__ __forceinline__ bf16x8 frag_kc(const char *lds, int tb, int kk) {
+    const int lane = threadIdx.x & 63;
+    const int row = tb * 32 + (lane & 31);
+    const int chunk = (2 * kk + (lane >> 5)) ^ ((row >> 1) & 3);
+    return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(lds + row * 64 + chunk * 16));
+}
+// ds_read_b64_tr_b16: in a group of 16 lanes, lane 4r+q supplies the address of 4 consecutive values
+// of k-row r, and lane i receives column i of that 4 x 16 block.  Two reads give 8 of k.
+__device__ __forceinline__ bf16x8 frag_ks(const char *lds, int tb, int kk) {
+    const int lane = threadIdx.x & 63;
+    const int gq = lane >> 4, l = lane & 15;
+    const int k = 16 * kk + 8 * (gq >> 1) + (l >> 2);                   // + 4 for the second read
+    const int gran = (tb * 2 + (gq & 1)) ^ ((l >> 2) << 1);            // (k & 3) == l >> 2
+    const char *a0 = lds + k * 512 + gran * 32 + (l & 3) * 8;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)(a0));
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)(a0 + 4 * 512));
+    typedef short s16x8 __attribute__((ext_vector_type(8)));
+    const s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(bf16x8, v);
+}
+template <bool KS> __device__ __forceinline__ bf16x8 frag(const char *lds, int tb, int kk) {
+    if constexpr (KS) return frag_ks(lds, tb, kk); else return frag_kc(lds, tb, kk);
+}
+
+template <bool M_KS, bool N_KS, int TMC> struct Frags {
+    bf16x8 m[TMC], n[2];
+    __device__ __forceinline__ void read(const char *stage, int wave, int kk) {
+#pragma unroll
+        for (int tm = 0; tm < TMC; ++tm) m[tm] = frag<M_KS>(stage, tm, kk);
+#pragma unroll
+        for (int tn = 0; tn < 2; ++tn) n[tn] = frag<N_KS>(stage + Q_OPERAND, wave * 2 + tn, kk);
+    }
+    __device__ __forceinline__ void mma(f32x16 (&acc)[8][2]) const {
+#pragma unroll
+        for (int tm = 0; tm < TMC; ++tm)
+#pragma unroll
+            for (int tn = 0; tn < 2; ++tn)
+                acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(n[tn], m[tm], acc[tm][tn], 0, 0, 0);
+    }
+};
+
+// interleave hint for a phase of `mfmas` MFMAs: one MFMA, then up to two LDS reads and one global load
+template <int MFMAS> __device__ __forceinline__ void interleave() {
+#pragma unroll
+    for (int i = 0; i < MFMAS; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // LDS read
+        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // global load
+    }
+}
+
+// The K loop.  Stage s (32 of K) lives in ring buffer s % 4; its loads were issued three stages
+// earlier.  Per stage: MFMAs of k-sub-step 0 while the fragments of sub-step 1 are read; then the
+// only synchronisation point - wait until this wave's share of stage s+1 has landed (the two newer
+// stages may still be in flight), barrier, issue the loads of stage s+3 into the buffer everyone
+// has just left - and the MFMAs of sub-step 1 while the first fragments of stage s+1 are read.
+template <bool M_KS, bool N_KS, bool WG, int TMC>
+__device__ __forceinline__ void main_loop(const bf16_t *Mp, long ldm, int m0, int m_ext, const bf16_t *Np, long ldn,
+                                          int n0, int n_ext, int k_ext, char *smem, int wave, f32x16 (&acc)[8][2]) {
+    const int nk = (k_ext + Q_BK - 1) / Q_BK;
+    if (nk == 0) return;
+    auto issue = [&](int s) {   // stage index is clamped: past the end the last stage is fetched again, harmlessly
+        const uint32_t buf = lds_offset_of(smem) + (s & (Q_NSTAGE - 1)) * Q_STAGE;
+        const int k0 = min(s, nk - 1) * Q_BK;
+        if constexpr (M_KS) load_ks(Mp, ldm, m0, m_ext, k0, k_ext, buf);
+        else load_kc(Mp, ldm, m0, m_ext, k0, buf);
+        if constexpr (N_KS) load_ks(Np, ldn, n0, n_ext, k0, k_ext, buf + Q_OPERAND);
+        else load_kc(Np, ldn, n0, n_ext, k0, buf + Q_OPERAND);
+    };
+    auto fix_tail = [&](int s) {   // ragged contraction: zero what lies past it in the last stage
+        if (WG && s == nk - 1 && (k_ext & (Q_BK - 1))) {
+            char *buf = smem + (s & (Q_NSTAGE - 1)) * Q_STAGE;
+            zero_k_tail(buf, k_ext & (Q_BK - 1));
+            zero_k_tail(buf + Q_OPERAND, k_ext & (Q_BK - 1));
+            __syncthreads();
+        }
+    };
+    issue(0);
+    issue(1);
+    issue(2);
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(2 * Q_LOADS_PER_STAGE));
+    __builtin_amdgcn_s_barrier();
+    fix_tail(0);
+    Frags<M_KS, N_KS, TMC> f0, f1;
+    f0.read(smem, wave, 0);
+    for (int s = 0; s < nk; ++s) {
+        const char *cur = smem + (s & (Q_NSTAGE - 1)) * Q_STAGE;
+        const char *nxt = smem + ((s + 1) & (Q_NSTAGE - 1)) * Q_STAGE;
+        f1.read(cur, wave, 1);
+        f0.mma(acc);
+        interleave<2 * TMC>();
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm(Q_LOADS_PER_STAGE));
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        issue(s + 3);
+        fix_tail(s + 1);
+        f0.read(nxt, wave, 0);
+        f1.mma(acc);
+        interleave<2 * TMC>();
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));   // nothing may still be writing LDS when the block retires
+}
+
+__device__ __forceinline__ uint2 pack4(float a, float b, float c, float d) {
+    const bf16x4 v = {(bf16_t)a, (bf16_t)b, (bf16_t)c, (bf16_t)d};
+    return __builtin_bit_cast(uint2, v);
+}
+__device__ __forceinline__ void unpack4(uint2 u, float *f) {
+    f[0] = __uint_as_float(u.x << 16);
+    f[1] = __uint_as_float(u.x & 0xffff0000u);
+    f[2] = __uint_as_float(u.y << 16);
+    f[3] = __uint_as_float(u.y & 0xffff0000u);
+}
+
+// Row-ragged (!WG): C[rows_e, N] = Mop[rows_e, K] . Nop_e ; Mop K-contiguous, Nop_e [N,K] or (N_KS) [K,N].
+// Weight gradient (WG): C_e[M, N] = sum_{r in rows_e} Mop[r, M]^T . Nop[r, N], both K-strided.
+template <bool N_KS, bool WG, int EPI>
+__global__ __launch_bounds__(Q_THREADS) void gemm256_kernel(const GemmArgs g) {
+    constexpr bool M_KS = WG;
+    extern __shared__ __align__(16) char smem[];
+    // ---- which tile am I?  Blocks are dealt round-robin to the 8 XCDs (block b runs on XCD b mod 8):
+    //      give each XCD a contiguous range of the REAL tiles, so that neighbours share operands in
+    //      its L2 and every XCD gets the same share.  For row-ragged products the number of real
+    //      tiles is only known here (the grid is sized for the worst case), hence the device-side sum.
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n_tiles = (g.N + Q_BN - 1) / Q_BN;
+    int e, mt, nt, m_ext, k_ext;
+    long row0;  // first row of the expert
+    if constexpr (!WG) {
+        int total_m_tiles;
+        if (g.offsets == nullptr) {
+            total_m_tiles = (g.single_rows + Q_BM - 1) / Q_BM;
+        } else {
+            int part = 0;
+            for (int ee = lane; ee < g.E; ee += WAVE) part += (g.kept[ee] + Q_BM - 1) / Q_BM;
+            for (int d = WAVE / 2; d >= 1; d >>= 1) part += __shfl_xor(part, d, WAVE);
+            total_m_tiles = part;
+        }
+        const int total = total_m_tiles * n_tiles;
+        const int per_xcd = (total + 7) >> 3;
+        const int slot = blockIdx.x >> 3;
+        const int t = (blockIdx.x & 7) * per_xcd + slot;
+        if (slot >= per_xcd || t >= total) return;
+        const int mtg = t / n_tiles;
+        nt = t % n_tiles;
+        if (g.offsets == nullptr) {
+            e = 0; mt = mtg; m_ext = g.single_rows; row0 = 0;
+        } else {
+            int run = 0, found = -1, fmt = 0;
+            for (int base = 0; base < g.E && found < 0; base += WAVE) {
+                const int ee = base + lane;
+                const int tiles = ee < g.E ? (g.kept[ee] + Q_BM - 1) / Q_BM : 0;
+                int incl = tiles;
+                for (int d = 1; d < WAVE; d <<= 1) {
+                    const int y = __shfl_up(incl, d, WAVE);
+                    if (lane >= d) incl += y;
+                }
+                const unsigned long long hit = __ballot(run + incl > mtg);
+                if (hit) {
+                    const int src = __ffsll(hit) - 1;
+                    found = base + src;
+                    fmt = mtg - (run + __shfl(incl - tiles, src, WAVE));
+                }
+                run += __shfl(incl, WAVE - 1, WAVE);
+            }
+            if (found < 0) return;
+            e = found; mt = fmt;
+            m_ext = g.kept[e];
+            row0 = g.offsets[e];
+        }
+        k_ext = g.K;
+    } else {
+        const int nblk = gridDim.x;
+        const int t = (blockIdx.x & 7) * (nblk >> 3) + (blockIdx.x >> 3);
+        if (t >= g.n_blocks) return;
+        const int m_tiles = (g.M + Q_BM - 1) / Q_BM;
+        e = t / (m_tiles * n_tiles);
+        const int rem = t % (m_tiles * n_tiles);
+        mt = rem / n_tiles;
+        nt = rem % n_tiles;
+        m_ext = g.M;
+        k_ext = g.kept ? g.kept[e] : g.single_rows;
+        row0 = g.offsets ? g.offsets[e] : 0;
+    }
+    const int m0 = mt * Q_BM, n0 = nt * Q_BN;
+    const bf16_t *Mp = (const bf16_t *)g.A + row0 * g.lda;
+    const bf16_t *Np = WG ? (const bf16_t *)g.B + row0 * g.ldb : (const bf16_t *)g.B + (long)e * g.strideB;
+
+    f32x16 acc[8][2];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
+
+    const int live = min(Q_BM, m_ext - m0);
+    const int tmc = (live + 31) >> 5;
+    if (tmc > 4)
+        main_loop<M_KS, N_KS, WG, 8>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wave, acc);
+    else if (tmc > 2)
+        main_loop<M_KS, N_KS, WG, 4>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wave, acc);
+    else
+        main_loop<M_KS, N_KS, WG, 2>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wave, acc);
+
+    // ---- epilogue.  acc[tm][tn][4q+j] = C[m, n] with m = m0 + 32 tm + lane%32 and
+    //      n = n0 + 64 wave + 32 tn + 8 q + 4 (lane/32) + j.  A wave owns a 256 x 64 slab of the tile.
+    //      bf16 results go through the wave's own 32 KiB of LDS (the K loop is done with it) so that
+    //      global memory sees whole 128-byte rows: 8 bytes per lane into LDS ([row][8 x 16 B], chunk
+    //      ^ (row & 7)), then 16 bytes per lane out, 8 rows per store instruction.  The pre-activation
+    //      that GELU' needs comes in the same way, in the opposite direction.
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+    __syncthreads();
+    const int lm = lane & 31, h = lane >> 5;
+    bf16_t *Cb = (bf16_t *)g.C;
+    long crow0 = row0;
+    if constexpr (WG) { crow0 = 0; Cb += (long)e * g.strideC; }
+    const int nw0 = n0 + wave * 64;                 // first column of this wave's slab
+    char *slab = smem + wave * (Q_BM * 128);
+    const int jr = lane >> 3, jc = lane & 7;        // row-in-group / 16-byte column of the wide accesses
+    const bool col_ok = nw0 + jc * 8 < g.N;
+
+    auto slab_at = [&](int row, int chunk, int half) -> char * {
+        return slab + row * 128 + ((chunk ^ (row & 7)) << 4) + half * 8;
+    };
+    // slab -> global: rows [0, live) of the slab, 128 bytes each
+    auto flush = [&](bf16_t *dst) {
+        for (int it = 0; it * 8 < live; ++it) {
+            const int row = it * 8 + jr;
+            const uint4 v = *reinterpret_cast<const uint4 *>(slab_at(row, jc, 0));
+            if (row < live && col_ok)
+                *reinterpret_cast<uint4 *>(dst + (crow0 + m0 + row) * g.ldc + nw0 + jc * 8) = v;
+        }
+    };
+    // global -> slab
+    auto fill = [&](const bf16_t *src) {
+        for (int it = 0; it * 8 < live; ++it) {
+            const int row = it * 8 + jr;
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (row < live && col_ok) v = *reinterpret_cast<const uint4 *>(src + (crow0 + m0 + row) * g.ldc + nw0 + jc * 8);
+            *reinterpret_cast<uint4 *>(slab_at(row, jc, 0)) = v;
+        }
+    };
+
+    if constexpr (EPI == EPI_F32) {
+#pragma unroll
+        for (int tn = 0; tn < 2; ++tn)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int n = nw0 + tn * 32 + 8 * q + 4 * h;
+                if (n >= g.N) continue;
+#pragma unroll
+                for (int tm = 0; tm < 8; ++tm) {
+                    const int m = m0 + tm * 32 + lm;
+                    if (tm >= tmc || m >= m_ext) continue;
+                    *reinterpret_cast<float4 *>((float *)g.C + (crow0 + m) * g.ldc + n) =
+                        make_float4(acc[tm][tn][4 * q], acc[tm][tn][4 * q + 1], acc[tm][tn][4 * q + 2], acc[tm][tn][4 * q + 3]);
+                }
+            }
+        return;
+    }
+    if constexpr (EPI == EPI_DGELU) fill((const bf16_t *)g.H);
+    if constexpr (EPI == EPI_WGRAD) { if (g.accumulate) fill(Cb); }
+
+    // pass 0 writes C; for EPI_BIAS_GELU pass 1 writes C2 = gelu(h)
+    constexpr int PASSES = EPI == EPI_BIAS_GELU ? 2 : 1;
+#pragma unroll
+    for (int pass = 0; pass < PASSES; ++pass) {
+#pragma unroll
+        for (int tn = 0; tn < 2; ++tn) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int n = nw0 + tn * 32 + 8 * q + 4 * h;
+                float bias[4] = {0.f, 0.f, 0.f, 0.f};
+                if constexpr (EPI == EPI_BIAS || EPI == EPI_BIAS_GELU) {
+                    if (n < g.N) unpack4(*reinterpret_cast<const uint2 *>((const bf16_t *)g.bias + (long)e * g.N + n), bias);
+                }
+#pragma unroll
+                for (int tm = 0; tm < 8; ++tm) {
+                    if (tm >= tmc) continue;
+                    char *cell = slab_at(tm * 32 + lm, tn * 4 + q, h);
+                    float v[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) v[j] = acc[tm][tn][4 * q + j];
+                    if constexpr (EPI == EPI_BIAS) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) v[j] += bias[j];
+                    } else if constexpr (EPI == EPI_BIAS_GELU) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) v[j] += bias[j];
+                        if (pass == 1) {
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) v[j] = fast_gelu_erf(v[j]);
+                        }
+                    } else if constexpr (EPI == EPI_DGELU) {
+                        float hv[4];
+                        unpack4(*reinterpret_cast<const uint2 *>(cell), hv);
+                        if (g.gelu_bwd == MOLE_GELU_BWD_TANH) {
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) v[j] *= fast_d_gelu_tanh(hv[j]);
+                        } else {
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) v[j] *= fast_d_gelu_exact(hv[j]);
+                        }
+                    } else if constexpr (EPI == EPI_WGRAD) {
+                        if (g.accumulate) {
+                            float old[4];
+                            unpack4(*reinterpret_cast<const uint2 *>(cell), old);
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) v[j] += old[j];
+                        }
+                    }
+                    *reinterpret_cast<uint2 *>(cell) = pack4(v[0], v[1], v[2], v[3]);
+                }
+            }
+        }
+        flush(pass == 0 ? Cb : (bf16_t *)g.C2);
+    }
+}
+
+template <bool N_KS, bool WG, int EPI>
+static int launch256(GemmArgs g, int tiles, hipStream_t st, int kid) {
+    if (tiles <= 0) return 0;
+    ScopedTiming timing(kid, st);
+    g.n_blocks = tiles;
+    const int grid = (tiles + 7) & ~7;
+    auto kern = gemm256_kernel<N_KS, WG, EPI>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        MOLE_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, Q_NSTAGE * Q_STAGE));
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(Q_THREADS), Q_NSTAGE * Q_STAGE, st, g);
+    MOLE_LAUNCH_CHECK();
+    return 0;
+}
+
+int launch_gemm256(const GemmArgs &g, bool a_ks, bool b_ks, bool wg, int epi, int max_rows, hipStream_t st, int kid) {
+    // alignment the direct-to-LDS path relies on: 16-byte rows, whole K-steps for row-ragged products
+    if (g.lda % 8 || g.ldb % 8 || g.ldc % 8 || g.N % 8) return -100;
+    if (!wg && (a_ks || g.K % Q_BK)) return -100;
+    if (wg && (!a_ks || !b_ks || g.M % 8)) return -100;
+    const int n_tiles = ceil_div(g.N, Q_BN);
+    if (wg) {
+        const int tiles = g.E * ceil_div(g.M, Q_BM) * n_tiles;
+        if (epi == EPI_WGRAD) return launch256<true, true, EPI_WGRAD>(g, tiles, st, kid);
+        return -100;
+    }
+    const int m_tiles = g.offsets ? max_rows / Q_BM + g.E : ceil_div(g.single_rows, Q_BM);
+    const int tiles = m_tiles * n_tiles;
+    if (!b_ks) {
+        if (epi == EPI_BIAS_GELU) return launch256<false, false, EPI_BIAS_GELU>(g, tiles, st, kid);
+        if (epi == EPI_DGELU) return launch256<false, false, EPI_DGELU>(g, tiles, st, kid);
+        if (epi == EPI_F32) return launch256<false, false, EPI_F32>(g, tiles, st, kid);
+    } else {
+        if (epi == EPI_BIAS) return launch256<true, false, EPI_BIAS>(g, tiles, st, kid);
+        if (epi == EPI_STORE) return launch256<true, false, EPI_STORE>(g, tiles, st, kid);
+    }
+    return -100;
+}
+
+}  // namespace mole
