@@ -52,6 +52,7 @@ struct GemmArgs {
     int accumulate;         // EPI_WGRAD: add into C
     int gelu_bwd;           // EPI_DGELU: MOLE_GELU_BWD_*
     int n_blocks;           // real number of tiles in the launch (grid is rounded up to 8)
+    int full_blocks;        // 256-wide kernel, row-ragged: block slots reserved for full m-tiles
 };
 
 

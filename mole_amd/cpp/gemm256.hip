@@ -1,32 +1,44 @@
-// bf16 grouped GEMM on 256 x 256 tiles for gfx950: the fast path of the six expert-FFN products.
+// bf16 grouped GEMM for gfx950: the fast path of the six expert-FFN products.
 //
-// A block of 4 waves owns a 256 (m) x 256 (n) output tile; every wave covers all 256 m and 64 n
-// (8 x 2 MFMA 32x32x16 blocks, 256 fp32 accumulators in AGPRs).  Operand tiles go from HBM/L2
-// straight into LDS (global_load_lds_dwordx4, no staging registers) through a ring of four stages of
-// 32 of K, so that three stages of loads are in flight while one is consumed: with a single stage
-// of look-ahead the loop ran at the memory latency, not at the MFMA rate.  One barrier per stage.
-// Each 16-byte piece is placed at a swizzled LDS position by choosing which global address the lane
-// that owns the slot fetches:
+// A block of 4 waves owns a BM (m) x 256 (n) output tile, BM = 256 or 128; every wave covers all BM
+// rows and 64 columns (BM/32 x 2 MFMA 32x32x16 blocks, fp32 accumulators in AGPRs).  BM = 256 runs
+// one block per CU (256 accumulator registers per lane); BM = 128 runs two, so that one block's
+// epilogue overlaps the other's K loop and ragged experts quantise into finer tiles.
+// Operand tiles go from HBM/L2 straight into LDS (global_load_lds_dwordx4, no staging registers)
+// through a ring of stages of 32 of K, several stages of loads in flight while one is consumed: with
+// a single stage of look-ahead the loop ran at the memory latency, not at the MFMA rate.  One
+// barrier per stage.  Each 16-byte piece is placed at a swizzled LDS position by choosing which
+// global address the lane that owns the slot fetches:
 //   * K-contiguous operand  -> LDS [row][4 x 16 B]; fragments read with ds_read_b128
-//   * K-strided operand     -> LDS [k][256 x 2 B] as it lies in HBM; fragments read with
+//   * K-strided operand     -> LDS [k][rows x 2 B] as it lies in HBM; fragments read with
 //                              ds_read_b64_tr_b16, the LDS transpose read
 // The MFMA "A" slot is fed with the n-side operand and the "B" slot with the m-side operand, so the
-// four consecutive accumulator rows a lane holds are four consecutive n: the epilogue stores (and
-// the bias / pre-activation loads) are 8 bytes per lane.
-// A ragged m-tile runs only the 32-row blocks it has rows for (2, 4 or 8 of 8).
+// four consecutive accumulator rows a lane holds are four consecutive n; results leave through LDS
+// as whole 128-byte rows.  A ragged m-tile runs only the 32-row blocks it has rows for.
 #include "gemm.h"
+
+#include <stdlib.h>
 
 namespace mole {
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 
-constexpr int Q_BM = 256, Q_BN = 256, Q_BK = 32;
-constexpr int Q_OPERAND = 16 * 1024;        // one operand tile of one stage
-constexpr int Q_STAGE = 2 * Q_OPERAND;
-constexpr int Q_NSTAGE = 4;                 // ring of LDS stages: one consumed, up to three in flight
+constexpr int Q_BN = 256, Q_BK = 32;
 constexpr int Q_THREADS = 256;
-constexpr int Q_LOADS_PER_STAGE = 8;        // asynchronous loads a wave issues per stage
+constexpr int Q_N_OPERAND = Q_BN * Q_BK * 2;   // bytes of the n-side tile of one stage
+
+// geometry of a tile with TMB 32-row m-blocks
+template <int TMB> struct Tile {
+    static constexpr int BM = TMB * 32;
+    static constexpr int M_OPERAND = BM * Q_BK * 2;
+    static constexpr int STAGE = M_OPERAND + Q_N_OPERAND;
+    static constexpr int NSTAGE = TMB >= 8 ? 4 : 3;
+    static constexpr int LOADS = (M_OPERAND + Q_N_OPERAND) / 4096;   // asynchronous loads per wave per stage
+    static constexpr int SLABS = 4 * BM * 128;                       // the four waves' epilogue staging areas
+    static constexpr int LDS_BYTES = NSTAGE * STAGE > SLABS ? NSTAGE * STAGE : SLABS;
+    static constexpr int BLOCKS_PER_CU = TMB >= 8 ? 1 : 2;
+};
 
 // s_waitcnt immediate that waits for vmcnt <= n and nothing else (gfx9 encoding: vmcnt in bits 3:0
 // and 15:14, expcnt 6:4, lgkmcnt 11:8)
@@ -56,9 +68,16 @@ __device__ __forceinline__ float fast_erf_abs(float z) {  // erf(z) for z >= 0
     const float e = __builtin_amdgcn_exp2f(-1.4426950408889634f * z * z);
     return fmaf(-p, e, 1.0f);
 }
+// gelu(x) = max(x,0) - |x/2| * erfc(|x|/sqrt 2), erfc from the same formula: no sign handling needed
 __device__ __forceinline__ float fast_gelu_erf(float x) {
-    const float er = fast_erf_abs(fabsf(x) * 0.70710678118654752f);
-    return 0.5f * x * (1.0f + copysignf(er, x));
+    const float z = fabsf(x) * 0.70710678118654752f;
+    const float t = __builtin_amdgcn_rcpf(fmaf(0.3275911f, z, 1.0f));
+    float p = fmaf(1.061405429f, t, -1.453152027f);
+    p = fmaf(p, t, 1.421413741f);
+    p = fmaf(p, t, -0.284496736f);
+    p = fmaf(p, t, 0.254829592f);
+    const float erfc_z = p * t * __builtin_amdgcn_exp2f(-1.4426950408889634f * z * z);
+    return fmaf(-fabsf(0.5f * x), erfc_z, fmaxf(x, 0.f));
 }
 __device__ __forceinline__ float fast_tanh(float u) {  // 1 - 2/(1+e^{2u}), saturates cleanly
     const float e = __builtin_amdgcn_exp2f(2.0f * 1.4426950408889634f * u);
@@ -85,13 +104,13 @@ __device__ __forceinline__ float fast_d_gelu_exact(float x) {
 // LDS for them is real, finite data that only contributes to output rows or columns the epilogue
 // does not store - except along a ragged contraction length, which zero_k_tail() repairs.
 //
-// K-contiguous operand, element (r, k) at p[r*ld + k]: LDS [256 rows][4 x 16 B], the chunk index
-// XORed with (row >> 1) & 3 so that 16 consecutive rows of one chunk column cover all 64 banks.
-// Wave w, load i fills LDS bytes [(4i+w)*1024, +1024) = rows 16(4i+w) .. +16.
+// K-contiguous operand, element (r, k) at p[r*ld + k]: LDS [ROWS][4 x 16 B], the chunk index XORed
+// with (row >> 1) & 3.  Wave w, load i fills LDS bytes [(4i+w)*1024, +1024) = rows 16(4i+w) .. +16.
+template <int ROWS>
 __device__ __forceinline__ void load_kc(const bf16_t *p, long ld, int r0, int r_ext, int k0, uint32_t lds) {
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < ROWS / 64; ++i) {
         const int blk = 4 * i + w;
         const int row = blk * 16 + (lane >> 2);
         const int c = (lane & 3) ^ ((row >> 1) & 3);
@@ -99,16 +118,19 @@ __device__ __forceinline__ void load_kc(const bf16_t *p, long ld, int r0, int r_
         dma16(p + (long)r * ld + k0 + c * 8, __builtin_amdgcn_readfirstlane(lds + blk * 1024));
     }
 }
-// K-strided operand, element (r, k) at p[k*ld + r]: LDS [32 k][256 x 2 B] as it lies in HBM, the
+// K-strided operand, element (r, k) at p[k*ld + r]: LDS [32 k][ROWS x 2 B] as it lies in HBM, the
 // 32-byte granule index XORed with (k & 3) << 1 (conflict-free transpose reads, see frag_ks).
-// Wave w, load i fills k-rows 2(4i+w), 2(4i+w)+1.
+// A k-row has ROWS/8 slots of 16 bytes; a wave load of 1 KiB covers 512/ROWS k-rows.
+template <int ROWS>
 __device__ __forceinline__ void load_ks(const bf16_t *p, long ld, int r0, int r_ext, int k0, int k_ext, uint32_t lds) {
+    constexpr int SPR = ROWS / 8;          // 16-byte slots per k-row
+    constexpr int KPL = 64 / SPR;          // k-rows per wave load
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < ROWS / 64; ++i) {
         const int blk = 4 * i + w;
-        const int kr = blk * 2 + (lane >> 5);
-        const int pc = lane & 31;                                        // physical 16-byte slot in the k-row
+        const int kr = blk * KPL + lane / SPR;
+        const int pc = lane % SPR;                                        // physical 16-byte slot in the k-row
         const int c = ((((pc >> 1) ^ ((kr & 3) << 1)) << 1) | (pc & 1));  // logical 16-byte chunk
         const int k = min(k0 + kr, k_ext - 1);
         const int r = min(r0 + c * 8, r_ext - 8);
@@ -116,9 +138,9 @@ __device__ __forceinline__ void load_ks(const bf16_t *p, long ld, int r0, int r_
     }
 }
 // zero the k-rows [k_valid, 32) of a K-strided tile (the last, partial stage of a weight gradient)
-__device__ __forceinline__ void zero_k_tail(char *lds, int k_valid) {
-    for (int idx = threadIdx.x; idx < (Q_BK - k_valid) * 32; idx += Q_THREADS)
-        *reinterpret_cast<uint4 *>(lds + k_valid * 512 + idx * 16) = make_uint4(0, 0, 0, 0);
+template <int ROWS> __device__ __forceinline__ void zero_k_tail(char *lds, int k_valid) {
+    for (int idx = threadIdx.x; idx < (Q_BK - k_valid) * (ROWS / 8); idx += Q_THREADS)
+        *reinterpret_cast<uint4 *>(lds + k_valid * (ROWS * 2) + idx * 16) = make_uint4(0, 0, 0, 0);
 }
 
 // ---- MFMA fragments: 8 bf16 of k for row (lane % 32) of 32-row block tb, k-sub-step kk (16 of k) --
@@ -130,31 +152,31 @@ __device__ __forceinline__ bf16x8 frag_kc(const char *lds, int tb, int kk) {
 }
 // ds_read_b64_tr_b16: in a group of 16 lanes, lane 4r+q supplies the address of 4 consecutive values
 // of k-row r, and lane i receives column i of that 4 x 16 block.  Two reads give 8 of k.
-__device__ __forceinline__ bf16x8 frag_ks(const char *lds, int tb, int kk) {
+template <int ROWS> __device__ __forceinline__ bf16x8 frag_ks(const char *lds, int tb, int kk) {
     const int lane = threadIdx.x & 63;
     const int gq = lane >> 4, l = lane & 15;
     const int k = 16 * kk + 8 * (gq >> 1) + (l >> 2);                   // + 4 for the second read
     const int gran = (tb * 2 + (gq & 1)) ^ ((l >> 2) << 1);            // (k & 3) == l >> 2
-    const char *a0 = lds + k * 512 + gran * 32 + (l & 3) * 8;
+    const char *a0 = lds + k * (ROWS * 2) + gran * 32 + (l & 3) * 8;
     const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)(a0));
-    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)(a0 + 4 * 512));
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)(a0 + 4 * ROWS * 2));
     typedef short s16x8 __attribute__((ext_vector_type(8)));
     const s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
     return __builtin_bit_cast(bf16x8, v);
 }
-template <bool KS> __device__ __forceinline__ bf16x8 frag(const char *lds, int tb, int kk) {
-    if constexpr (KS) return frag_ks(lds, tb, kk); else return frag_kc(lds, tb, kk);
+template <bool KS, int ROWS> __device__ __forceinline__ bf16x8 frag(const char *lds, int tb, int kk) {
+    if constexpr (KS) return frag_ks<ROWS>(lds, tb, kk); else return frag_kc(lds, tb, kk);
 }
 
-template <bool M_KS, bool N_KS, int TMC> struct Frags {
+template <int TMB, bool M_KS, bool N_KS, int TMC> struct Frags {
     bf16x8 m[TMC], n[2];
     __device__ __forceinline__ void read(const char *stage, int wave, int kk) {
 #pragma unroll
-        for (int tm = 0; tm < TMC; ++tm) m[tm] = frag<M_KS>(stage, tm, kk);
+        for (int tm = 0; tm < TMC; ++tm) m[tm] = frag<M_KS, Tile<TMB>::BM>(stage, tm, kk);
 #pragma unroll
-        for (int tn = 0; tn < 2; ++tn) n[tn] = frag<N_KS>(stage + Q_OPERAND, wave * 2 + tn, kk);
+        for (int tn = 0; tn < 2; ++tn) n[tn] = frag<N_KS, Q_BN>(stage + Tile<TMB>::M_OPERAND, wave * 2 + tn, kk);
     }
-    __device__ __forceinline__ void mma(f32x16 (&acc)[8][2]) const {
+    __device__ __forceinline__ void mma(f32x16 (&acc)[TMB][2]) const {
 #pragma unroll
         for (int tm = 0; tm < TMC; ++tm)
 #pragma unroll
@@ -163,7 +185,7 @@ template <bool M_KS, bool N_KS, int TMC> struct Frags {
     }
 };
 
-// interleave hint for a phase of `mfmas` MFMAs: one MFMA, then up to two LDS reads and one global load
+// interleave hint for a phase of MFMAS MFMAs: one MFMA, then up to two LDS reads and one global load
 template <int MFMAS> __device__ __forceinline__ void interleave() {
 #pragma unroll
     for (int i = 0; i < MFMAS; ++i) {
@@ -173,56 +195,62 @@ template <int MFMAS> __device__ __forceinline__ void interleave() {
     }
 }
 
-// The K loop.  Stage s (32 of K) lives in ring buffer s % 4; its loads were issued three stages
-// earlier.  Per stage: MFMAs of k-sub-step 0 while the fragments of sub-step 1 are read; then the
-// only synchronisation point - wait until this wave's share of stage s+1 has landed (the two newer
-// stages may still be in flight), barrier, issue the loads of stage s+3 into the buffer everyone
-// has just left - and the MFMAs of sub-step 1 while the first fragments of stage s+1 are read.
-template <bool M_KS, bool N_KS, bool WG, int TMC>
+// The K loop.  Stage s (32 of K) lives in ring buffer s mod NSTAGE; its loads were issued NSTAGE-1
+// stages earlier.  Per stage: MFMAs of k-sub-step 0 while the fragments of sub-step 1 are read; then
+// the only synchronisation point - wait until this wave's share of stage s+1 has landed (newer
+// stages may still be in flight), barrier, issue the loads of stage s+NSTAGE-1 into the buffer
+// everyone has just left - and the MFMAs of sub-step 1 while the first fragments of stage s+1 are read.
+template <int TMB, bool M_KS, bool N_KS, bool WG, int TMC>
 __device__ __forceinline__ void main_loop(const bf16_t *Mp, long ldm, int m0, int m_ext, const bf16_t *Np, long ldn,
-                                          int n0, int n_ext, int k_ext, char *smem, int wave, f32x16 (&acc)[8][2]) {
+                                          int n0, int n_ext, int k_ext, char *smem, int wave, f32x16 (&acc)[TMB][2]) {
+    typedef Tile<TMB> TL;
+    constexpr int AHEAD = TL::NSTAGE - 1;
     const int nk = (k_ext + Q_BK - 1) / Q_BK;
     if (nk == 0) return;
-    auto issue = [&](int s) {   // stage index is clamped: past the end the last stage is fetched again, harmlessly
-        const uint32_t buf = lds_offset_of(smem) + (s & (Q_NSTAGE - 1)) * Q_STAGE;
+    const uint32_t lds0 = lds_offset_of(smem);
+    auto issue = [&](int s, int buf) {   // stage index is clamped: past the end the last stage is fetched again, harmlessly
+        const uint32_t dst = lds0 + buf * TL::STAGE;
         const int k0 = min(s, nk - 1) * Q_BK;
-        if constexpr (M_KS) load_ks(Mp, ldm, m0, m_ext, k0, k_ext, buf);
-        else load_kc(Mp, ldm, m0, m_ext, k0, buf);
-        if constexpr (N_KS) load_ks(Np, ldn, n0, n_ext, k0, k_ext, buf + Q_OPERAND);
-        else load_kc(Np, ldn, n0, n_ext, k0, buf + Q_OPERAND);
+        if constexpr (M_KS) load_ks<TL::BM>(Mp, ldm, m0, m_ext, k0, k_ext, dst);
+        else load_kc<TL::BM>(Mp, ldm, m0, m_ext, k0, dst);
+        if constexpr (N_KS) load_ks<Q_BN>(Np, ldn, n0, n_ext, k0, k_ext, dst + TL::M_OPERAND);
+        else load_kc<Q_BN>(Np, ldn, n0, n_ext, k0, dst + TL::M_OPERAND);
     };
-    auto fix_tail = [&](int s) {   // ragged contraction: zero what lies past it in the last stage
+    auto fix_tail = [&](int s, int buf) {   // ragged contraction: zero what lies past it in the last stage
         if (WG && s == nk - 1 && (k_ext & (Q_BK - 1))) {
-            char *buf = smem + (s & (Q_NSTAGE - 1)) * Q_STAGE;
-            zero_k_tail(buf, k_ext & (Q_BK - 1));
-            zero_k_tail(buf + Q_OPERAND, k_ext & (Q_BK - 1));
+            char *b = smem + buf * TL::STAGE;
+            zero_k_tail<TL::BM>(b, k_ext & (Q_BK - 1));
+            zero_k_tail<Q_BN>(b + TL::M_OPERAND, k_ext & (Q_BK - 1));
             __syncthreads();
         }
     };
-    issue(0);
-    issue(1);
-    issue(2);
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm(2 * Q_LOADS_PER_STAGE));
+#pragma unroll
+    for (int s = 0; s < AHEAD; ++s) issue(s, s);
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm((AHEAD - 1) * TL::LOADS));
     __builtin_amdgcn_s_barrier();
-    fix_tail(0);
-    Frags<M_KS, N_KS, TMC> f0, f1;
+    fix_tail(0, 0);
+    Frags<TMB, M_KS, N_KS, TMC> f0, f1;
     f0.read(smem, wave, 0);
+    int cur_b = 0;                    // ring buffer of stage s
     for (int s = 0; s < nk; ++s) {
-        const char *cur = smem + (s & (Q_NSTAGE - 1)) * Q_STAGE;
-        const char *nxt = smem + ((s + 1) & (Q_NSTAGE - 1)) * Q_STAGE;
+        const int nxt_b = cur_b + 1 == TL::NSTAGE ? 0 : cur_b + 1;
+        const int free_b = cur_b == 0 ? TL::NSTAGE - 1 : cur_b - 1;     // held stage s-1, takes stage s+AHEAD
+        const char *cur = smem + cur_b * TL::STAGE;
+        const char *nxt = smem + nxt_b * TL::STAGE;
         f1.read(cur, wave, 1);
         f0.mma(acc);
         interleave<2 * TMC>();
         __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm(Q_LOADS_PER_STAGE));
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm((AHEAD - 2) * TL::LOADS));
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
-        issue(s + 3);
-        fix_tail(s + 1);
+        issue(s + AHEAD, free_b);
+        fix_tail(s + 1, nxt_b);
         f0.read(nxt, wave, 0);
         f1.mma(acc);
         interleave<2 * TMC>();
         __builtin_amdgcn_sched_barrier(0);
+        cur_b = nxt_b;
     }
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));   // nothing may still be writing LDS when the block retires
 }
@@ -240,9 +268,10 @@ __device__ __forceinline__ void unpack4(uint2 u, float *f) {
 
 // Row-ragged (!WG): C[rows_e, N] = Mop[rows_e, K] . Nop_e ; Mop K-contiguous, Nop_e [N,K] or (N_KS) [K,N].
 // Weight gradient (WG): C_e[M, N] = sum_{r in rows_e} Mop[r, M]^T . Nop[r, N], both K-strided.
-template <bool N_KS, bool WG, int EPI>
-__global__ __launch_bounds__(Q_THREADS) void gemm256_kernel(const GemmArgs g) {
+template <int TMB, bool N_KS, bool WG, int EPI>
+__global__ __launch_bounds__(Q_THREADS, Tile<TMB>::BLOCKS_PER_CU) void gemm256_kernel(const GemmArgs g) {
     constexpr bool M_KS = WG;
+    constexpr int Q_BM = Tile<TMB>::BM;
     extern __shared__ __align__(16) char smem[];
     // ---- which tile am I?  Blocks are dealt round-robin to the 8 XCDs (block b runs on XCD b mod 8):
     //      give each XCD a contiguous range of the REAL tiles, so that neighbours share operands in
@@ -253,47 +282,65 @@ __global__ __launch_bounds__(Q_THREADS) void gemm256_kernel(const GemmArgs g) {
     int e, mt, nt, m_ext, k_ext;
     long row0;  // first row of the expert
     if constexpr (!WG) {
-        int total_m_tiles;
-        if (g.offsets == nullptr) {
-            total_m_tiles = (g.single_rows + Q_BM - 1) / Q_BM;
-        } else {
-            int part = 0;
-            for (int ee = lane; ee < g.E; ee += WAVE) part += (g.kept[ee] + Q_BM - 1) / Q_BM;
-            for (int d = WAVE / 2; d >= 1; d >>= 1) part += __shfl_xor(part, d, WAVE);
-            total_m_tiles = part;
+        // Heavy m-tiles (more than BM/2 live rows) take the first g.full_blocks block slots, in
+        // contiguous per-XCD ranges; the light ones (an expert's last tile with at most BM/2 rows)
+        // take the slots after them in plain order.  The hardware starts blocks in index order, so
+        // the short tiles fill the end of the launch instead of holding CUs for a full tile's time.
+        const bool single = g.offsets == nullptr;
+        auto rows_of = [&](int ee) { return single ? g.single_rows : g.kept[ee]; };
+        const int nE = single ? 1 : g.E;
+        int n_full = 0, n_part = 0;
+        for (int ee = lane; ee < nE; ee += WAVE) {
+            const int r = rows_of(ee);
+            n_full += r / Q_BM + ((r % Q_BM) > Q_BM / 2);
+            n_part += (r % Q_BM) != 0 && (r % Q_BM) <= Q_BM / 2;
         }
-        const int total = total_m_tiles * n_tiles;
-        const int per_xcd = (total + 7) >> 3;
-        const int slot = blockIdx.x >> 3;
-        const int t = (blockIdx.x & 7) * per_xcd + slot;
-        if (slot >= per_xcd || t >= total) return;
-        const int mtg = t / n_tiles;
-        nt = t % n_tiles;
-        if (g.offsets == nullptr) {
-            e = 0; mt = mtg; m_ext = g.single_rows; row0 = 0;
+        for (int d = WAVE / 2; d >= 1; d >>= 1) {
+            n_full += __shfl_xor(n_full, d, WAVE);
+            n_part += __shfl_xor(n_part, d, WAVE);
+        }
+        int target;            // index among the full (or partial) m-tiles
+        bool want_full;
+        if ((int)blockIdx.x < g.full_blocks) {
+            const int total = n_full * n_tiles;
+            const int per_xcd = (total + 7) >> 3;
+            const int slot = blockIdx.x >> 3;
+            const int t = (blockIdx.x & 7) * per_xcd + slot;
+            if (slot >= per_xcd || t >= total) return;
+            target = t / n_tiles;
+            nt = t % n_tiles;
+            want_full = true;
         } else {
-            int run = 0, found = -1, fmt = 0;
-            for (int base = 0; base < g.E && found < 0; base += WAVE) {
-                const int ee = base + lane;
-                const int tiles = ee < g.E ? (g.kept[ee] + Q_BM - 1) / Q_BM : 0;
-                int incl = tiles;
-                for (int d = 1; d < WAVE; d <<= 1) {
-                    const int y = __shfl_up(incl, d, WAVE);
-                    if (lane >= d) incl += y;
-                }
-                const unsigned long long hit = __ballot(run + incl > mtg);
-                if (hit) {
-                    const int src = __ffsll(hit) - 1;
-                    found = base + src;
-                    fmt = mtg - (run + __shfl(incl - tiles, src, WAVE));
-                }
-                run += __shfl(incl, WAVE - 1, WAVE);
+            const int p = blockIdx.x - g.full_blocks;
+            if (p >= n_part * n_tiles) return;
+            target = p / n_tiles;
+            nt = p % n_tiles;
+            want_full = false;
+        }
+        // the expert whose running count passes `target`
+        int run = 0, found = -1, before = 0;
+        for (int base = 0; base < nE && found < 0; base += WAVE) {
+            const int ee = base + lane;
+            const int r = ee < nE ? rows_of(ee) : 0;
+            const int cnt = want_full ? r / Q_BM + ((r % Q_BM) > Q_BM / 2) : ((r % Q_BM) != 0 && (r % Q_BM) <= Q_BM / 2);
+            int incl = cnt;
+            for (int d = 1; d < WAVE; d <<= 1) {
+                const int y = __shfl_up(incl, d, WAVE);
+                if (lane >= d) incl += y;
             }
-            if (found < 0) return;
-            e = found; mt = fmt;
-            m_ext = g.kept[e];
-            row0 = g.offsets[e];
+            const unsigned long long hit = __ballot(run + incl > target);
+            if (hit) {
+                const int src = __ffsll(hit) - 1;
+                found = base + src;
+                before = run + __shfl(incl - cnt, src, WAVE);
+            }
+            run += __shfl(incl, WAVE - 1, WAVE);
         }
+        if (found < 0) return;
+        e = found;
+        m_ext = rows_of(e);
+        mt = want_full ? target - before : m_ext / Q_BM;
+        row0 = single ? 0 : g.offsets[e];
         k_ext = g.K;
     } else {
         const int nblk = gridDim.x;
@@ -312,9 +359,9 @@ __global__ __launch_bounds__(Q_THREADS) void gemm256_kernel(const GemmArgs g) {
     const bf16_t *Mp = (const bf16_t *)g.A + row0 * g.lda;
     const bf16_t *Np = WG ? (const bf16_t *)g.B + row0 * g.ldb : (const bf16_t *)g.B + (long)e * g.strideB;
 
-    f32x16 acc[8][2];
+    f32x16 acc[TMB][2];
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < TMB; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -322,16 +369,16 @@ __global__ __launch_bounds__(Q_THREADS) void gemm256_kernel(const GemmArgs g) {
 
     const int live = min(Q_BM, m_ext - m0);
     const int tmc = (live + 31) >> 5;
-    if (tmc > 4)
-        main_loop<M_KS, N_KS, WG, 8>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wave, acc);
-    else if (tmc > 2)
-        main_loop<M_KS, N_KS, WG, 4>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wave, acc);
+    if (tmc > TMB / 2)
+        main_loop<TMB, M_KS, N_KS, WG, TMB>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wave, acc);
+    else if (tmc > TMB / 4)
+        main_loop<TMB, M_KS, N_KS, WG, TMB / 2>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wave, acc);
     else
-        main_loop<M_KS, N_KS, WG, 2>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wave, acc);
+        main_loop<TMB, M_KS, N_KS, WG, TMB / 4>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wave, acc);
 
     // ---- epilogue.  acc[tm][tn][4q+j] = C[m, n] with m = m0 + 32 tm + lane%32 and
-    //      n = n0 + 64 wave + 32 tn + 8 q + 4 (lane/32) + j.  A wave owns a 256 x 64 slab of the tile.
-    //      bf16 results go through the wave's own 32 KiB of LDS (the K loop is done with it) so that
+    //      n = n0 + 64 wave + 32 tn + 8 q + 4 (lane/32) + j.  A wave owns a BM x 64 slab of the tile.
+    //      bf16 results go through the wave's own BM x 128 bytes of LDS (the K loop is done with it) so that
     //      global memory sees whole 128-byte rows: 8 bytes per lane into LDS ([row][8 x 16 B], chunk
     //      ^ (row & 7)), then 16 bytes per lane out, 8 rows per store instruction.  The pre-activation
     //      that GELU' needs comes in the same way, in the opposite direction.
@@ -376,7 +423,7 @@ __global__ __launch_bounds__(Q_THREADS) void gemm256_kernel(const GemmArgs g) {
                 const int n = nw0 + tn * 32 + 8 * q + 4 * h;
                 if (n >= g.N) continue;
 #pragma unroll
-                for (int tm = 0; tm < 8; ++tm) {
+                for (int tm = 0; tm < TMB; ++tm) {
                     const int m = m0 + tm * 32 + lm;
                     if (tm >= tmc || m >= m_ext) continue;
                     *reinterpret_cast<float4 *>((float *)g.C + (crow0 + m) * g.ldc + n) =
@@ -402,7 +449,7 @@ __global__ __launch_bounds__(Q_THREADS) void gemm256_kernel(const GemmArgs g) {
                     if (n < g.N) unpack4(*reinterpret_cast<const uint2 *>((const bf16_t *)g.bias + (long)e * g.N + n), bias);
                 }
 #pragma unroll
-                for (int tm = 0; tm < 8; ++tm) {
+                for (int tm = 0; tm < TMB; ++tm) {
                     if (tm >= tmc) continue;
                     char *cell = slab_at(tm * 32 + lm, tn * 4 + q, h);
                     float v[4];
@@ -444,45 +491,71 @@ __global__ __launch_bounds__(Q_THREADS) void gemm256_kernel(const GemmArgs g) {
     }
 }
 
-template <bool N_KS, bool WG, int EPI>
+template <int TMB, bool N_KS, bool WG, int EPI>
 static int launch256(GemmArgs g, int tiles, hipStream_t st, int kid) {
     if (tiles <= 0) return 0;
     ScopedTiming timing(kid, st);
     g.n_blocks = tiles;
     const int grid = (tiles + 7) & ~7;
-    auto kern = gemm256_kernel<N_KS, WG, EPI>;
+    auto kern = gemm256_kernel<TMB, N_KS, WG, EPI>;
     static bool attr_done = false;
     if (!attr_done) {
-        MOLE_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, Q_NSTAGE * Q_STAGE));
+        MOLE_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, Tile<TMB>::LDS_BYTES));
         attr_done = true;
     }
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(Q_THREADS), Q_NSTAGE * Q_STAGE, st, g);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(Q_THREADS), Tile<TMB>::LDS_BYTES, st, g);
     MOLE_LAUNCH_CHECK();
     return 0;
 }
 
+template <int TMB>
+static int dispatch256(const GemmArgs &g, bool b_ks, bool wg, int epi, int max_rows, hipStream_t st, int kid) {
+    constexpr int BM = Tile<TMB>::BM;
+    const int n_tiles = ceil_div(g.N, Q_BN);
+    if (wg) {
+        const int tiles = g.E * ceil_div(g.M, BM) * n_tiles;
+        if (epi == EPI_WGRAD) return launch256<TMB, true, true, EPI_WGRAD>(g, tiles, st, kid);
+        return -100;
+    }
+    // block slots: worst-case number of heavy m-tiles (each has more than BM/2 rows; rounded to the
+    // 8 XCDs), then at most one light m-tile per expert
+    const int rows_bound = g.offsets ? max_rows : g.single_rows;
+    GemmArgs gg = g;
+    gg.full_blocks = ((rows_bound / (BM / 2)) * n_tiles + 7) & ~7;
+    const int tiles = gg.full_blocks + (g.offsets ? g.E : 1) * n_tiles;
+    if (!b_ks) {
+        if (epi == EPI_BIAS_GELU) return launch256<TMB, false, false, EPI_BIAS_GELU>(gg, tiles, st, kid);
+        if (epi == EPI_DGELU) return launch256<TMB, false, false, EPI_DGELU>(gg, tiles, st, kid);
+        if (epi == EPI_F32) return launch256<TMB, false, false, EPI_F32>(gg, tiles, st, kid);
+    } else {
+        if (epi == EPI_BIAS) return launch256<TMB, true, false, EPI_BIAS>(gg, tiles, st, kid);
+        if (epi == EPI_STORE) return launch256<TMB, true, false, EPI_STORE>(gg, tiles, st, kid);
+    }
+    return -100;
+}
+
+// Tile height per product: 128 rows (two blocks per CU) or 256 rows (one block per CU).
+// MOLE_TMB=4|8 in the environment overrides the choice (tuning aid).
+static int tile_blocks_for(int kid) {
+    static const int forced = [] {
+        const char *v = getenv("MOLE_TMB");
+        return v ? atoi(v) : 0;
+    }();
+    if (forced == 4 || forced == 8) return forced;
+    // the products with a heavy epilogue (GELU, GELU') and the weight gradients gain from two
+    // co-resident blocks that overlap one's epilogue with the other's K loop; the two K = F
+    // products are better off with the larger tile
+    return (kid == MOLE_K_FFN_FWD2 || kid == MOLE_K_FFN_GX) ? 8 : 4;
+}
+
 int launch_gemm256(const GemmArgs &g, bool a_ks, bool b_ks, bool wg, int epi, int max_rows, hipStream_t st, int kid) {
-    // alignment the direct-to-LDS path relies on: 16-byte rows, whole K-steps for row-ragged products
+    // alignment the direct-to-LDS path relies on: 16-byte rows, whole stages of K for row-ragged products
     if (g.lda % 8 || g.ldb % 8 || g.ldc % 8 || g.N % 8) return -100;
     if (!wg && (a_ks || g.K % Q_BK)) return -100;
     if (wg && (!a_ks || !b_ks || g.M % 8)) return -100;
-    const int n_tiles = ceil_div(g.N, Q_BN);
-    if (wg) {
-        const int tiles = g.E * ceil_div(g.M, Q_BM) * n_tiles;
-        if (epi == EPI_WGRAD) return launch256<true, true, EPI_WGRAD>(g, tiles, st, kid);
-        return -100;
-    }
-    const int m_tiles = g.offsets ? max_rows / Q_BM + g.E : ceil_div(g.single_rows, Q_BM);
-    const int tiles = m_tiles * n_tiles;
-    if (!b_ks) {
-        if (epi == EPI_BIAS_GELU) return launch256<false, false, EPI_BIAS_GELU>(g, tiles, st, kid);
-        if (epi == EPI_DGELU) return launch256<false, false, EPI_DGELU>(g, tiles, st, kid);
-        if (epi == EPI_F32) return launch256<false, false, EPI_F32>(g, tiles, st, kid);
-    } else {
-        if (epi == EPI_BIAS) return launch256<true, false, EPI_BIAS>(g, tiles, st, kid);
-        if (epi == EPI_STORE) return launch256<true, false, EPI_STORE>(g, tiles, st, kid);
-    }
-    return -100;
+    const int tmb = tile_blocks_for(kid);
+    if (tmb == 4) return dispatch256<4>(g, b_ks, wg, epi, max_rows, st, kid);
+    return dispatch256<8>(g, b_ks, wg, epi, max_rows, st, kid);
 }
 
 }  // namespace mole
