@@ -105,7 +105,10 @@ __device__ __forceinline__ float fast_d_gelu_exact(float x) {
 // does not store - except along a ragged contraction length, which zero_k_tail() repairs.
 //
 // K-contiguous operand, element (r, k) at p[r*ld + k]: LDS [ROWS][4 x 16 B], the chunk index XORed
-// with (row >> 1) & 3.  Wave w, load i fills LDS bytes [(4i+w)*1024, +1024) = rows 16(4i+w) .. +16.
+// with swz4(row), chosen so that the 16 rows a ds_read_b128 pass touches (and any 8 aligned rows)
+// fall into distinct bank groups of the 64-bank LDS.
+// Wave w, load i fills LDS bytes [(4i+w)*1024, +1024) = rows 16(4i+w) .. +16.
+__device__ __forceinline__ int swz4(int row) { return (((row >> 1) ^ (row >> 3)) & 1) | ((row >> 1) & 2); }
 template <int ROWS>
 __device__ __forceinline__ void load_kc(const bf16_t *p, long ld, int r0, int r_ext, int k0, uint32_t lds) {
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -113,7 +116,7 @@ __device__ __forceinline__ void load_kc(const bf16_t *p, long ld, int r0, int r_
     for (int i = 0; i < ROWS / 64; ++i) {
         const int blk = 4 * i + w;
         const int row = blk * 16 + (lane >> 2);
-        const int c = (lane & 3) ^ ((row >> 1) & 3);
+        const int c = (lane & 3) ^ swz4(row);
         const int r = min(r0 + row, r_ext - 1);
         dma16(p + (long)r * ld + k0 + c * 8, __builtin_amdgcn_readfirstlane(lds + blk * 1024));
     }
@@ -147,7 +150,7 @@ template <int ROWS> __device__ __forceinline__ void zero_k_tail(char *lds, int k
 __device__ __forceinline__ bf16x8 frag_kc(const char *lds, int tb, int kk) {
     const int lane = threadIdx.x & 63;
     const int row = tb * 32 + (lane & 31);
-    const int chunk = (2 * kk + (lane >> 5)) ^ ((row >> 1) & 3);
+    const int chunk = (2 * kk + (lane >> 5)) ^ swz4(row);
     return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4 *>(lds + row * 64 + chunk * 16));
 }
 // ds_read_b64_tr_b16: in a group of 16 lanes, lane 4r+q supplies the address of 4 consecutive values
@@ -393,14 +396,20 @@ __global__ __launch_bounds__(Q_THREADS, Tile<TMB>::BLOCKS_PER_CU) void gemm256_k
     const int jr = lane >> 3, jc = lane & 7;        // row-in-group / 16-byte column of the wide accesses
     const bool col_ok = nw0 + jc * 8 < g.N;
 
+    // 8-byte cell (row, chunk, half): chunk ^ (row >> 1) & 7 and half ^ (row >> 4) & 1 make the 32 rows
+    // one ds_write_b64 pass touches land in 32 distinct 8-byte bank groups
     auto slab_at = [&](int row, int chunk, int half) -> char * {
-        return slab + row * 128 + ((chunk ^ (row & 7)) << 4) + half * 8;
+        return slab + row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4) + ((half ^ (row >> 4)) & 1) * 8;
+    };
+    // a 16-byte access sees the two halves of a chunk swapped on rows with bit 4 set
+    auto fix16 = [&](uint4 v, int row) -> uint4 {
+        return (row & 16) ? make_uint4(v.z, v.w, v.x, v.y) : v;
     };
     // slab -> global: rows [0, live) of the slab, 128 bytes each
     auto flush = [&](bf16_t *dst) {
         for (int it = 0; it * 8 < live; ++it) {
             const int row = it * 8 + jr;
-            const uint4 v = *reinterpret_cast<const uint4 *>(slab_at(row, jc, 0));
+            const uint4 v = fix16(*reinterpret_cast<const uint4 *>(slab_at(row, jc, (row >> 4) & 1)), row);
             if (row < live && col_ok)
                 *reinterpret_cast<uint4 *>(dst + (crow0 + m0 + row) * g.ldc + nw0 + jc * 8) = v;
         }
@@ -411,7 +420,7 @@ __global__ __launch_bounds__(Q_THREADS, Tile<TMB>::BLOCKS_PER_CU) void gemm256_k
             const int row = it * 8 + jr;
             uint4 v = make_uint4(0, 0, 0, 0);
             if (row < live && col_ok) v = *reinterpret_cast<const uint4 *>(src + (crow0 + m0 + row) * g.ldc + nw0 + jc * 8);
-            *reinterpret_cast<uint4 *>(slab_at(row, jc, 0)) = v;
+            *reinterpret_cast<uint4 *>(slab_at(row, jc, (row >> 4) & 1)) = fix16(v, row);
         }
     };
 
