@@ -86,6 +86,12 @@ int mole_softmax_fwd(const float *logits, const float *logit_bias, int S, int E,
                      mole_stream_t stream);
 int mole_gate_bwd(const float *dgates, const float *scores, const int32_t *idx, int S, int E,
                   int k, int normalize_gate, int through_softmax, float *dout, mole_stream_t stream);
+/* Gradient of the gate's Linear (MOLE/utils/Ugate.py:12, run by autograd in the reference):
+ * dwg[E,M] = dlogits[S,E]^T . x[S,M], fp32, summed in a fixed order.  1 <= E <= 32; larger gates use
+ * a library GEMM.  workspace of mole_gate_wgrad_workspace_bytes(S, E, M) bytes. */
+size_t mole_gate_wgrad_workspace_bytes(int S, int E, int M);
+int mole_gate_wgrad(const float *dlogits, const void *x, int dtype, int S, int E, int M, float *dwg,
+                    void *workspace, size_t workspace_bytes, mole_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
  * Routing.  Replaces tutel.impls.fast_dispatch.extract_critical (call site

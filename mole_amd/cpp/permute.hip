@@ -117,6 +117,112 @@ __global__ __launch_bounds__(PM_THREADS) void dispatch_bwd_kernel(const T *__res
     }
 }
 
+// dispatch backward with the gate's input gradient folded in, for small gates (E <= 32): a thread
+// owns 4 columns and keeps its 4 x E slice of Wg in registers; the block walks DB_TOKENS tokens, whose
+// row indices and dlogits are block-uniform (scalar loads).  Larger gates use the kernel above.
+constexpr int DB_TOKENS = 32;
+template <typename T, int EB>
+__global__ __launch_bounds__(256) void dispatch_bwd_gate_kernel(const T *__restrict__ dxd,
+                                                                const int32_t *__restrict__ row, int S, int M, int k,
+                                                                const float *__restrict__ dlogits,
+                                                                const float *__restrict__ wg, int E,
+                                                                T *__restrict__ dx) {
+    const int m = (blockIdx.y * 256 + threadIdx.x) * 4;
+    if (m >= M) return;
+    float w[EB][4];
+#pragma unroll
+    for (int e = 0; e < EB; ++e) {
+        const float4 v = e < E ? *reinterpret_cast<const float4 *>(wg + (size_t)e * M + m) : make_float4(0.f, 0.f, 0.f, 0.f);
+        w[e][0] = v.x; w[e][1] = v.y; w[e][2] = v.z; w[e][3] = v.w;
+    }
+    const int i0 = blockIdx.x * DB_TOKENS, i1 = min(i0 + DB_TOKENS, S);
+    for (int i = i0; i < i1; ++i) {
+        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < k; ++j) {
+            const int r = row[(size_t)j * S + i];
+            if (r < 0) continue;
+            if constexpr (sizeof(T) == 2) {
+                const uint2 v = *reinterpret_cast<const uint2 *>(dxd + (size_t)r * M + m);
+                acc[0] += __uint_as_float(v.x << 16); acc[1] += __uint_as_float(v.x & 0xffff0000u);
+                acc[2] += __uint_as_float(v.y << 16); acc[3] += __uint_as_float(v.y & 0xffff0000u);
+            } else {
+                const float4 v = *reinterpret_cast<const float4 *>(dxd + (size_t)r * M + m);
+                acc[0] += v.x; acc[1] += v.y; acc[2] += v.z; acc[3] += v.w;
+            }
+        }
+        const float *dl = dlogits + (size_t)i * E;
+#pragma unroll
+        for (int e = 0; e < EB; ++e) {
+            const float d = e < E ? dl[e] : 0.f;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) acc[q] += d * w[e][q];
+        }
+        if constexpr (sizeof(T) == 2) {
+            const bf16_t b0 = (bf16_t)acc[0], b1 = (bf16_t)acc[1], b2 = (bf16_t)acc[2], b3 = (bf16_t)acc[3];
+            uint2 o;
+            o.x = (uint32_t)__builtin_bit_cast(uint16_t, b0) | ((uint32_t)__builtin_bit_cast(uint16_t, b1) << 16);
+            o.y = (uint32_t)__builtin_bit_cast(uint16_t, b2) | ((uint32_t)__builtin_bit_cast(uint16_t, b3) << 16);
+            *reinterpret_cast<uint2 *>(dx + (size_t)i * M + m) = o;
+        } else {
+            *reinterpret_cast<float4 *>(dx + (size_t)i * M + m) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+        }
+    }
+}
+
+// Gate weight gradient dWg[e, m] = sum_i dlogits[i, e] * x[i, m] (the Linear backward that
+// autograd runs for MOLETopk, MOLE/utils/Ugate.py:12), in two deterministic passes: blocks of
+// GW_TOKENS tokens write partial [E, M] sums, a second kernel adds the partials in order.
+constexpr int GW_TOKENS = 64;
+template <typename T, int EB>
+__global__ __launch_bounds__(256) void gate_wgrad_partial_kernel(const float *__restrict__ dlogits,
+                                                                 const T *__restrict__ x, int S, int E, int M,
+                                                                 float *__restrict__ part) {
+    const int m = (blockIdx.y * 256 + threadIdx.x) * 4;
+    const int i0 = blockIdx.x * GW_TOKENS;
+    float acc[EB][4];
+#pragma unroll
+    for (int e = 0; e < EB; ++e)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) acc[e][q] = 0.f;
+    if (m < M) {
+        const int i1 = min(i0 + GW_TOKENS, S);
+        for (int i = i0; i < i1; ++i) {
+            float xv[4];
+            if constexpr (sizeof(T) == 2) {
+                const uint2 v = *reinterpret_cast<const uint2 *>(x + (size_t)i * M + m);
+                xv[0] = __uint_as_float(v.x << 16); xv[1] = __uint_as_float(v.x & 0xffff0000u);
+                xv[2] = __uint_as_float(v.y << 16); xv[3] = __uint_as_float(v.y & 0xffff0000u);
+            } else {
+                const float4 v = *reinterpret_cast<const float4 *>(x + (size_t)i * M + m);
+                xv[0] = v.x; xv[1] = v.y; xv[2] = v.z; xv[3] = v.w;
+            }
+            const float *dl = dlogits + (size_t)i * E;
+#pragma unroll
+            for (int e = 0; e < EB; ++e) {
+                const float d = e < E ? dl[e] : 0.f;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) acc[e][q] += d * xv[q];
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < EB; ++e)
+            if (e < E)
+                *reinterpret_cast<float4 *>(part + ((size_t)blockIdx.x * E + e) * M + m) =
+                    make_float4(acc[e][0], acc[e][1], acc[e][2], acc[e][3]);
+    }
+}
+__global__ __launch_bounds__(256) void gate_wgrad_reduce_kernel(const float *__restrict__ part, int nblocks, int EM,
+                                                                float *__restrict__ dwg) {
+    const int idx = (blockIdx.x * 256 + threadIdx.x) * 4;
+    if (idx >= EM) return;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int b = 0; b < nblocks; ++b) {
+        const float4 v = *reinterpret_cast<const float4 *>(part + (size_t)b * EM + idx);
+        acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+    }
+    *reinterpret_cast<float4 *>(dwg + idx) = acc;
+}
+
 template <typename T>
 __global__ __launch_bounds__(PM_THREADS) void combine_fwd_kernel(const T *__restrict__ o,
                                                                  const int32_t *__restrict__ row,
@@ -246,14 +352,63 @@ extern "C" int mole_dispatch_bwd(const void *dxd, int dtype, const int32_t *row,
     MOLE_REQUIRE(dxd && row && dx && aligned16(dxd) && aligned16(dx), "mole_dispatch_bwd: null or misaligned pointer");
     MOLE_REQUIRE(dlogits == nullptr || (wg != nullptr && E >= 1 && aligned16(wg) && M % 4 == 0),
                  "mole_dispatch_bwd: dlogits given without a valid wg/E");
-    const dim3 grid(ceil_div(S, PM_THREADS / WAVE));
     ScopedTiming timing(MOLE_K_DISPATCH_BWD, (hipStream_t)stream);
+    if (dlogits != nullptr && E <= 32 && M % 4 == 0) {
+        const dim3 grid(ceil_div(S, DB_TOKENS), ceil_div(M, 1024));
+        hipStream_t st = (hipStream_t)stream;
+#define MOLE_DB(T, EB) hipLaunchKernelGGL((dispatch_bwd_gate_kernel<T, EB>), grid, dim3(256), 0, st, (const T *)dxd, row, S, M, k, dlogits, wg, E, (T *)dx)
+        if (dtype == MOLE_BF16) {
+            if (E <= 8) MOLE_DB(bf16_t, 8); else if (E <= 16) MOLE_DB(bf16_t, 16); else MOLE_DB(bf16_t, 32);
+        } else {
+            if (E <= 8) MOLE_DB(float, 8); else if (E <= 16) MOLE_DB(float, 16); else MOLE_DB(float, 32);
+        }
+#undef MOLE_DB
+        MOLE_LAUNCH_CHECK();
+        return 0;
+    }
+    const dim3 grid(ceil_div(S, PM_THREADS / WAVE));
     if (dtype == MOLE_BF16)
         hipLaunchKernelGGL(dispatch_bwd_kernel<bf16_t>, grid, dim3(PM_THREADS), 0, (hipStream_t)stream,
                            (const bf16_t *)dxd, row, S, M, k, dlogits, wg, E, (bf16_t *)dx);
     else
         hipLaunchKernelGGL(dispatch_bwd_kernel<float>, grid, dim3(PM_THREADS), 0, (hipStream_t)stream,
                            (const float *)dxd, row, S, M, k, dlogits, wg, E, (float *)dx);
+    MOLE_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" size_t mole_gate_wgrad_workspace_bytes(int S, int E, int M) {
+    if (S <= 0 || E <= 0 || M <= 0) return 0;
+    return (size_t)ceil_div(S, GW_TOKENS) * E * M * sizeof(float);
+}
+
+extern "C" int mole_gate_wgrad(const float *dlogits, const void *x, int dtype, int S, int E, int M, float *dwg,
+                               void *workspace, size_t workspace_bytes, mole_stream_t stream) {
+    MOLE_REQUIRE(dtype == MOLE_F32 || dtype == MOLE_BF16, "mole_gate_wgrad: bad dtype %d", dtype);
+    MOLE_REQUIRE(S >= 0 && E >= 1 && E <= 32 && M > 0 && M % 4 == 0, "mole_gate_wgrad: need 1 <= E <= 32 and M %% 4 == 0 (S=%d E=%d M=%d)", S, E, M);
+    MOLE_REQUIRE(dwg != nullptr, "mole_gate_wgrad: null output");
+    hipStream_t st = (hipStream_t)stream;
+    if (S == 0) {
+        MOLE_HIP(hipMemsetAsync(dwg, 0, (size_t)E * M * sizeof(float), st));
+        return 0;
+    }
+    MOLE_REQUIRE(dlogits && x && workspace && aligned16(x) && aligned16(dwg) && aligned16(workspace), "mole_gate_wgrad: null or misaligned pointer");
+    if (workspace_bytes < mole_gate_wgrad_workspace_bytes(S, E, M)) {
+        set_error("mole_gate_wgrad: workspace of %zu bytes, need %zu", workspace_bytes, mole_gate_wgrad_workspace_bytes(S, E, M));
+        return MOLE_E_WORKSPACE;
+    }
+    const int nb = ceil_div(S, GW_TOKENS);
+    const dim3 grid(nb, ceil_div(M, 1024));
+    float *part = (float *)workspace;
+#define MOLE_GW(T, EB) hipLaunchKernelGGL((gate_wgrad_partial_kernel<T, EB>), grid, dim3(256), 0, st, dlogits, (const T *)x, S, E, M, part)
+    if (dtype == MOLE_BF16) {
+        if (E <= 8) MOLE_GW(bf16_t, 8); else if (E <= 16) MOLE_GW(bf16_t, 16); else MOLE_GW(bf16_t, 32);
+    } else {
+        if (E <= 8) MOLE_GW(float, 8); else if (E <= 16) MOLE_GW(float, 16); else MOLE_GW(float, 32);
+    }
+#undef MOLE_GW
+    MOLE_LAUNCH_CHECK();
+    hipLaunchKernelGGL(gate_wgrad_reduce_kernel, dim3(ceil_div(E * M, 1024)), dim3(256), 0, st, part, nb, E * M, dwg);
     MOLE_LAUNCH_CHECK();
     return 0;
 }

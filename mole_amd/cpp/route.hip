@@ -5,11 +5,11 @@
 // MOLETopk.forward (MOLE/utils/Ugate.py:13).
 //
 // Four launches, all on the caller's stream:
-//   route_topk      256 tokens per block.  A group of G lanes (G = pow2 >= E, at most 64) owns one
+//   route_topk      64 tokens per block (16 per wave).  A group of G lanes (G = pow2 >= E, at most 64) owns one
 //                   token and holds VPL = ceil(E/G) scores per lane; k rounds of a shuffle arg-max
 //                   with the (score desc, index asc) order.  Then, per choice j, the rank of each
 //                   token among the block's earlier tokens with the same expert: wave ballot +
-//                   popcount inside a wave, LDS wave histograms across the four waves.
+//                   popcount over the block's 64 tokens.
 //   route_scan      one wave per (choice, expert): exclusive prefix over the blocks' histograms.
 //   route_finish    one block: per-expert totals, capacity, kept rows, row offsets, l_aux.
 //   route_finalize  loc = base(choice, expert) + block prefix + in-block rank; row = offset + loc.
@@ -21,7 +21,8 @@
 namespace mole {
 
 constexpr int RT_THREADS = 256;
-constexpr int RT_TOKENS = 256;  // tokens per block == threads per block (phase B/C map thread -> token)
+constexpr int RT_TOKENS = 64;   // tokens per block: 16 per wave in the top-k phase, one wave ranks all 64
+constexpr int RT_WTOK = RT_TOKENS / 4;
 constexpr float FP32_EPS = 1.1920928955078125e-07f;
 
 // strict "a ranks above b" of torch.topk: NaN above everything, NaNs equal among themselves
@@ -40,10 +41,10 @@ __global__ __launch_bounds__(RT_THREADS) void route_topk_kernel(
     int32_t *__restrict__ idx, int32_t *__restrict__ lrank, float *__restrict__ gates,
     int32_t *__restrict__ hist /* [k][E][nb] */, float *__restrict__ colsum /* [nb][E] */, int nb) {
     extern __shared__ char smem[];
-    int *s_idx = (int *)smem;                        // [k][256]
-    float *s_graw = (float *)(s_idx + k * RT_TOKENS);  // [k][256]
-    int *s_whist = (int *)(s_graw + k * RT_TOKENS);    // [4][E]
-    float *s_col = (float *)(s_whist + 4 * E);         // [4][E]
+    int *s_idx = (int *)smem;                          // [k][64]
+    float *s_graw = (float *)(s_idx + k * RT_TOKENS);  // [k][64]
+    int *s_hist = (int *)(s_graw + k * RT_TOKENS);     // [E]
+    float *s_col = (float *)(s_hist + E);              // [4][E]
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int b = blockIdx.x, tok0 = b * RT_TOKENS;
@@ -51,15 +52,16 @@ __global__ __launch_bounds__(RT_THREADS) void route_topk_kernel(
     const int tpw = 64 >> logG;  // tokens a wave handles per pass
     const int g = lane & (G - 1), tg = lane >> logG;
 
-    // ---- phase A: top-k of every token -------------------------------------------------------
+    // ---- phase A: top-k of every token (wave w owns tokens 16w .. 16w+15 of the block) ----------
     float colacc[VPL];
 #pragma unroll
     for (int r = 0; r < VPL; ++r) colacc[r] = 0.f;
 
-    for (int it = 0; it < G; ++it) {
-        const int tl = w * 64 + it * tpw + tg;
+    for (int it = 0; it * tpw < RT_WTOK; ++it) {
+        const int tw = it * tpw + tg;                  // token within the wave's 16
+        const int tl = w * RT_WTOK + tw;
         const int token = tok0 + tl;
-        const bool tv = token < S;
+        const bool tv = tw < RT_WTOK && token < S;
         float v[VPL];
         uint64_t taken = 0;
 #pragma unroll
@@ -102,9 +104,9 @@ __global__ __launch_bounds__(RT_THREADS) void route_topk_kernel(
     for (int e = tid; e < E; e += RT_THREADS)
         colsum[(size_t)b * E + e] = ((s_col[e] + s_col[E + e]) + s_col[2 * E + e]) + s_col[3 * E + e];
 
-    // ---- phase B: gate values and indices out --------------------------------------------------
+    // ---- phase B: gate values and indices out (threads 0..63 = the block's tokens) -------------
     const int token = tok0 + tid;
-    const bool tv = token < S;
+    const bool tv = tid < RT_TOKENS && token < S;
     if (tv) {
         float denom = 0.f;
         for (int j = 0; j < k; ++j) denom += s_graw[j * RT_TOKENS + tid];  // left to right, fp32
@@ -117,31 +119,27 @@ __global__ __launch_bounds__(RT_THREADS) void route_topk_kernel(
         }
     }
 
-    // ---- phase C: in-block ranks per choice -----------------------------------------------------
+    // ---- phase C: in-block ranks per choice (wave 0: lane = token) -------------------------------
     const uint64_t lt_mask = (1ull << lane) - 1ull;
     for (int j = 0; j < k; ++j) {
-        for (int e = tid; e < 4 * E; e += RT_THREADS) s_whist[e] = 0;
+        for (int e = tid; e < E; e += RT_THREADS) s_hist[e] = 0;
         __syncthreads();
-        const int e = tv ? s_idx[j * RT_TOKENS + tid] : -1;
-        int rank = 0;
-        uint64_t remaining = __ballot(tv);
-        while (remaining) {
-            const int leader = __ffsll((unsigned long long)remaining) - 1;
-            const int e0 = __shfl(e, leader, WAVE);
-            const uint64_t m = __ballot(tv && e == e0);
-            if (tv && e == e0) rank = __popcll(m & lt_mask);
-            if (lane == leader) s_whist[w * E + e0] = __popcll(m);
-            remaining &= ~m;
+        if (w == 0) {
+            const int e = tv ? s_idx[j * RT_TOKENS + tid] : -1;
+            int rank = 0;
+            uint64_t remaining = __ballot(tv);
+            while (remaining) {
+                const int leader = __ffsll((unsigned long long)remaining) - 1;
+                const int e0 = __shfl(e, leader, WAVE);
+                const uint64_t m = __ballot(tv && e == e0);
+                if (tv && e == e0) rank = __popcll(m & lt_mask);
+                if (lane == leader) s_hist[e0] = __popcll(m);
+                remaining &= ~m;
+            }
+            if (tv) lrank[(size_t)j * S + token] = rank;
         }
         __syncthreads();
-        if (tv) {
-            int base = 0;
-            for (int ww = 0; ww < w; ++ww) base += s_whist[ww * E + e];
-            lrank[(size_t)j * S + token] = base + rank;
-        }
-        for (int e2 = tid; e2 < E; e2 += RT_THREADS)
-            hist[((size_t)j * E + e2) * nb + b] =
-                s_whist[e2] + s_whist[E + e2] + s_whist[2 * E + e2] + s_whist[3 * E + e2];
+        for (int e2 = tid; e2 < E; e2 += RT_THREADS) hist[((size_t)j * E + e2) * nb + b] = s_hist[e2];
         __syncthreads();
     }
 }
@@ -232,12 +230,24 @@ __global__ __launch_bounds__(FIN_THREADS) void route_finish_kernel(
     if (tid == 0) capacity[0] = cap;
 
     if (l_aux != nullptr) {
-        float acc = 0.f;
-        for (int e = tid; e < E; e += FIN_THREADS) {
+        // me[e] = sum over blocks of the partial column sums, in a fixed order: thread (g, e) adds
+        // blocks g, g+groups, ...; thread e then adds the groups in order
+        __syncthreads();
+        const int groups = FIN_THREADS / E > 0 ? FIN_THREADS / E : 1;
+        if (tid < groups * E && E <= FIN_THREADS) {
+            const int e = tid % E, gq = tid / E;
             float me = 0.f;
-            for (int b = 0; b < nb; ++b) me += colsum[(size_t)b * E + e];
-            acc += me * (float)counts[e];
+            for (int b = gq; b < nb; b += groups) me += colsum[(size_t)b * E + e];
+            s_fred[tid] = me;
         }
+        __syncthreads();
+        float acc = 0.f;
+        if (tid < E) {
+            float me = 0.f;
+            for (int gq = 0; gq < groups; ++gq) me += s_fred[gq * E + tid];
+            acc = me * (float)counts[tid];
+        }
+        __syncthreads();
         s_fred[tid] = acc;
         __syncthreads();
         for (int d = FIN_THREADS / 2; d >= 1; d >>= 1) {
@@ -278,7 +288,7 @@ extern "C" size_t mole_route_workspace_bytes(int S, int E, int k) {
 template <int VPL>
 static void launch_topk(const float *scores, int S, int E, int k, int logG, int normalize, int32_t *idx,
                         int32_t *loc, float *gates, int32_t *hist, float *colsum, int nb, hipStream_t st) {
-    const size_t lds = (size_t)k * RT_TOKENS * 8 + (size_t)E * 4 * 8;
+    const size_t lds = (size_t)k * RT_TOKENS * 8 + (size_t)E * 4 + (size_t)E * 4 * 4;
     hipLaunchKernelGGL(route_topk_kernel<VPL>, dim3(nb), dim3(RT_THREADS), lds, st, scores, S, E, k, logG,
                        normalize, idx, loc, gates, hist, colsum, nb);
 }

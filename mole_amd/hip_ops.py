@@ -48,6 +48,22 @@ def gate_bwd(dgates: torch.Tensor, scores: torch.Tensor, idx: torch.Tensor, norm
     return dlogits
 
 
+def gate_wgrad(dlogits: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+    """dWg [E,M] fp32 = dlogits[S,E]^T @ x[S,M].  Small gates (E <= 32) run the deterministic HIP kernel;
+    larger ones are a plain library GEMM (plumbing)."""
+    _dev(dlogits), _dev(x)
+    S, E = dlogits.shape
+    M = x.shape[1]
+    if E > 32 or M % 4 != 0:
+        return (dlogits.t().to(x.dtype) @ x).float()
+    dwg = torch.empty(E, M, dtype=torch.float32, device=x.device)
+    nbytes = L.lib().mole_gate_wgrad_workspace_bytes(S, E, M)
+    ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
+    L.check(L.lib().mole_gate_wgrad(L.ptr(dlogits), L.ptr(x), L.dtype_code(x.dtype), S, E, M, L.ptr(dwg), L.ptr(ws), nbytes,
+                                    L.stream()), "mole_gate_wgrad")
+    return dwg
+
+
 @dataclass
 class Route:
     """Device-side result of mole_route (what tutel's extract_critical returns, plus the ragged

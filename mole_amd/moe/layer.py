@@ -81,7 +81,7 @@ class _FusedMoE(torch.autograd.Function):
         dlogits = H.gate_bwd(dgates, scores, r.idx, m.normalize_gate, through_softmax=True)
         wg32 = wg.detach().float().contiguous()
         dx = H.dispatch_bwd(gxd, r.row, dlogits, wg32)
-        dwg = (dlogits.t().to(x.dtype) @ x).to(wg.dtype)
+        dwg = H.gate_wgrad(dlogits, x).to(wg.dtype)
         return dx, dwg, torch.zeros_like(m.dummy_param), None, None
 
 

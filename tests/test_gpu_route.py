@@ -81,3 +81,16 @@ def test_softmax_and_gate_bwd(S, E):
         idx = torch.from_numpy(np.stack(c.indices_s)).cuda()
         got = H.gate_bwd(dg.cuda(), sc, idx, norm)
         assert rel_err(got, want_dl) < 1e-5
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("S,E,M", [(1, 1, 4), (100, 8, 64), (1000, 16, 1024), (333, 32, 520), (70, 5, 2048)])
+def test_gate_wgrad(S, E, M, dtype):
+    from mole_amd import hip_ops as H
+    print(f"gate_wgrad S={S} E={E} M={M} {dtype}", flush=True)
+    g = torch.Generator().manual_seed(S + E)
+    dl = torch.randn(S, E, generator=g) * 0.1
+    x = torch.randn(S, M, generator=g).to(dtype)
+    got = H.gate_wgrad(dl.cuda(), x.cuda())
+    want = dl.double().t() @ x.double()
+    assert rel_err(got, want) < 1e-5       # fp32 sums of exact products in both dtypes
