@@ -127,6 +127,7 @@ int mole_route(const float *scores, int S, int E, int k, float capacity_factor, 
  *   dispatch_fwd : xd[row[j,i],:] = x[i,:]                      for kept pairs
  *   dispatch_bwd : dx[i,:] = sum_j dxd[row[j,i],:]  (+ dlogits[i,:] . Wg  when dlogits != NULL,
  *                  the gate's contribution to the input gradient, Wg [E,M] fp32)
+ *                  (+ dx_add[i,:] when dx_add != NULL: the same contribution computed beforehand)
  *   combine_fwd  : y[i,:] = sum_j gates[j,i] * o[row[j,i],:]    (zeros for a fully dropped token)
  *   combine_bwd  : d_o[row[j,i],:] = gates[j,i]*dy[i,:];  dgates[j,i] = <dy[i,:], o[row[j,i],:]>
  *                  (0 for dropped pairs)
@@ -137,7 +138,8 @@ int mole_route(const float *scores, int S, int E, int k, float capacity_factor, 
 int mole_dispatch_fwd(const void *x, int dtype, const int32_t *row, int S, int M, int k, void *xd,
                       mole_stream_t stream);
 int mole_dispatch_bwd(const void *dxd, int dtype, const int32_t *row, int S, int M, int k,
-                      const float *dlogits, const float *wg, int E, void *dx, mole_stream_t stream);
+                      const float *dlogits, const float *wg, int E, const void *dx_add, void *dx,
+                      mole_stream_t stream);
 int mole_combine_fwd(const void *o, int dtype, const int32_t *row, const float *gates, int S,
                      int M, int k, void *y, mole_stream_t stream);
 int mole_combine_bwd(const void *dy, const void *o, int dtype, const int32_t *row,
@@ -170,6 +172,10 @@ int mole_ffn_bwd(const void *go, const void *xd, const void *h, const void *a, i
 
 /* Plain GEMMs on the same tiles, used by the gate: c[rows,N] = a[rows,K] . b[N,K]^T  (fp32 out). */
 int mole_gemm_nt(const void *a, const void *b, int dtype, int rows, int N, int K, float *c,
+                 mole_stream_t stream);
+/* c[rows,N] = a[rows,K] . b[K,N], result in `dtype` (the gate's input gradient dlogits . Wg for gates
+ * too large for mole_dispatch_bwd to fold in). */
+int mole_gemm_nn(const void *a, const void *b, int dtype, int rows, int N, int K, void *c,
                  mole_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------

@@ -35,7 +35,7 @@ _SIGNATURES = {
     "mole_route": (c_int, [_P, c_int, c_int, c_int, c_float, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P,
                            _P, _P, c_size_t, _P]),
     "mole_dispatch_fwd": (c_int, [_P, c_int, _P, c_int, c_int, c_int, _P, _P]),
-    "mole_dispatch_bwd": (c_int, [_P, c_int, _P, c_int, c_int, c_int, _P, _P, c_int, _P, _P]),
+    "mole_dispatch_bwd": (c_int, [_P, c_int, _P, c_int, c_int, c_int, _P, _P, c_int, _P, _P, _P]),
     "mole_combine_fwd": (c_int, [_P, c_int, _P, _P, c_int, c_int, c_int, _P, _P]),
     "mole_combine_bwd": (c_int, [_P, _P, c_int, _P, _P, c_int, c_int, c_int, _P, _P, _P]),
     "mole_zero_pad_rows": (c_int, [_P, c_int, _P, _P, c_int, c_int, _P]),
@@ -43,6 +43,7 @@ _SIGNATURES = {
     "mole_ffn_bwd": (c_int, [_P, _P, _P, _P, c_int, _P, _P, c_int, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P,
                              _P, c_int, c_int, _P]),
     "mole_gemm_nt": (c_int, [_P, _P, c_int, c_int, c_int, c_int, _P, _P]),
+    "mole_gemm_nn": (c_int, [_P, _P, c_int, c_int, c_int, c_int, _P, _P]),
     "mole_unimem_create": (c_int, [c_int, c_int, c_int, c_int64, c_int64, POINTER(_P)]),
     "mole_unimem_destroy": (c_int, [_P]),
     "mole_unimem_clear_virtual_mem": (c_int, [_P]),

@@ -542,3 +542,18 @@ extern "C" int mole_gemm_nt(const void *a, const void *b, int dtype, int rows, i
     if (dtype == MOLE_BF16) return run_gemm<bf16_t, false, false, false, EPI_F32>(g, rows, tiles, (hipStream_t)stream, MOLE_K_GEMM_NT);
     return launch_gemm<float, false, false, false, TBM, TBN, EPI_F32>(g, tiles, (hipStream_t)stream, MOLE_K_GEMM_NT);
 }
+
+extern "C" int mole_gemm_nn(const void *a, const void *b, int dtype, int rows, int N, int K, void *c,
+                            mole_stream_t stream) {
+    MOLE_REQUIRE(dtype == MOLE_F32 || dtype == MOLE_BF16, "mole_gemm_nn: bad dtype %d", dtype);
+    const int epc = dtype == MOLE_BF16 ? 8 : 4;
+    MOLE_REQUIRE(rows >= 0 && N > 0 && K > 0 && K % epc == 0 && N % epc == 0, "mole_gemm_nn: bad sizes rows=%d N=%d K=%d", rows, N, K);
+    if (rows == 0) return 0;
+    MOLE_REQUIRE(a && b && c && al16(a) && al16(b) && al16(c), "mole_gemm_nn: null or misaligned pointer");
+    GemmArgs g{};
+    g.single_rows = rows; g.E = 1;
+    g.A = a; g.lda = K; g.B = b; g.ldb = N; g.N = N; g.K = K; g.C = c; g.ldc = N;
+    const int tiles = ceil_div(rows, TBM) * ceil_div(N, TBN);
+    if (dtype == MOLE_BF16) return run_gemm<bf16_t, false, true, false, EPI_STORE>(g, rows, tiles, (hipStream_t)stream, MOLE_K_GEMM_NT);
+    return launch_gemm<float, false, true, false, TBM, TBN, EPI_STORE>(g, tiles, (hipStream_t)stream, MOLE_K_GEMM_NT);
+}

@@ -73,7 +73,7 @@ __global__ __launch_bounds__(PM_THREADS) void dispatch_bwd_kernel(const T *__res
                                                                   const int32_t *__restrict__ row, int S, int M,
                                                                   int k, const float *__restrict__ dlogits,
                                                                   const float *__restrict__ wg, int E,
-                                                                  T *__restrict__ dx) {
+                                                                  const T *__restrict__ dx_add, T *__restrict__ dx) {
     const int i = blockIdx.x * (PM_THREADS / WAVE) + (threadIdx.x >> 6);
     if (i >= S) return;
     const int lane = lane_id();
@@ -96,6 +96,14 @@ __global__ __launch_bounds__(PM_THREADS) void dispatch_bwd_kernel(const T *__res
 #pragma unroll
                 for (int q = 0; q < N; ++q) acc[q] += f[q];
             }
+        }
+        if (dx_add != nullptr) {
+            Vec<T> v;
+            float f[N];
+            v.load(dx_add + (size_t)i * M + (size_t)c * N);
+            v.unpack(f);
+#pragma unroll
+            for (int q = 0; q < N; ++q) acc[q] += f[q];
         }
         if (dlogits != nullptr) {
             for (int e = 0; e < E; ++e) {
@@ -346,14 +354,16 @@ extern "C" int mole_dispatch_fwd(const void *x, int dtype, const int32_t *row, i
 }
 
 extern "C" int mole_dispatch_bwd(const void *dxd, int dtype, const int32_t *row, int S, int M, int k,
-                                 const float *dlogits, const float *wg, int E, void *dx, mole_stream_t stream) {
+                                 const float *dlogits, const float *wg, int E, const void *dx_add, void *dx,
+                                 mole_stream_t stream) {
     if (int rc = check_perm("mole_dispatch_bwd", dtype, S, M, k)) return rc;
     if (S == 0) return 0;
     MOLE_REQUIRE(dxd && row && dx && aligned16(dxd) && aligned16(dx), "mole_dispatch_bwd: null or misaligned pointer");
     MOLE_REQUIRE(dlogits == nullptr || (wg != nullptr && E >= 1 && aligned16(wg) && M % 4 == 0),
                  "mole_dispatch_bwd: dlogits given without a valid wg/E");
     ScopedTiming timing(MOLE_K_DISPATCH_BWD, (hipStream_t)stream);
-    if (dlogits != nullptr && E <= 32 && M % 4 == 0) {
+    MOLE_REQUIRE(dx_add == nullptr || aligned16(dx_add), "mole_dispatch_bwd: misaligned dx_add");
+    if (dlogits != nullptr && dx_add == nullptr && E <= 32 && M % 4 == 0) {
         const dim3 grid(ceil_div(S, DB_TOKENS), ceil_div(M, 1024));
         hipStream_t st = (hipStream_t)stream;
 #define MOLE_DB(T, EB) hipLaunchKernelGGL((dispatch_bwd_gate_kernel<T, EB>), grid, dim3(256), 0, st, (const T *)dxd, row, S, M, k, dlogits, wg, E, (T *)dx)
@@ -369,10 +379,10 @@ extern "C" int mole_dispatch_bwd(const void *dxd, int dtype, const int32_t *row,
     const dim3 grid(ceil_div(S, PM_THREADS / WAVE));
     if (dtype == MOLE_BF16)
         hipLaunchKernelGGL(dispatch_bwd_kernel<bf16_t>, grid, dim3(PM_THREADS), 0, (hipStream_t)stream,
-                           (const bf16_t *)dxd, row, S, M, k, dlogits, wg, E, (bf16_t *)dx);
+                           (const bf16_t *)dxd, row, S, M, k, dlogits, wg, E, (const bf16_t *)dx_add, (bf16_t *)dx);
     else
         hipLaunchKernelGGL(dispatch_bwd_kernel<float>, grid, dim3(PM_THREADS), 0, (hipStream_t)stream,
-                           (const float *)dxd, row, S, M, k, dlogits, wg, E, (float *)dx);
+                           (const float *)dxd, row, S, M, k, dlogits, wg, E, (const float *)dx_add, (float *)dx);
     MOLE_LAUNCH_CHECK();
     return 0;
 }

@@ -28,6 +28,16 @@ def gemm_nt(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
     return c
 
 
+def gemm_nn(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """c[rows,N] = a[rows,K] @ b[K,N] in the operands' dtype."""
+    _dev(a), _dev(b)
+    rows, K = a.shape
+    N = b.shape[1]
+    c = torch.empty(rows, N, dtype=a.dtype, device=a.device)
+    L.check(L.lib().mole_gemm_nn(L.ptr(a), L.ptr(b), L.dtype_code(a.dtype), rows, N, K, L.ptr(c), L.stream()), "mole_gemm_nn")
+    return c
+
+
 def softmax_fwd(logits: torch.Tensor, logit_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     _dev(logits)
     S, E = logits.shape
@@ -122,18 +132,25 @@ def dispatch_fwd(x: torch.Tensor, row: torch.Tensor, total_rows: int, out: Optio
 
 def dispatch_bwd(dxd: torch.Tensor, row: torch.Tensor, dlogits: Optional[torch.Tensor] = None,
                  wg: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """dx = gather-sum of dxd rows (+ dlogits @ wg, the gate's share of the input gradient).  Small gates
+    are folded into the gather kernel; for larger ones the product runs first on the MFMA GEMM."""
     _dev(dxd), _dev(row)
     k, S = row.shape
     M = dxd.shape[-1]
     dx = torch.empty(S, M, dtype=dxd.dtype, device=dxd.device)
     E = 0
+    dx_add = None
     if dlogits is not None:
         _dev(dlogits), _dev(wg)
         E = wg.shape[0]
         if wg.dtype != torch.float32 or dlogits.dtype != torch.float32:
             raise TypeError("gate tensors are fp32")
+        epc = 8 if dxd.dtype == torch.bfloat16 else 4
+        if E > 32 and E % epc == 0 and M % epc == 0:
+            dx_add = gemm_nn(dlogits.to(dxd.dtype), wg.to(dxd.dtype))
+            dlogits, wg, E = None, None, 0
     L.check(L.lib().mole_dispatch_bwd(L.ptr(dxd), L.dtype_code(dxd.dtype), L.ptr(row), S, M, k, L.ptr(dlogits), L.ptr(wg),
-                                      E, L.ptr(dx), L.stream()), "mole_dispatch_bwd")
+                                      E, L.ptr(dx_add), L.ptr(dx), L.stream()), "mole_dispatch_bwd")
     return dx
 
 

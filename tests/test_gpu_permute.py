@@ -12,7 +12,7 @@ pytestmark = pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("ragged", [True, False])
 @pytest.mark.parametrize("S,E,k,cf,M", [(1, 2, 1, 1.0, 8), (300, 8, 2, 1.0, 64), (1000, 16, 1, 0.5, 520),
-                                        (513, 4, 4, 0.0, 1024), (200, 32, 8, 0.0, 2048)])
+                                        (513, 4, 4, 0.0, 1024), (200, 32, 8, 0.0, 2048), (300, 64, 4, 0.0, 256)])
 def test_permutes_match_oracle(S, E, k, cf, M, ragged, dtype):
     from mole_amd import hip_ops as H, _lib as L
     print(f"permute S={S} E={E} k={k} cf={cf} M={M} ragged={ragged} {dtype}", flush=True)
