@@ -28,6 +28,13 @@ WORKLOADS = {
 }
 PEAK_MFMA_TFLOPS = {"bf16": 2500.0, "f32": 157.3}   # MI355X dense peaks
 PEAK_HBM_GBS = 8000.0
+# HBM bytes per launch (read + write) of the grouped GEMMs at workload c2, from rocprofv3 FETCH_SIZE and
+# WRITE_SIZE runs of this script scaled by the same counters' readings for a copy of known size
+# (profiles/bench_c2_hbm_traffic.txt); other workloads have no counter run and report null
+MEASURED_TRAFFIC_BYTES = {
+    "c2": {"ffn_fwd1": 894.3e6, "ffn_fwd2": 464.0e6, "ffn_gw2": 335.7e6, "ffn_da": 854.2e6, "ffn_gw1": 335.7e6,
+           "ffn_gx": 463.8e6},
+}
 
 
 def make_layer(w, seed=0):
@@ -154,7 +161,8 @@ def main():
     peak = PEAK_MFMA_TFLOPS[w["dtype"]]
     gemm_total_us = sum(kernels[n]["avg_us"] for n in gemms)
     roofline = {"bound": "mfma", "kernel": dom, "achieved": kernels[dom]["tflops"], "peak": peak, "unit": "TFLOP/s",
-                "frac": round(kernels[dom]["tflops"] / peak, 4), "traffic": None,
+                "frac": round(kernels[dom]["tflops"] / peak, 4),
+                "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload, {}).get(dom),
                 "all_ffn_gemms_frac": round(6 * gemm_flop / (gemm_total_us * 1e-6) / 1e12 / peak, 4)}
 
     out = {
@@ -163,7 +171,11 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": w["dtype"], "data": "synthetic",
         "config": {"workload": f"{args.workload}: single MoE layer fwd+bwd, S={S} M={M} E={w['E']} top-{k} F={F} "
                                f"capacity_factor={cf}, kept rows R={R}"},
-        "roofline": roofline, "kernels": kernels,
+        "roofline": roofline,
+        "hbm_permutes": {n: {"achieved": kernels[n]["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                             "frac": round(kernels[n]["gbs"] / PEAK_HBM_GBS, 4)}
+                         for n in ("dispatch_fwd", "combine_fwd", "combine_bwd", "dispatch_bwd") if n in kernels},
+        "kernels": kernels,
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w)

@@ -185,50 +185,74 @@ template <typename T, int EB>
 __global__ __launch_bounds__(256) void gate_wgrad_partial_kernel(const float *__restrict__ dlogits,
                                                                  const T *__restrict__ x, int S, int E, int M,
                                                                  float *__restrict__ part) {
-    const int m = (blockIdx.y * 256 + threadIdx.x) * 4;
+    __shared__ __align__(16) float s_dl[GW_TOKENS][EB];
     const int i0 = blockIdx.x * GW_TOKENS;
-    float acc[EB][4];
+    const int nt = min(GW_TOKENS, S - i0);
+    for (int idx = threadIdx.x; idx < GW_TOKENS * EB; idx += 256) {
+        const int t = idx / EB, e = idx % EB;
+        s_dl[t][e] = (t < nt && e < E) ? dlogits[(size_t)(i0 + t) * E + e] : 0.f;
+    }
+    __syncthreads();
+    const int m = (blockIdx.y * 256 + threadIdx.x) * 2;    // two columns per thread
+    if (m >= M) return;
+    float acc[EB][2];
 #pragma unroll
-    for (int e = 0; e < EB; ++e)
+    for (int e = 0; e < EB; ++e) acc[e][0] = acc[e][1] = 0.f;
+    const T *px = x + (size_t)i0 * M + m;
+    for (int t0 = 0; t0 < nt; t0 += 8) {
+        float xv[8][2];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) acc[e][q] = 0.f;
-    if (m < M) {
-        const int i1 = min(i0 + GW_TOKENS, S);
-        for (int i = i0; i < i1; ++i) {
-            float xv[4];
+        for (int u = 0; u < 8; ++u) {       // 8 rows in flight
+            const int t = min(t0 + u, nt - 1);
             if constexpr (sizeof(T) == 2) {
-                const uint2 v = *reinterpret_cast<const uint2 *>(x + (size_t)i * M + m);
-                xv[0] = __uint_as_float(v.x << 16); xv[1] = __uint_as_float(v.x & 0xffff0000u);
-                xv[2] = __uint_as_float(v.y << 16); xv[3] = __uint_as_float(v.y & 0xffff0000u);
+                const uint32_t v = *reinterpret_cast<const uint32_t *>(px + (size_t)t * M);
+                xv[u][0] = __uint_as_float(v << 16); xv[u][1] = __uint_as_float(v & 0xffff0000u);
             } else {
-                const float4 v = *reinterpret_cast<const float4 *>(x + (size_t)i * M + m);
-                xv[0] = v.x; xv[1] = v.y; xv[2] = v.z; xv[3] = v.w;
-            }
-            const float *dl = dlogits + (size_t)i * E;
-#pragma unroll
-            for (int e = 0; e < EB; ++e) {
-                const float d = e < E ? dl[e] : 0.f;
-#pragma unroll
-                for (int q = 0; q < 4; ++q) acc[e][q] += d * xv[q];
+                const float2 v = *reinterpret_cast<const float2 *>(px + (size_t)t * M);
+                xv[u][0] = v.x; xv[u][1] = v.y;
             }
         }
 #pragma unroll
-        for (int e = 0; e < EB; ++e)
-            if (e < E)
-                *reinterpret_cast<float4 *>(part + ((size_t)blockIdx.x * E + e) * M + m) =
-                    make_float4(acc[e][0], acc[e][1], acc[e][2], acc[e][3]);
+        for (int u = 0; u < 8; ++u) {
+            if (t0 + u >= nt) break;
+#pragma unroll
+            for (int e = 0; e < EB; e += 4) {
+                const float4 d = *reinterpret_cast<const float4 *>(&s_dl[t0 + u][e]);   // same address in every lane
+                acc[e][0] += d.x * xv[u][0]; acc[e][1] += d.x * xv[u][1];
+                acc[e + 1][0] += d.y * xv[u][0]; acc[e + 1][1] += d.y * xv[u][1];
+                acc[e + 2][0] += d.z * xv[u][0]; acc[e + 2][1] += d.z * xv[u][1];
+                acc[e + 3][0] += d.w * xv[u][0]; acc[e + 3][1] += d.w * xv[u][1];
+            }
+        }
     }
+#pragma unroll
+    for (int e = 0; e < EB; ++e)
+        if (e < E)
+            *reinterpret_cast<float2 *>(part + ((size_t)blockIdx.x * E + e) * M + m) = make_float2(acc[e][0], acc[e][1]);
 }
+// sums the partials in a fixed order: 4 slices of the block list per output, then the slices in order
 __global__ __launch_bounds__(256) void gate_wgrad_reduce_kernel(const float *__restrict__ part, int nblocks, int EM,
                                                                 float *__restrict__ dwg) {
-    const int idx = (blockIdx.x * 256 + threadIdx.x) * 4;
-    if (idx >= EM) return;
+    __shared__ float4 s_acc[4][64];
+    const int o = threadIdx.x & 63, slice = threadIdx.x >> 6;
+    const int idx = (blockIdx.x * 64 + o) * 4;
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (int b = 0; b < nblocks; ++b) {
-        const float4 v = *reinterpret_cast<const float4 *>(part + (size_t)b * EM + idx);
-        acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+    if (idx < EM) {
+        const int per = (nblocks + 3) / 4;
+        const int b1 = min(nblocks, (slice + 1) * per);
+        for (int b = slice * per; b < b1; ++b) {
+            const float4 v = *reinterpret_cast<const float4 *>(part + (size_t)b * EM + idx);
+            acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+        }
     }
-    *reinterpret_cast<float4 *>(dwg + idx) = acc;
+    s_acc[slice][o] = acc;
+    __syncthreads();
+    if (slice == 0 && idx < EM) {
+        float4 r = s_acc[0][o];
+#pragma unroll
+        for (int sl = 1; sl < 4; ++sl) { r.x += s_acc[sl][o].x; r.y += s_acc[sl][o].y; r.z += s_acc[sl][o].z; r.w += s_acc[sl][o].w; }
+        *reinterpret_cast<float4 *>(dwg + idx) = r;
+    }
 }
 
 template <typename T>
@@ -408,7 +432,7 @@ extern "C" int mole_gate_wgrad(const float *dlogits, const void *x, int dtype, i
         return MOLE_E_WORKSPACE;
     }
     const int nb = ceil_div(S, GW_TOKENS);
-    const dim3 grid(nb, ceil_div(M, 1024));
+    const dim3 grid(nb, ceil_div(M, 512));
     float *part = (float *)workspace;
 #define MOLE_GW(T, EB) hipLaunchKernelGGL((gate_wgrad_partial_kernel<T, EB>), grid, dim3(256), 0, st, dlogits, (const T *)x, S, E, M, part)
     if (dtype == MOLE_BF16) {
@@ -418,7 +442,7 @@ extern "C" int mole_gate_wgrad(const float *dlogits, const void *x, int dtype, i
     }
 #undef MOLE_GW
     MOLE_LAUNCH_CHECK();
-    hipLaunchKernelGGL(gate_wgrad_reduce_kernel, dim3(ceil_div(E * M, 1024)), dim3(256), 0, st, part, nb, E * M, dwg);
+    hipLaunchKernelGGL(gate_wgrad_reduce_kernel, dim3(ceil_div(E * M, 256)), dim3(256), 0, st, part, nb, E * M, dwg);
     MOLE_LAUNCH_CHECK();
     return 0;
 }
