@@ -94,12 +94,91 @@ def cpu_baseline(w, budget_s=12.0):
             "sample": f"{len(times)} steps of the {w['name']} layer shape at {S} tokens, fp32 torch-CPU oracle, median"}
 
 
+def bench_offloaded_stack(args):
+    """BASELINE configuration 4: a stack of MoE layers whose experts all live in pinned host memory and
+    stream through the device slot pool (32 experts of 4096 -> 14336 -> 4096, bf16: 235 MB per expert,
+    7.5 GB per layer; 4096 tokens x 4096, top-2, no drop).  The step is PCIe bound by construction, so
+    the figures of interest are the copy stream's host-to-device rate and how much of the step the
+    copies cover.  --layers sets the depth (12 in the configuration; each layer pins 15 GB of host
+    memory for weights and gradients, the default of 2 keeps set-up within a minute or two)."""
+    import torch
+    from mole_amd import _lib as L, core
+    from mole_amd.moe.layer import MOLEModule
+    S, M, E, k, F = 4096, 4096, 32, 2, 14336
+    n_layers, pool, ebatch = args.layers, 64, 8
+    MOLEModule.reset_instances()
+    dist = {"local_rank": 0, "world_size": 1, "rank": 0}
+    layers = []
+    for i in range(n_layers):
+        print(f"[c4] building layer {i} (pinned host weights)", file=sys.stderr, flush=True)
+        layers.append(MOLEModule(E, 0, M, F, pool, k, ebatch, dist, "gelu", 1, False, True, dtype=torch.bfloat16))
+    for m in layers:
+        m.set_prefetch(E, E)
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(S, M, generator=g).to(torch.bfloat16).cuda().requires_grad_(True)
+    dy = (torch.randn(S, M, generator=g) * 1e-3).to(torch.bfloat16).cuda()
+    um = core.get_UniMem()
+
+    def one_step():
+        layers[0].prefetch_fwd(E)                 # what the scheduler does before the first layer
+        h = x
+        for m in layers:
+            h = m(h, capacity_factor=0.0, prefetch=True)
+        h.backward(dy)
+        x.grad = None
+        for m in layers:
+            m.gate[0].linear.weight.grad = None
+
+    for i in range(args.warmup):
+        print(f"[c4] warm-up step {i}", file=sys.stderr, flush=True)
+        one_step()
+    torch.cuda.synchronize(); core.synchronize_tran()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        print(f"[c4] timed step {i}", file=sys.stderr, flush=True)
+        one_step()
+    torch.cuda.synchronize(); core.synchronize_tran()
+    wall = (time.perf_counter() - t0) / args.steps
+    h2d_bytes, h2d_ms = um.copy_stats()
+    h2d_bytes /= args.steps; h2d_ms /= args.steps
+    d2h_bytes, d2h_ms = um.writeback_stats()
+    d2h_bytes /= args.steps; d2h_ms /= args.steps
+    L.kernel_timing_enable(True)
+    one_step()
+    torch.cuda.synchronize(); core.synchronize_tran()
+    timing = L.kernel_timing_read()
+    L.kernel_timing_enable(False)
+    kernel_ms = sum(ms for _, ms in timing.values())
+    gemm_ms = sum(ms for n, (_, ms) in timing.items() if n.startswith("ffn_") and n != "ffn_gb")
+    R = S * k
+    expert_bytes = (2 * F * M + F + M) * 2
+    out = {
+        "metric": "MoE layer tokens/sec fwd+bwd on 1 MI355X", "value": round(S / wall, 1), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall * 1e3, 2),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"c4: {n_layers}-layer offloaded-expert stack fwd+bwd, S={S} M={M} E={E} top-{k} F={F}, "
+                               f"experts in pinned host memory, pool {pool} slots, chunks of {ebatch} experts"},
+        "prefetch": {"h2d_bytes_per_step": int(h2d_bytes), "h2d_busy_ms": round(h2d_ms, 2),
+                     "h2d_gbs": round(h2d_bytes / (h2d_ms * 1e-3) / 1e9, 2),
+                     "h2d_busy_frac_of_step": round(h2d_ms / (wall * 1e3), 4),
+                     "expected_h2d_bytes": 2 * n_layers * E * expert_bytes,
+                     "d2h_gradient_bytes_per_step": int(d2h_bytes), "d2h_busy_ms": round(d2h_ms, 2),
+                     "d2h_gbs": round(d2h_bytes / (d2h_ms * 1e-3) / 1e9, 2)},
+        "kernel_ms_per_step": round(kernel_ms, 2),
+        "roofline": {"bound": "mfma", "kernel": "all six grouped products", "unit": "TFLOP/s", "peak": 2500.0,
+                     "achieved": round(12.0 * R * M * F * n_layers / (gemm_ms * 1e-3) / 1e12, 1),
+                     "frac": round(12.0 * R * M * F * n_layers / (gemm_ms * 1e-3) / 1e12 / 2500.0, 4), "traffic": None},
+    }
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c4"])
+    ap.add_argument("--layers", type=int, default=2, help="depth of the c4 stack (12 in the configuration)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -110,6 +189,8 @@ def main():
     import torch
     from mole_amd import _lib as L
     assert torch.cuda.is_available(), "bench.py needs an MI355X"
+    if args.workload == "c4":
+        return bench_offloaded_stack(args)
     w = dict(WORKLOADS[args.workload], name=args.workload)
     m, x, dy = make_layer(w)
     cf = w["cf"]

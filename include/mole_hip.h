@@ -220,6 +220,20 @@ int mole_unimem_tran_stream(void *handle, mole_stream_t *out);
  * mole_unimem_sync_tran() calls, measured with events on the copy stream */
 int mole_unimem_copy_stats(void *handle, uint64_t *bytes, float *busy_ms);
 
+/* Gradient write-back of offloaded experts; replaces _MOLECore::store_grad / _CPUParamCore::store_grad
+ * (MOLE/cpp/core.cpp:77-103, MOLE/cpp/uparameter.cpp:68-83) and the "tranback" stream
+ * (MOLE/cpp/stream.cpp:129-134).  dev_src[p] holds the gradients of n experts, [n, ...] contiguous, for
+ * parameter kind p; they are copied to experts [base, base+n) of the pinned host arrays host_dst[p] on a
+ * second library-owned stream once the work already enqueued on compute_stream has finished.  The caller
+ * keeps dev_src alive until that stream has passed the copy (mole_unimem_tranback_stream tells which) and
+ * reads the host arrays only after mole_unimem_sync_tranback().  Overwrites; accumulation is the caller's.
+ * mole_unimem_writeback_stats: bytes and copy time between the two most recent sync_tranback calls. */
+int mole_unimem_store_grads(void *handle, void *const host_dst[4], const void *const dev_src[4], int base,
+                            int n, mole_stream_t compute_stream);
+int mole_unimem_sync_tranback(void *handle);
+int mole_unimem_tranback_stream(void *handle, mole_stream_t *out);
+int mole_unimem_writeback_stats(void *handle, uint64_t *bytes, float *busy_ms);
+
 /* Greedy cross-layer prefetch assignment; replaces fast_assign_prefetch
  * (MOLE/cpp/core.cpp:1302-1345).  lp_out [n]; gp_out holds up to gp_cap triples
  * (from_layer, for_layer, count), *gp_n the number written. */

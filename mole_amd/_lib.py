@@ -58,6 +58,10 @@ _SIGNATURES = {
     "mole_unimem_sync_tran": (c_int, [_P]),
     "mole_unimem_tran_stream": (c_int, [_P, POINTER(_P)]),
     "mole_unimem_copy_stats": (c_int, [_P, POINTER(c_uint64), POINTER(c_float)]),
+    "mole_unimem_store_grads": (c_int, [_P, POINTER(_P), POINTER(_P), c_int, c_int, _P]),
+    "mole_unimem_sync_tranback": (c_int, [_P]),
+    "mole_unimem_tranback_stream": (c_int, [_P, POINTER(_P)]),
+    "mole_unimem_writeback_stats": (c_int, [_P, POINTER(c_uint64), POINTER(c_float)]),
     "mole_fast_assign_prefetch": (c_int, [c_int, POINTER(c_int), POINTER(c_int), c_int, POINTER(c_int),
                                           POINTER(c_int), c_int, POINTER(c_int)]),
 }

@@ -88,6 +88,24 @@ class UniMem:
 
     def sync_tran(self):
         L.check(L.lib().mole_unimem_sync_tran(self._h), "mole_unimem_sync_tran")
+        L.check(L.lib().mole_unimem_sync_tranback(self._h), "mole_unimem_sync_tranback")
+
+    def store_grads(self, host_grads, dev_grads, base: int, n: int):
+        """Device gradients of n experts -> experts [base, base+n) of the pinned host gradient arrays, on the
+        pool's write-back stream, after the compute already enqueued on the current stream."""
+        L.check(L.lib().mole_unimem_store_grads(self._h, self._src(host_grads), self._src(dev_grads), base, n, L.stream()),
+                "mole_unimem_store_grads")
+        out = c_void_p()
+        L.check(L.lib().mole_unimem_tranback_stream(self._h, ctypes.byref(out)), "mole_unimem_tranback_stream")
+        wb = torch.cuda.ExternalStream(int(out.value), device=dev_grads[0].device)
+        for g in dev_grads:           # the allocator must not hand these blocks out again before the copy has run
+            g.record_stream(wb)
+
+    def writeback_stats(self):
+        b, ms = c_uint64(), c_float()
+        L.check(L.lib().mole_unimem_writeback_stats(self._h, ctypes.byref(b), ctypes.byref(ms)),
+                "mole_unimem_writeback_stats")
+        return b.value, ms.value
 
     def tran_stream_handle(self) -> int:
         out = c_void_p()
@@ -332,12 +350,12 @@ class MOLECore:
     def _store_grad(self, host_grads, g, base, size):
         """Gradients of offloaded experts go back to their pinned host buffers (core.cpp:77-103,
         uparameter.cpp:68-83): overwrite, or add when accumulating and the buffer is not lazily zero."""
-        for hg, gg in zip(host_grads, g):
-            dst = hg[base:base + size]
-            if self.acc_step > 1 and not getattr(hg, "lazy_zero", True):
-                dst += gg.to("cpu")
-            else:
-                dst.copy_(gg, non_blocking=True)
+        if self.acc_step > 1 and not getattr(host_grads[0], "lazy_zero", True):
+            get_UniMem().sync_tran()      # an earlier step's overwrite may still be in flight
+            for hg, gg in zip(host_grads, g):
+                hg[base:base + size] += gg.to("cpu")
+        else:
+            get_UniMem().store_grads(host_grads, g, base, size)
 
 
 class BatchFusedFWD(torch.autograd.Function):

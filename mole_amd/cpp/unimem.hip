@@ -21,8 +21,8 @@ struct UniMem {
     int device = 0, pool_size = 0, dtype = 0;
     size_t slot_bytes[4] = {0, 0, 0, 0};
     char *pool[4] = {nullptr, nullptr, nullptr, nullptr};
-    hipStream_t tran = nullptr;
-    hipEvent_t para_event = nullptr;
+    hipStream_t tran = nullptr, tranback = nullptr;
+    hipEvent_t para_event = nullptr, grads_ready = nullptr;
     bool para_recorded = false;
     std::vector<hipEvent_t> slot_event;
     std::vector<char> slot_pending;  // slot_event[s] was recorded and not yet waited on
@@ -33,30 +33,48 @@ struct UniMem {
     size_t timers_used = 0;
     uint64_t bytes_open = 0, bytes_last = 0;
     float ms_last = 0.f;
+    std::vector<std::array<hipEvent_t, 2>> wb_timers;
+    size_t wb_timers_used = 0;
+    uint64_t wb_bytes_open = 0, wb_bytes_last = 0;
+    float wb_ms_last = 0.f;
 };
 
-static int copy_experts(UniMem *u, const void *const host_src[4], int slot0, int base, int n) {
-    if (n <= 0) return 0;
-    for (int s = slot0; s < slot0 + n; ++s)
-        if (u->slot_pending[s]) {
-            MOLE_HIP(hipStreamWaitEvent(u->tran, u->slot_event[s], 0));
-            u->slot_pending[s] = 0;
-        }
+static int next_timer(UniMem *u, std::array<hipEvent_t, 2> **out) {
     if (u->timers_used == u->timers.size()) {
         std::array<hipEvent_t, 2> p;
         MOLE_HIP(hipEventCreate(&p[0]));
         MOLE_HIP(hipEventCreate(&p[1]));
         u->timers.push_back(p);
     }
-    auto &tm = u->timers[u->timers_used++];
-    MOLE_HIP(hipEventRecord(tm[0], u->tran));
-    for (int p = 0; p < 4; ++p) {
-        const size_t sb = u->slot_bytes[p];
-        MOLE_HIP(hipMemcpyAsync(u->pool[p] + (size_t)slot0 * sb, (const char *)host_src[p] + (size_t)base * sb,
-                                (size_t)n * sb, hipMemcpyHostToDevice, u->tran));
-        u->bytes_open += (uint64_t)n * sb;
+    *out = &u->timers[u->timers_used++];
+    return 0;
+}
+
+// Host -> pool copy of experts [base, base+n) into slots [slot0, slot0+n).  The copy is cut at every
+// slot whose previous user has not been waited for yet, so that a prefetch trails the compute that
+// still owns the later slots instead of waiting for all of it.
+static int copy_experts(UniMem *u, const void *const host_src[4], int slot0, int base, int n) {
+    if (n <= 0) return 0;
+    int i = 0;
+    while (i < n) {
+        int run = 1;
+        while (i + run < n && !u->slot_pending[slot0 + i + run]) ++run;
+        if (u->slot_pending[slot0 + i]) {
+            MOLE_HIP(hipStreamWaitEvent(u->tran, u->slot_event[slot0 + i], 0));
+            u->slot_pending[slot0 + i] = 0;
+        }
+        std::array<hipEvent_t, 2> *tm;
+        if (int rc = next_timer(u, &tm)) return rc;
+        MOLE_HIP(hipEventRecord((*tm)[0], u->tran));
+        for (int p = 0; p < 4; ++p) {
+            const size_t sb = u->slot_bytes[p];
+            MOLE_HIP(hipMemcpyAsync(u->pool[p] + (size_t)(slot0 + i) * sb, (const char *)host_src[p] + (size_t)(base + i) * sb,
+                                    (size_t)run * sb, hipMemcpyHostToDevice, u->tran));
+            u->bytes_open += (uint64_t)run * sb;
+        }
+        MOLE_HIP(hipEventRecord((*tm)[1], u->tran));
+        i += run;
     }
-    MOLE_HIP(hipEventRecord(tm[1], u->tran));
     MOLE_HIP(hipEventRecord(u->para_event, u->tran));
     u->para_recorded = true;
     return 0;
@@ -97,7 +115,9 @@ extern "C" int mole_unimem_create(int device, int pool_size, int dtype, int64_t 
         }
     }
     MOLE_HIP(hipStreamCreateWithFlags(&u->tran, hipStreamNonBlocking));
+    MOLE_HIP(hipStreamCreateWithFlags(&u->tranback, hipStreamNonBlocking));
     MOLE_HIP(hipEventCreateWithFlags(&u->para_event, hipEventDisableTiming));
+    MOLE_HIP(hipEventCreateWithFlags(&u->grads_ready, hipEventDisableTiming));
     u->slot_event.resize(pool_size);
     u->slot_pending.assign(pool_size, 0);
     for (int s = 0; s < pool_size; ++s) MOLE_HIP(hipEventCreateWithFlags(&u->slot_event[s], hipEventDisableTiming));
@@ -109,10 +129,14 @@ extern "C" int mole_unimem_destroy(void *handle) {
     UM(handle);
     (void)hipSetDevice(u->device);
     (void)hipStreamSynchronize(u->tran);
+    (void)hipStreamSynchronize(u->tranback);
     for (auto &e : u->slot_event) (void)hipEventDestroy(e);
     for (auto &t : u->timers) { (void)hipEventDestroy(t[0]); (void)hipEventDestroy(t[1]); }
+    for (auto &t : u->wb_timers) { (void)hipEventDestroy(t[0]); (void)hipEventDestroy(t[1]); }
     (void)hipEventDestroy(u->para_event);
+    (void)hipEventDestroy(u->grads_ready);
     (void)hipStreamDestroy(u->tran);
+    (void)hipStreamDestroy(u->tranback);
     for (int p = 0; p < 4; ++p)
         if (u->pool[p]) (void)hipFree(u->pool[p]);
     delete u;
@@ -222,6 +246,62 @@ extern "C" int mole_unimem_sync_tran(void *handle) {
     u->bytes_last = u->bytes_open;
     u->bytes_open = 0;
     u->timers_used = 0;
+    return 0;
+}
+
+extern "C" int mole_unimem_store_grads(void *handle, void *const host_dst[4], const void *const dev_src[4], int base,
+                                       int n, mole_stream_t compute_stream) {
+    UM(handle);
+    MOLE_REQUIRE(host_dst && dev_src && base >= 0 && n >= 0, "mole_unimem_store_grads: bad arguments base=%d n=%d", base, n);
+    if (n == 0) return 0;
+    for (int p = 0; p < 4; ++p)
+        MOLE_REQUIRE(host_dst[p] && dev_src[p], "mole_unimem_store_grads: null buffer for parameter kind %d", p);
+    MOLE_HIP(hipEventRecord(u->grads_ready, (hipStream_t)compute_stream));
+    MOLE_HIP(hipStreamWaitEvent(u->tranback, u->grads_ready, 0));
+    if (u->wb_timers_used == u->wb_timers.size()) {
+        std::array<hipEvent_t, 2> p;
+        MOLE_HIP(hipEventCreate(&p[0]));
+        MOLE_HIP(hipEventCreate(&p[1]));
+        u->wb_timers.push_back(p);
+    }
+    auto &tm = u->wb_timers[u->wb_timers_used++];
+    MOLE_HIP(hipEventRecord(tm[0], u->tranback));
+    for (int p = 0; p < 4; ++p) {
+        const size_t sb = u->slot_bytes[p];
+        MOLE_HIP(hipMemcpyAsync((char *)host_dst[p] + (size_t)base * sb, dev_src[p], (size_t)n * sb, hipMemcpyDeviceToHost,
+                                u->tranback));
+        u->wb_bytes_open += (uint64_t)n * sb;
+    }
+    MOLE_HIP(hipEventRecord(tm[1], u->tranback));
+    return 0;
+}
+
+extern "C" int mole_unimem_sync_tranback(void *handle) {
+    UM(handle);
+    MOLE_HIP(hipStreamSynchronize(u->tranback));
+    float total = 0.f;
+    for (size_t i = 0; i < u->wb_timers_used; ++i) {
+        float ms = 0.f;
+        MOLE_HIP(hipEventElapsedTime(&ms, u->wb_timers[i][0], u->wb_timers[i][1]));
+        total += ms;
+    }
+    u->wb_ms_last = total;
+    u->wb_bytes_last = u->wb_bytes_open;
+    u->wb_bytes_open = 0;
+    u->wb_timers_used = 0;
+    return 0;
+}
+
+extern "C" int mole_unimem_tranback_stream(void *handle, mole_stream_t *out) {
+    UM(handle);
+    *out = (mole_stream_t)u->tranback;
+    return 0;
+}
+
+extern "C" int mole_unimem_writeback_stats(void *handle, uint64_t *bytes, float *busy_ms) {
+    UM(handle);
+    if (bytes) *bytes = u->wb_bytes_last;
+    if (busy_ms) *busy_ms = u->wb_ms_last;
     return 0;
 }
 
