@@ -19,6 +19,8 @@
 
 #include <stdlib.h>
 
+#include <type_traits>
+
 namespace mole {
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -51,6 +53,16 @@ constexpr int waitcnt_vm(int n) { return (n & 0xf) | ((n >> 4) << 14) | 0x0070 |
 // reserved by the compiler and nothing else in these kernels uses it.
 __device__ __forceinline__ void dma16(const void *gptr, uint32_t lds_off) {
     asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(gptr), "s"(lds_off) : "memory");
+}
+// The same with the address split into a wave-uniform 64-bit base (SGPR pair) and a 32-bit per-lane byte
+// offset: the K loop then advances the base with scalar adds and spends no VALU work on addresses.
+__device__ __forceinline__ void dma16s(const void *sbase, uint32_t voff, uint32_t lds_off) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(voff), "s"(sbase), "s"(lds_off) : "memory");
+}
+__device__ __forceinline__ const char *uniform_ptr(const void *p) {   // tell the compiler the pointer is wave-uniform
+    const uint64_t v = (uint64_t)p;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (const char *)(((uint64_t)hi << 32) | lo);
 }
 __device__ __forceinline__ uint32_t lds_offset_of(const char *p) {
     return (uint32_t)(size_t)(__attribute__((address_space(3))) const char *)p;
@@ -109,37 +121,43 @@ __device__ __forceinline__ float fast_d_gelu_exact(float x) {
 // fall into distinct bank groups of the 64-bank LDS.
 // Wave w, load i fills LDS bytes [(4i+w)*1024, +1024) = rows 16(4i+w) .. +16.
 __device__ __forceinline__ int swz4(int row) { return (((row >> 1) ^ (row >> 3)) & 1) | ((row >> 1) & 2); }
-template <int ROWS>
-__device__ __forceinline__ void load_kc(const bf16_t *p, long ld, int r0, int r_ext, int k0, uint32_t lds) {
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+// Per-lane byte offsets of the ROWS/64 loads a wave issues for one stage of an operand tile, relative to
+// the tile's first element at the stage's first k (what the scalar base points at).  r_left = rows of the
+// operand from the tile's first row on, k_left = k-rows from the stage's first k on (only the last stage
+// of a ragged contraction has fewer than 32).
+template <int ROWS> struct OffKC {
+    uint32_t off[ROWS / 64];
+    __device__ __forceinline__ void init(long ld, int r_left) {
+        const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
 #pragma unroll
-    for (int i = 0; i < ROWS / 64; ++i) {
-        const int blk = 4 * i + w;
-        const int row = blk * 16 + (lane >> 2);
-        const int c = (lane & 3) ^ swz4(row);
-        const int r = min(r0 + row, r_ext - 1);
-        dma16(p + (long)r * ld + k0 + c * 8, __builtin_amdgcn_readfirstlane(lds + blk * 1024));
+        for (int i = 0; i < ROWS / 64; ++i) {
+            const int row = (4 * i + w) * 16 + (lane >> 2);
+            const int c = (lane & 3) ^ swz4(row);
+            off[i] = (uint32_t)(min(row, r_left - 1) * ld * 2 + c * 16);
+        }
     }
-}
+};
 // K-strided operand, element (r, k) at p[k*ld + r]: LDS [32 k][ROWS x 2 B] as it lies in HBM, the
 // 32-byte granule index XORed with (k & 3) << 1 (conflict-free transpose reads, see frag_ks).
 // A k-row has ROWS/8 slots of 16 bytes; a wave load of 1 KiB covers 512/ROWS k-rows.
-template <int ROWS>
-__device__ __forceinline__ void load_ks(const bf16_t *p, long ld, int r0, int r_ext, int k0, int k_ext, uint32_t lds) {
-    constexpr int SPR = ROWS / 8;          // 16-byte slots per k-row
-    constexpr int KPL = 64 / SPR;          // k-rows per wave load
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+template <int ROWS> struct OffKS {
+    uint32_t off[ROWS / 64];
+    __device__ __forceinline__ void init(long ld, int r_left, int k_left) {
+        constexpr int SPR = ROWS / 8;          // 16-byte slots per k-row
+        constexpr int KPL = 64 / SPR;          // k-rows per wave load
+        const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
 #pragma unroll
-    for (int i = 0; i < ROWS / 64; ++i) {
-        const int blk = 4 * i + w;
-        const int kr = blk * KPL + lane / SPR;
-        const int pc = lane % SPR;                                        // physical 16-byte slot in the k-row
-        const int c = ((((pc >> 1) ^ ((kr & 3) << 1)) << 1) | (pc & 1));  // logical 16-byte chunk
-        const int k = min(k0 + kr, k_ext - 1);
-        const int r = min(r0 + c * 8, r_ext - 8);
-        dma16(p + (long)k * ld + r, __builtin_amdgcn_readfirstlane(lds + blk * 1024));
+        for (int i = 0; i < ROWS / 64; ++i) {
+            const int kr = (4 * i + w) * KPL + lane / SPR;
+            const int pc = lane % SPR;                                        // physical 16-byte slot in the k-row
+            const int c = ((((pc >> 1) ^ ((kr & 3) << 1)) << 1) | (pc & 1));  // logical 16-byte chunk
+            off[i] = (uint32_t)(min(kr, k_left - 1) * ld * 2 + min(c * 8, r_left - 8) * 2);
+        }
     }
-}
+};
+template <int ROWS, bool KS> struct Off;
+template <int ROWS> struct Off<ROWS, false> : OffKC<ROWS> {};
+template <int ROWS> struct Off<ROWS, true> : OffKS<ROWS> {};
 // zero the k-rows [k_valid, 32) of a K-strided tile (the last, partial stage of a weight gradient)
 template <int ROWS> __device__ __forceinline__ void zero_k_tail(char *lds, int k_valid) {
     for (int idx = threadIdx.x; idx < (Q_BK - k_valid) * (ROWS / 8); idx += Q_THREADS)
@@ -171,55 +189,98 @@ template <bool KS, int ROWS> __device__ __forceinline__ bf16x8 frag(const char *
     if constexpr (KS) return frag_ks<ROWS>(lds, tb, kk); else return frag_kc(lds, tb, kk);
 }
 
+// first index of part P when N items are dealt to NP consecutive parts
+template <int P, int NP, int N> constexpr int part_lo() { return P * N / NP; }
+
 template <int TMB, bool M_KS, bool N_KS, int TMC> struct Frags {
     bf16x8 m[TMC], n[2];
-    __device__ __forceinline__ void read(const char *stage, int wave, int kk) {
+    // the TMC + 2 fragment reads of a k-sub-step, n-side first, dealt to NP parts
+    template <int P, int NP> __device__ __forceinline__ void read_part(const char *stage, int wave, int kk) {
 #pragma unroll
-        for (int tm = 0; tm < TMC; ++tm) m[tm] = frag<M_KS, Tile<TMB>::BM>(stage, tm, kk);
-#pragma unroll
-        for (int tn = 0; tn < 2; ++tn) n[tn] = frag<N_KS, Q_BN>(stage + Tile<TMB>::M_OPERAND, wave * 2 + tn, kk);
+        for (int r = part_lo<P, NP, TMC + 2>(); r < part_lo<P + 1, NP, TMC + 2>(); ++r) {
+            if (r < 2) n[r] = frag<N_KS, Q_BN>(stage + Tile<TMB>::M_OPERAND, wave * 2 + r, kk);
+            else m[r - 2] = frag<M_KS, Tile<TMB>::BM>(stage, r - 2, kk);
+        }
     }
-    __device__ __forceinline__ void mma(f32x16 (&acc)[TMB][2]) const {
+    __device__ __forceinline__ void read(const char *stage, int wave, int kk) { read_part<0, 1>(stage, wave, kk); }
+    // the 2 TMC MFMAs of a k-sub-step dealt to NP parts
+    template <int P, int NP> __device__ __forceinline__ void mma_part(f32x16 (&acc)[TMB][2]) const {
 #pragma unroll
-        for (int tm = 0; tm < TMC; ++tm)
-#pragma unroll
-            for (int tn = 0; tn < 2; ++tn)
-                acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(n[tn], m[tm], acc[tm][tn], 0, 0, 0);
+        for (int i = part_lo<P, NP, 2 * TMC>(); i < part_lo<P + 1, NP, 2 * TMC>(); ++i)
+            acc[i >> 1][i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(n[i & 1], m[i >> 1], acc[i >> 1][i & 1], 0, 0, 0);
     }
 };
 
-// interleave hint for a phase of MFMAS MFMAs: one MFMA, then up to two LDS reads and one global load
-template <int MFMAS> __device__ __forceinline__ void interleave() {
-#pragma unroll
-    for (int i = 0; i < MFMAS; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // LDS read
-        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // global load
+// Issues the asynchronous loads of the operand stages of one tile.  The two operand tiles are addressed
+// by a scalar base (advanced by one stage of K after a stage's last load) plus per-lane offsets that stay
+// fixed for the whole K loop.  Stages are fetched in order; past the last one the last is fetched again,
+// harmlessly: it keeps the number of loads per stage, which the vmcnt arithmetic of the loop relies on.
+template <int TMB, bool M_KS, bool N_KS, bool WG> struct Feeder {
+    typedef Tile<TMB> TL;
+    static constexpr int LM = TL::BM / 64, L = TL::LOADS;
+    Off<TL::BM, M_KS> om, cm;
+    Off<Q_BN, N_KS> on, cn;
+    const char *bm, *bn;
+    long step_m, step_n;
+    uint32_t lds_w;      // LDS address of ring buffer 0 + this wave's 1 KiB lane
+    int nk;
+    bool ragged_k;
+    __device__ __forceinline__ void init(const bf16_t *Mp, long ldm, int m0, int m_ext, const bf16_t *Np, long ldn, int n0,
+                                         int n_ext, int k_ext, char *smem, int wave) {
+        if constexpr (M_KS) om.init(ldm, m_ext - m0, Q_BK); else om.init(ldm, m_ext - m0);
+        if constexpr (N_KS) on.init(ldn, n_ext - n0, Q_BK); else on.init(ldn, n_ext - n0);
+        ragged_k = WG && (k_ext & (Q_BK - 1));
+        if constexpr (WG) {   // last stage of a ragged contraction: k-rows past the end are clamped to the last one
+            cm.init(ldm, m_ext - m0, ragged_k ? (k_ext & (Q_BK - 1)) : Q_BK);
+            cn.init(ldn, n_ext - n0, ragged_k ? (k_ext & (Q_BK - 1)) : Q_BK);
+        }
+        bm = uniform_ptr(M_KS ? Mp + m0 : Mp + (long)m0 * ldm);
+        bn = uniform_ptr(N_KS ? Np + n0 : Np + (long)n0 * ldn);
+        step_m = M_KS ? ldm * (Q_BK * 2) : Q_BK * 2;
+        step_n = N_KS ? ldn * (Q_BK * 2) : Q_BK * 2;
+        lds_w = lds_offset_of(smem) + __builtin_amdgcn_readfirstlane(wave * 1024);
+        nk = (k_ext + Q_BK - 1) / Q_BK;
     }
-}
+    // loads [J0, J1) of stage s (the m-side tile's loads come first) into ring buffer buf
+    template <int J0, int J1> __device__ __forceinline__ void issue(int s, int buf) {
+        const uint32_t dst = lds_w + buf * TL::STAGE;
+        const bool clamp_k = WG && ragged_k && s >= nk - 1;
+#pragma unroll
+        for (int j = J0; j < J1; ++j) {
+            if (j < LM) {
+                uint32_t o = om.off[j];
+                if constexpr (WG) o = clamp_k ? cm.off[j] : o;
+                dma16s(bm, o, dst + j * 4096);
+            } else {
+                uint32_t o = on.off[j - LM];
+                if constexpr (WG) o = clamp_k ? cn.off[j - LM] : o;
+                dma16s(bn, o, dst + TL::M_OPERAND + (j - LM) * 4096);
+            }
+        }
+        if (J1 == L && s + 1 < nk) { bm += step_m; bn += step_n; }
+    }
+};
 
-// The K loop.  Stage s (32 of K) lives in ring buffer s mod NSTAGE; its loads were issued NSTAGE-1
-// stages earlier.  Per stage: MFMAs of k-sub-step 0 while the fragments of sub-step 1 are read; then
-// the only synchronisation point - wait until this wave's share of stage s+1 has landed (newer
-// stages may still be in flight), barrier, issue the loads of stage s+NSTAGE-1 into the buffer
-// everyone has just left - and the MFMAs of sub-step 1 while the first fragments of stage s+1 are read.
+// The K loop.  Stage s (32 of K) lives in ring buffer s mod NSTAGE and is fetched NSTAGE-1 stages ahead.
+// A wave cannot issue MFMAs while one of its loads waits for the memory pipeline to take it, so the loads
+// of a stage are not issued in one burst: each half of an iteration is cut into parts, and a part issues
+// its share of the loads, then its share of the fragment reads for the next sub-step, then its MFMAs.
+// The second half of iteration s issues the first half of the loads of stage s+AHEAD, the first half of
+// iteration s+1 the rest, into the buffer that stage s-1 has left.  One synchronisation point per
+// iteration, between the halves: wait until this wave's share of stage s+1 has landed (newer stages may
+// still be in flight), then the barrier.
 template <int TMB, bool M_KS, bool N_KS, bool WG, int TMC>
 __device__ __forceinline__ void main_loop(const bf16_t *Mp, long ldm, int m0, int m_ext, const bf16_t *Np, long ldn,
                                           int n0, int n_ext, int k_ext, char *smem, int wave, f32x16 (&acc)[TMB][2]) {
     typedef Tile<TMB> TL;
-    constexpr int AHEAD = TL::NSTAGE - 1;
+    constexpr int AHEAD = TL::NSTAGE - 1, NP = 4;
+    constexpr int L = TL::LOADS, LH = L / 2;
+    static_assert(L % 2 == 0, "a stage's loads are issued in two halves");
     const int nk = (k_ext + Q_BK - 1) / Q_BK;
     if (nk == 0) return;
-    const uint32_t lds0 = lds_offset_of(smem);
-    auto issue = [&](int s, int buf) {   // stage index is clamped: past the end the last stage is fetched again, harmlessly
-        const uint32_t dst = lds0 + buf * TL::STAGE;
-        const int k0 = min(s, nk - 1) * Q_BK;
-        if constexpr (M_KS) load_ks<TL::BM>(Mp, ldm, m0, m_ext, k0, k_ext, dst);
-        else load_kc<TL::BM>(Mp, ldm, m0, m_ext, k0, dst);
-        if constexpr (N_KS) load_ks<Q_BN>(Np, ldn, n0, n_ext, k0, k_ext, dst + TL::M_OPERAND);
-        else load_kc<Q_BN>(Np, ldn, n0, n_ext, k0, dst + TL::M_OPERAND);
-    };
-    auto fix_tail = [&](int s, int buf) {   // ragged contraction: zero what lies past it in the last stage
+    Feeder<TMB, M_KS, N_KS, WG> fd;
+    fd.init(Mp, ldm, m0, m_ext, Np, ldn, n0, n_ext, k_ext, smem, wave);
+    auto fix_tail = [&](int s, int buf) __attribute__((always_inline)) {   // ragged contraction: zero what lies past it in the last stage
         if (WG && s == nk - 1 && (k_ext & (Q_BK - 1))) {
             char *b = smem + buf * TL::STAGE;
             zero_k_tail<TL::BM>(b, k_ext & (Q_BK - 1));
@@ -227,9 +288,13 @@ __device__ __forceinline__ void main_loop(const bf16_t *Mp, long ldm, int m0, in
             __syncthreads();
         }
     };
+    // SPLIT: with three or more stages in flight a stage's loads are spread over two halves (one iteration
+    // of look-ahead is lost for the later half); with two, all of them go into the half after the barrier.
+    constexpr bool SPLIT = AHEAD >= 3;
 #pragma unroll
-    for (int s = 0; s < AHEAD; ++s) issue(s, s);
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm((AHEAD - 1) * TL::LOADS));
+    for (int s = 0; s < AHEAD - 1; ++s) fd.template issue<0, L>(s, s);
+    fd.template issue<0, SPLIT ? LH : L>(AHEAD - 1, AHEAD - 1);
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm((AHEAD - 2) * L + (SPLIT ? LH : L)));
     __builtin_amdgcn_s_barrier();
     fix_tail(0, 0);
     Frags<TMB, M_KS, N_KS, TMC> f0, f1;
@@ -238,21 +303,27 @@ __device__ __forceinline__ void main_loop(const bf16_t *Mp, long ldm, int m0, in
     for (int s = 0; s < nk; ++s) {
         const int nxt_b = cur_b + 1 == TL::NSTAGE ? 0 : cur_b + 1;
         const int free_b = cur_b == 0 ? TL::NSTAGE - 1 : cur_b - 1;     // held stage s-1, takes stage s+AHEAD
+        const int fill_b = free_b == 0 ? TL::NSTAGE - 1 : free_b - 1;   // takes the rest of stage s+AHEAD-1
         const char *cur = smem + cur_b * TL::STAGE;
         const char *nxt = smem + nxt_b * TL::STAGE;
-        f1.read(cur, wave, 1);
-        f0.mma(acc);
-        interleave<2 * TMC>();
+#define MOLE_HALF(P, J0, N, S_LOAD, BUF, FR, STAGE_PTR, KK, FM)                                           \
+        fd.template issue<(J0) + part_lo<P, NP, (N)>(), (J0) + part_lo<P + 1, NP, (N)>()>(S_LOAD, BUF);   \
+        FR.template read_part<P, NP>(STAGE_PTR, wave, KK);                                                \
+        FM.template mma_part<P, NP>(acc);                                                                 \
         __builtin_amdgcn_sched_barrier(0);
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm((AHEAD - 2) * TL::LOADS));
+        MOLE_HALF(0, SPLIT ? LH : 0, SPLIT ? LH : 0, s + AHEAD - 1, fill_b, f1, cur, 1, f0)
+        MOLE_HALF(1, SPLIT ? LH : 0, SPLIT ? LH : 0, s + AHEAD - 1, fill_b, f1, cur, 1, f0)
+        MOLE_HALF(2, SPLIT ? LH : 0, SPLIT ? LH : 0, s + AHEAD - 1, fill_b, f1, cur, 1, f0)
+        MOLE_HALF(3, SPLIT ? LH : 0, SPLIT ? LH : 0, s + AHEAD - 1, fill_b, f1, cur, 1, f0)
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm((AHEAD - 2) * L));
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
-        issue(s + AHEAD, free_b);
         fix_tail(s + 1, nxt_b);
-        f0.read(nxt, wave, 0);
-        f1.mma(acc);
-        interleave<2 * TMC>();
-        __builtin_amdgcn_sched_barrier(0);
+        MOLE_HALF(0, 0, SPLIT ? LH : L, s + AHEAD, free_b, f0, nxt, 0, f1)
+        MOLE_HALF(1, 0, SPLIT ? LH : L, s + AHEAD, free_b, f0, nxt, 0, f1)
+        MOLE_HALF(2, 0, SPLIT ? LH : L, s + AHEAD, free_b, f0, nxt, 0, f1)
+        MOLE_HALF(3, 0, SPLIT ? LH : L, s + AHEAD, free_b, f0, nxt, 0, f1)
+#undef MOLE_HALF
         cur_b = nxt_b;
     }
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));   // nothing may still be writing LDS when the block retires
@@ -358,6 +429,14 @@ __global__ __launch_bounds__(Q_THREADS, Tile<TMB>::BLOCKS_PER_CU) void gemm256_k
         k_ext = g.kept ? g.kept[e] : g.single_rows;
         row0 = g.offsets ? g.offsets[e] : 0;
     }
+    // the tile's coordinates are the same in every lane: say so, so that everything derived from them
+    // (operand bases, LDS destinations, loop bounds) lives in scalar registers
+    e = __builtin_amdgcn_readfirstlane(e);
+    mt = __builtin_amdgcn_readfirstlane(mt);
+    nt = __builtin_amdgcn_readfirstlane(nt);
+    m_ext = __builtin_amdgcn_readfirstlane(m_ext);
+    k_ext = __builtin_amdgcn_readfirstlane(k_ext);
+    row0 = ((long)__builtin_amdgcn_readfirstlane((int)(row0 >> 32)) << 32) | (unsigned)__builtin_amdgcn_readfirstlane((int)row0);
     const int m0 = mt * Q_BM, n0 = nt * Q_BN;
     const bf16_t *Mp = (const bf16_t *)g.A + row0 * g.lda;
     const bf16_t *Np = WG ? (const bf16_t *)g.B + row0 * g.ldb : (const bf16_t *)g.B + (long)e * g.strideB;
