@@ -340,130 +340,29 @@ __device__ __forceinline__ void unpack4(uint2 u, float *f) {
     f[3] = __uint_as_float(u.y & 0xffff0000u);
 }
 
-// Row-ragged (!WG): C[rows_e, N] = Mop[rows_e, K] . Nop_e ; Mop K-contiguous, Nop_e [N,K] or (N_KS) [K,N].
-// Weight gradient (WG): C_e[M, N] = sum_{r in rows_e} Mop[r, M]^T . Nop[r, N], both K-strided.
-template <int TMB, bool N_KS, bool WG, int EPI>
-__global__ __launch_bounds__(Q_THREADS, Tile<TMB>::BLOCKS_PER_CU) void gemm256_kernel(const GemmArgs g) {
-    constexpr bool M_KS = WG;
-    constexpr int Q_BM = Tile<TMB>::BM;
-    extern __shared__ __align__(16) char smem[];
-    // ---- which tile am I?  Blocks are dealt round-robin to the 8 XCDs (block b runs on XCD b mod 8):
-    //      give each XCD a contiguous range of the REAL tiles, so that neighbours share operands in
-    //      its L2 and every XCD gets the same share.  For row-ragged products the number of real
-    //      tiles is only known here (the grid is sized for the worst case), hence the device-side sum.
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int n_tiles = (g.N + Q_BN - 1) / Q_BN;
-    int e, mt, nt, m_ext, k_ext;
-    long row0;  // first row of the expert
-    if constexpr (!WG) {
-        // Heavy m-tiles (more than BM/2 live rows) take the first g.full_blocks block slots, in
-        // contiguous per-XCD ranges; the light ones (an expert's last tile with at most BM/2 rows)
-        // take the slots after them in plain order.  The hardware starts blocks in index order, so
-        // the short tiles fill the end of the launch instead of holding CUs for a full tile's time.
-        const bool single = g.offsets == nullptr;
-        auto rows_of = [&](int ee) { return single ? g.single_rows : g.kept[ee]; };
-        const int nE = single ? 1 : g.E;
-        int n_full = 0, n_part = 0;
-        for (int ee = lane; ee < nE; ee += WAVE) {
-            const int r = rows_of(ee);
-            n_full += r / Q_BM + ((r % Q_BM) > Q_BM / 2);
-            n_part += (r % Q_BM) != 0 && (r % Q_BM) <= Q_BM / 2;
+// The bias of the 8 x 4 columns a lane holds results for, as raw bf16 quadruples; fetched before the K loop
+// so that the epilogue does not wait for it (zero bits are 0.0 in bf16).
+template <int EPI> __device__ __forceinline__ void load_bias(const GemmArgs &g, int e, int n0, int lane, int wave, uint2 (&bias_raw)[8]) {
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        bias_raw[c] = make_uint2(0, 0);
+        if constexpr (EPI == EPI_BIAS || EPI == EPI_BIAS_GELU) {
+            const int n = n0 + wave * 64 + (c >> 2) * 32 + 8 * (c & 3) + 4 * (lane >> 5);
+            if (n < g.N) bias_raw[c] = *reinterpret_cast<const uint2 *>((const bf16_t *)g.bias + (long)e * g.N + n);
         }
-        for (int d = WAVE / 2; d >= 1; d >>= 1) {
-            n_full += __shfl_xor(n_full, d, WAVE);
-            n_part += __shfl_xor(n_part, d, WAVE);
-        }
-        int target;            // index among the full (or partial) m-tiles
-        bool want_full;
-        if ((int)blockIdx.x < g.full_blocks) {
-            const int total = n_full * n_tiles;
-            const int per_xcd = (total + 7) >> 3;
-            const int slot = blockIdx.x >> 3;
-            const int t = (blockIdx.x & 7) * per_xcd + slot;
-            if (slot >= per_xcd || t >= total) return;
-            target = t / n_tiles;
-            nt = t % n_tiles;
-            want_full = true;
-        } else {
-            const int p = blockIdx.x - g.full_blocks;
-            if (p >= n_part * n_tiles) return;
-            target = p / n_tiles;
-            nt = p % n_tiles;
-            want_full = false;
-        }
-        // the expert whose running count passes `target`
-        int run = 0, found = -1, before = 0;
-        for (int base = 0; base < nE && found < 0; base += WAVE) {
-            const int ee = base + lane;
-            const int r = ee < nE ? rows_of(ee) : 0;
-            const int cnt = want_full ? r / Q_BM + ((r % Q_BM) > Q_BM / 2) : ((r % Q_BM) != 0 && (r % Q_BM) <= Q_BM / 2);
-            int incl = cnt;
-            for (int d = 1; d < WAVE; d <<= 1) {
-                const int y = __shfl_up(incl, d, WAVE);
-                if (lane >= d) incl += y;
-            }
-            const unsigned long long hit = __ballot(run + incl > target);
-            if (hit) {
-                const int src = __ffsll(hit) - 1;
-                found = base + src;
-                before = run + __shfl(incl - cnt, src, WAVE);
-            }
-            run += __shfl(incl, WAVE - 1, WAVE);
-        }
-        if (found < 0) return;
-        e = found;
-        m_ext = rows_of(e);
-        mt = want_full ? target - before : m_ext / Q_BM;
-        row0 = single ? 0 : g.offsets[e];
-        k_ext = g.K;
-    } else {
-        const int nblk = gridDim.x;
-        const int t = (blockIdx.x & 7) * (nblk >> 3) + (blockIdx.x >> 3);
-        if (t >= g.n_blocks) return;
-        const int m_tiles = (g.M + Q_BM - 1) / Q_BM;
-        e = t / (m_tiles * n_tiles);
-        const int rem = t % (m_tiles * n_tiles);
-        mt = rem / n_tiles;
-        nt = rem % n_tiles;
-        m_ext = g.M;
-        k_ext = g.kept ? g.kept[e] : g.single_rows;
-        row0 = g.offsets ? g.offsets[e] : 0;
     }
-    // the tile's coordinates are the same in every lane: say so, so that everything derived from them
-    // (operand bases, LDS destinations, loop bounds) lives in scalar registers
-    e = __builtin_amdgcn_readfirstlane(e);
-    mt = __builtin_amdgcn_readfirstlane(mt);
-    nt = __builtin_amdgcn_readfirstlane(nt);
-    m_ext = __builtin_amdgcn_readfirstlane(m_ext);
-    k_ext = __builtin_amdgcn_readfirstlane(k_ext);
-    row0 = ((long)__builtin_amdgcn_readfirstlane((int)(row0 >> 32)) << 32) | (unsigned)__builtin_amdgcn_readfirstlane((int)row0);
-    const int m0 = mt * Q_BM, n0 = nt * Q_BN;
-    const bf16_t *Mp = (const bf16_t *)g.A + row0 * g.lda;
-    const bf16_t *Np = WG ? (const bf16_t *)g.B + row0 * g.ldb : (const bf16_t *)g.B + (long)e * g.strideB;
+}
 
-    f32x16 acc[TMB][2];
-#pragma unroll
-    for (int i = 0; i < TMB; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
-
-    const int live = min(Q_BM, m_ext - m0);
-    const int tmc = (live + 31) >> 5;
-    if (tmc > TMB / 2)
-        main_loop<TMB, M_KS, N_KS, WG, TMB>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wave, acc);
-    else if (tmc > TMB / 4)
-        main_loop<TMB, M_KS, N_KS, WG, TMB / 2>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wave, acc);
-    else
-        main_loop<TMB, M_KS, N_KS, WG, TMB / 4>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wave, acc);
-
-    // ---- epilogue.  acc[tm][tn][4q+j] = C[m, n] with m = m0 + 32 tm + lane%32 and
-    //      n = n0 + 64 wave + 32 tn + 8 q + 4 (lane/32) + j.  A wave owns a BM x 64 slab of the tile.
-    //      bf16 results go through the wave's own BM x 128 bytes of LDS (the K loop is done with it) so that
-    //      global memory sees whole 128-byte rows: 8 bytes per lane into LDS ([row][8 x 16 B], chunk
-    //      ^ (row & 7)), then 16 bytes per lane out, 8 rows per store instruction.  The pre-activation
-    //      that GELU' needs comes in the same way, in the opposite direction.
+// The epilogue of a tile whose first TMC 32-row blocks hold live rows.  acc[tm][tn][4q+j] = C[m, n] with
+// m = m0 + 32 tm + lane%32 and n = n0 + 64 wave + 32 tn + 8 q + 4 (lane/32) + j.  A wave owns a BM x 64 slab
+// of the tile.  bf16 results go through the wave's own BM x 128 bytes of LDS (the K loop is done with it) so
+// that global memory sees whole 128-byte rows: 8 bytes per lane into LDS, then 16 bytes per lane out, 8 rows
+// per store instruction.  The pre-activation that GELU' needs comes in the same way, in the opposite
+// direction.  TMC is a compile-time bound so that the work of different cells can be interleaved.
+template <int TMB, bool WG, int EPI, int TMC>
+__device__ __forceinline__ void epilogue(const GemmArgs &g, f32x16 (&acc)[TMB][2], char *smem, int lane, int wave, int e,
+                                         long row0, int m0, int n0, int m_ext, int live, const uint2 (&bias_raw)[8]) {
+    constexpr int Q_BM = Tile<TMB>::BM;
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
     __syncthreads();
     const int lm = lane & 31, h = lane >> 5;
@@ -485,21 +384,32 @@ __global__ __launch_bounds__(Q_THREADS, Tile<TMB>::BLOCKS_PER_CU) void gemm256_k
         return (row & 16) ? make_uint4(v.z, v.w, v.x, v.y) : v;
     };
     // slab -> global: rows [0, live) of the slab, 128 bytes each
-    auto flush = [&](bf16_t *dst) {
-        for (int it = 0; it * 8 < live; ++it) {
+    auto flush = [&](bf16_t *dst) __attribute__((always_inline)) {
+#pragma unroll
+        for (int it = 0; it < TMC * 4; ++it) {
             const int row = it * 8 + jr;
             const uint4 v = fix16(*reinterpret_cast<const uint4 *>(slab_at(row, jc, (row >> 4) & 1)), row);
             if (row < live && col_ok)
                 *reinterpret_cast<uint4 *>(dst + (crow0 + m0 + row) * g.ldc + nw0 + jc * 8) = v;
         }
     };
-    // global -> slab
-    auto fill = [&](const bf16_t *src) {
-        for (int it = 0; it * 8 < live; ++it) {
-            const int row = it * 8 + jr;
-            uint4 v = make_uint4(0, 0, 0, 0);
-            if (row < live && col_ok) v = *reinterpret_cast<const uint4 *>(src + (crow0 + m0 + row) * g.ldc + nw0 + jc * 8);
-            *reinterpret_cast<uint4 *>(slab_at(row, jc, (row >> 4) & 1)) = fix16(v, row);
+    // global -> slab, eight rows' loads in flight at a time
+    auto fill = [&](const bf16_t *src) __attribute__((always_inline)) {
+#pragma unroll
+        for (int it0 = 0; it0 < TMC * 4; it0 += 8) {
+            uint4 v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int row = (it0 + i) * 8 + jr;
+                v[i] = make_uint4(0, 0, 0, 0);
+                if (it0 + i < TMC * 4 && row < live && col_ok)
+                    v[i] = *reinterpret_cast<const uint4 *>(src + (crow0 + m0 + row) * g.ldc + nw0 + jc * 8);
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int row = (it0 + i) * 8 + jr;
+                if (it0 + i < TMC * 4) *reinterpret_cast<uint4 *>(slab_at(row, jc, (row >> 4) & 1)) = fix16(v[i], row);
+            }
         }
     };
 
@@ -511,9 +421,9 @@ __global__ __launch_bounds__(Q_THREADS, Tile<TMB>::BLOCKS_PER_CU) void gemm256_k
                 const int n = nw0 + tn * 32 + 8 * q + 4 * h;
                 if (n >= g.N) continue;
 #pragma unroll
-                for (int tm = 0; tm < TMB; ++tm) {
+                for (int tm = 0; tm < TMC; ++tm) {
                     const int m = m0 + tm * 32 + lm;
-                    if (tm >= tmc || m >= m_ext) continue;
+                    if (m >= m_ext) continue;
                     *reinterpret_cast<float4 *>((float *)g.C + (crow0 + m) * g.ldc + n) =
                         make_float4(acc[tm][tn][4 * q], acc[tm][tn][4 * q + 1], acc[tm][tn][4 * q + 2], acc[tm][tn][4 * q + 3]);
                 }
@@ -533,12 +443,10 @@ __global__ __launch_bounds__(Q_THREADS, Tile<TMB>::BLOCKS_PER_CU) void gemm256_k
             for (int q = 0; q < 4; ++q) {
                 const int n = nw0 + tn * 32 + 8 * q + 4 * h;
                 float bias[4] = {0.f, 0.f, 0.f, 0.f};
-                if constexpr (EPI == EPI_BIAS || EPI == EPI_BIAS_GELU) {
-                    if (n < g.N) unpack4(*reinterpret_cast<const uint2 *>((const bf16_t *)g.bias + (long)e * g.N + n), bias);
-                }
+                if constexpr (EPI == EPI_BIAS || EPI == EPI_BIAS_GELU) unpack4(bias_raw[tn * 4 + q], bias);
+                (void)n;
 #pragma unroll
-                for (int tm = 0; tm < TMB; ++tm) {
-                    if (tm >= tmc) continue;
+                for (int tm = 0; tm < TMC; ++tm) {
                     char *cell = slab_at(tm * 32 + lm, tn * 4 + q, h);
                     float v[4];
 #pragma unroll
@@ -576,6 +484,135 @@ __global__ __launch_bounds__(Q_THREADS, Tile<TMB>::BLOCKS_PER_CU) void gemm256_k
             }
         }
         flush(pass == 0 ? Cb : (bf16_t *)g.C2);
+    }
+}
+
+// Row-ragged (!WG): C[rows_e, N] = Mop[rows_e, K] . Nop_e ; Mop K-contiguous, Nop_e [N,K] or (N_KS) [K,N].
+// Weight gradient (WG): C_e[M, N] = sum_{r in rows_e} Mop[r, M]^T . Nop[r, N], both K-strided.
+template <int TMB, bool N_KS, bool WG, int EPI>
+__global__ __launch_bounds__(Q_THREADS, Tile<TMB>::BLOCKS_PER_CU) void gemm256_kernel(const GemmArgs g) {
+    constexpr bool M_KS = WG;
+    constexpr int Q_BM = Tile<TMB>::BM;
+    extern __shared__ __align__(16) char smem[];
+    // ---- which tile am I?  Blocks are dealt round-robin to the 8 XCDs (block b runs on XCD b mod 8):
+    //      give each XCD a contiguous range of the REAL tiles, so that neighbours share operands in
+    //      its L2 and every XCD gets the same share.  For row-ragged products the number of real
+    //      tiles is only known here (the grid is sized for the worst case), hence the device-side sum.
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n_tiles = (g.N + Q_BN - 1) / Q_BN;
+    int e, mt, nt, m_ext, k_ext;
+    long row0;  // first row of the expert
+    if constexpr (!WG) {
+        // Heavy m-tiles (more than BM/2 live rows) take the first g.full_blocks block slots, in
+        // contiguous per-XCD ranges; the light ones (an expert's last tile with at most BM/2 rows)
+        // take the slots after them in plain order.  The hardware starts blocks in index order, so
+        // the short tiles fill the end of the launch instead of holding CUs for a full tile's time.
+        const bool single = g.offsets == nullptr;
+        auto rows_of = [&](int ee) { return single ? g.single_rows : g.kept[ee]; };
+        const int nE = single ? 1 : g.E;
+        // rows and first row of the first 64 experts, fetched together: the lookups below then need no further
+        // dependent loads (the scan itself re-reads rows_of through the cache)
+        const int rows_lane = lane < nE ? rows_of(lane) : 0;
+        const int off_lane = (!single && lane < nE) ? g.offsets[lane] : 0;
+        int n_full = 0, n_part = 0;
+        for (int ee = lane; ee < nE; ee += WAVE) {
+            const int r = ee < WAVE ? rows_lane : rows_of(ee);
+            n_full += r / Q_BM + ((r % Q_BM) > Q_BM / 2);
+            n_part += (r % Q_BM) != 0 && (r % Q_BM) <= Q_BM / 2;
+        }
+        for (int d = WAVE / 2; d >= 1; d >>= 1) {
+            n_full += __shfl_xor(n_full, d, WAVE);
+            n_part += __shfl_xor(n_part, d, WAVE);
+        }
+        int target;            // index among the full (or partial) m-tiles
+        bool want_full;
+        if ((int)blockIdx.x < g.full_blocks) {
+            const int total = n_full * n_tiles;
+            const int per_xcd = (total + 7) >> 3;
+            const int slot = blockIdx.x >> 3;
+            const int t = (blockIdx.x & 7) * per_xcd + slot;
+            if (slot >= per_xcd || t >= total) return;
+            target = t / n_tiles;
+            nt = t % n_tiles;
+            want_full = true;
+        } else {
+            const int p = blockIdx.x - g.full_blocks;
+            if (p >= n_part * n_tiles) return;
+            target = p / n_tiles;
+            nt = p % n_tiles;
+            want_full = false;
+        }
+        // the expert whose running count passes `target`
+        int run = 0, found = -1, before = 0;
+        for (int base = 0; base < nE && found < 0; base += WAVE) {
+            const int ee = base + lane;
+            const int r = base == 0 ? rows_lane : (ee < nE ? rows_of(ee) : 0);
+            const int cnt = want_full ? r / Q_BM + ((r % Q_BM) > Q_BM / 2) : ((r % Q_BM) != 0 && (r % Q_BM) <= Q_BM / 2);
+            int incl = cnt;
+            for (int d = 1; d < WAVE; d <<= 1) {
+                const int y = __shfl_up(incl, d, WAVE);
+                if (lane >= d) incl += y;
+            }
+            const unsigned long long hit = __ballot(run + incl > target);
+            if (hit) {
+                const int src = __ffsll(hit) - 1;
+                found = base + src;
+                before = run + __shfl(incl - cnt, src, WAVE);
+            }
+            run += __shfl(incl, WAVE - 1, WAVE);
+        }
+        if (found < 0) return;
+        e = found;
+        m_ext = found < WAVE ? __shfl(rows_lane, found, WAVE) : rows_of(e);
+        mt = want_full ? target - before : m_ext / Q_BM;
+        row0 = single ? 0 : (found < WAVE ? __shfl(off_lane, found, WAVE) : g.offsets[e]);
+        k_ext = g.K;
+    } else {
+        const int nblk = gridDim.x;
+        const int t = (blockIdx.x & 7) * (nblk >> 3) + (blockIdx.x >> 3);
+        if (t >= g.n_blocks) return;
+        const int m_tiles = (g.M + Q_BM - 1) / Q_BM;
+        e = t / (m_tiles * n_tiles);
+        const int rem = t % (m_tiles * n_tiles);
+        mt = rem / n_tiles;
+        nt = rem % n_tiles;
+        m_ext = g.M;
+        k_ext = g.kept ? g.kept[e] : g.single_rows;
+        row0 = g.offsets ? g.offsets[e] : 0;
+    }
+    // the tile's coordinates are the same in every lane: say so, so that everything derived from them
+    // (operand bases, LDS destinations, loop bounds) lives in scalar registers
+    e = __builtin_amdgcn_readfirstlane(e);
+    mt = __builtin_amdgcn_readfirstlane(mt);
+    nt = __builtin_amdgcn_readfirstlane(nt);
+    m_ext = __builtin_amdgcn_readfirstlane(m_ext);
+    k_ext = __builtin_amdgcn_readfirstlane(k_ext);
+    row0 = ((long)__builtin_amdgcn_readfirstlane((int)(row0 >> 32)) << 32) | (unsigned)__builtin_amdgcn_readfirstlane((int)row0);
+    const int m0 = mt * Q_BM, n0 = nt * Q_BN;
+    const bf16_t *Mp = (const bf16_t *)g.A + row0 * g.lda;
+    const bf16_t *Np = WG ? (const bf16_t *)g.B + row0 * g.ldb : (const bf16_t *)g.B + (long)e * g.strideB;
+
+    f32x16 acc[TMB][2];
+#pragma unroll
+    for (int i = 0; i < TMB; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
+
+    const int live = min(Q_BM, m_ext - m0);
+    const int tmc = (live + 31) >> 5;
+    uint2 bias_raw[8];
+    load_bias<EPI>(g, e, n0, lane, wave, bias_raw);
+    if (tmc > TMB / 2) {
+        main_loop<TMB, M_KS, N_KS, WG, TMB>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wave, acc);
+        epilogue<TMB, WG, EPI, TMB>(g, acc, smem, lane, wave, e, row0, m0, n0, m_ext, live, bias_raw);
+    } else if (tmc > TMB / 4) {
+        main_loop<TMB, M_KS, N_KS, WG, TMB / 2>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wave, acc);
+        epilogue<TMB, WG, EPI, TMB / 2>(g, acc, smem, lane, wave, e, row0, m0, n0, m_ext, live, bias_raw);
+    } else {
+        main_loop<TMB, M_KS, N_KS, WG, TMB / 4>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wave, acc);
+        epilogue<TMB, WG, EPI, TMB / 4>(g, acc, smem, lane, wave, e, row0, m0, n0, m_ext, live, bias_raw);
     }
 }
 
