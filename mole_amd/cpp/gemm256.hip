@@ -42,6 +42,19 @@ template <int TMB> struct Tile {
     static constexpr int BLOCKS_PER_CU = TMB >= 8 ? 1 : 2;
 };
 
+// One stage of the operand ring for a tile of which the first TMC 32-row blocks are live.  Of a K-contiguous
+// m-side tile only the 64-row groups that hold live blocks are fetched and stored, so a light tile has
+// smaller stages and its ring, in the same LDS, is deeper: light tiles do little arithmetic per stage and
+// run at the memory latency divided by the stages in flight.
+template <int TMB, bool M_KS, int TMC> struct Stage {
+    static constexpr int LM = M_KS ? Tile<TMB>::BM / 64 : (TMC * 32 + 63) / 64;   // m-side loads per wave
+    static constexpr int L = LM + Q_BN / 64;                                       // loads per wave
+    static constexpr int M_OPERAND = LM * 64 * Q_BK * 2;
+    static constexpr int BYTES = M_OPERAND + Q_N_OPERAND;
+    static constexpr int FIT = Tile<TMB>::NSTAGE * Tile<TMB>::STAGE / BYTES;
+    static constexpr int NSTAGE = FIT > 6 ? 6 : FIT;
+};
+
 // s_waitcnt immediate that waits for vmcnt <= n and nothing else (gfx9 encoding: vmcnt in bits 3:0
 // and 15:14, expcnt 6:4, lgkmcnt 11:8)
 constexpr int waitcnt_vm(int n) { return (n & 0xf) | ((n >> 4) << 14) | 0x0070 | 0x0f00; }
@@ -198,7 +211,7 @@ template <int TMB, bool M_KS, bool N_KS, int TMC> struct Frags {
     template <int P, int NP> __device__ __forceinline__ void read_part(const char *stage, int wave, int kk) {
 #pragma unroll
         for (int r = part_lo<P, NP, TMC + 2>(); r < part_lo<P + 1, NP, TMC + 2>(); ++r) {
-            if (r < 2) n[r] = frag<N_KS, Q_BN>(stage + Tile<TMB>::M_OPERAND, wave * 2 + r, kk);
+            if (r < 2) n[r] = frag<N_KS, Q_BN>(stage + Stage<TMB, M_KS, TMC>::M_OPERAND, wave * 2 + r, kk);
             else m[r - 2] = frag<M_KS, Tile<TMB>::BM>(stage, r - 2, kk);
         }
     }
@@ -215,9 +228,11 @@ template <int TMB, bool M_KS, bool N_KS, int TMC> struct Frags {
 // by a scalar base (advanced by one stage of K after a stage's last load) plus per-lane offsets that stay
 // fixed for the whole K loop.  Stages are fetched in order; past the last one the last is fetched again,
 // harmlessly: it keeps the number of loads per stage, which the vmcnt arithmetic of the loop relies on.
-template <int TMB, bool M_KS, bool N_KS, bool WG> struct Feeder {
+// Of a K-contiguous m-side tile only the 64-row groups that hold live 32-row blocks (the first TMC) are fetched.
+template <int TMB, bool M_KS, bool N_KS, bool WG, int TMC> struct Feeder {
     typedef Tile<TMB> TL;
-    static constexpr int LM = TL::BM / 64, L = TL::LOADS;
+    typedef Stage<TMB, M_KS, TMC> SG;
+    static constexpr int LM = SG::LM, L = SG::L;
     Off<TL::BM, M_KS> om, cm;
     Off<Q_BN, N_KS> on, cn;
     const char *bm, *bn;
@@ -243,7 +258,7 @@ template <int TMB, bool M_KS, bool N_KS, bool WG> struct Feeder {
     }
     // loads [J0, J1) of stage s (the m-side tile's loads come first) into ring buffer buf
     template <int J0, int J1> __device__ __forceinline__ void issue(int s, int buf) {
-        const uint32_t dst = lds_w + buf * TL::STAGE;
+        const uint32_t dst = lds_w + buf * SG::BYTES;
         const bool clamp_k = WG && ragged_k && s >= nk - 1;
 #pragma unroll
         for (int j = J0; j < J1; ++j) {
@@ -254,7 +269,7 @@ template <int TMB, bool M_KS, bool N_KS, bool WG> struct Feeder {
             } else {
                 uint32_t o = on.off[j - LM];
                 if constexpr (WG) o = clamp_k ? cn.off[j - LM] : o;
-                dma16s(bn, o, dst + TL::M_OPERAND + (j - LM) * 4096);
+                dma16s(bn, o, dst + SG::M_OPERAND + (j - LM) * 4096);
             }
         }
         if (J1 == L && s + 1 < nk) { bm += step_m; bn += step_n; }
@@ -273,18 +288,19 @@ template <int TMB, bool M_KS, bool N_KS, bool WG, int TMC>
 __device__ __forceinline__ void main_loop(const bf16_t *Mp, long ldm, int m0, int m_ext, const bf16_t *Np, long ldn,
                                           int n0, int n_ext, int k_ext, char *smem, int wave, f32x16 (&acc)[TMB][2]) {
     typedef Tile<TMB> TL;
-    constexpr int AHEAD = TL::NSTAGE - 1, NP = 4;
-    constexpr int L = TL::LOADS, LH = L / 2;
-    static_assert(L % 2 == 0, "a stage's loads are issued in two halves");
+    typedef Stage<TMB, M_KS, TMC> SG;
+    constexpr int AHEAD = SG::NSTAGE - 1, NP = 4;
+    typedef Feeder<TMB, M_KS, N_KS, WG, TMC> FD;
+    constexpr int L = FD::L, LH = L / 2;      // loads per wave per stage; the halves are LH and L - LH
     const int nk = (k_ext + Q_BK - 1) / Q_BK;
     if (nk == 0) return;
-    Feeder<TMB, M_KS, N_KS, WG> fd;
+    FD fd;
     fd.init(Mp, ldm, m0, m_ext, Np, ldn, n0, n_ext, k_ext, smem, wave);
     auto fix_tail = [&](int s, int buf) __attribute__((always_inline)) {   // ragged contraction: zero what lies past it in the last stage
         if (WG && s == nk - 1 && (k_ext & (Q_BK - 1))) {
-            char *b = smem + buf * TL::STAGE;
+            char *b = smem + buf * SG::BYTES;
             zero_k_tail<TL::BM>(b, k_ext & (Q_BK - 1));
-            zero_k_tail<Q_BN>(b + TL::M_OPERAND, k_ext & (Q_BK - 1));
+            zero_k_tail<Q_BN>(b + SG::M_OPERAND, k_ext & (Q_BK - 1));
             __syncthreads();
         }
     };
@@ -301,20 +317,20 @@ __device__ __forceinline__ void main_loop(const bf16_t *Mp, long ldm, int m0, in
     f0.read(smem, wave, 0);
     int cur_b = 0;                    // ring buffer of stage s
     for (int s = 0; s < nk; ++s) {
-        const int nxt_b = cur_b + 1 == TL::NSTAGE ? 0 : cur_b + 1;
-        const int free_b = cur_b == 0 ? TL::NSTAGE - 1 : cur_b - 1;     // held stage s-1, takes stage s+AHEAD
-        const int fill_b = free_b == 0 ? TL::NSTAGE - 1 : free_b - 1;   // takes the rest of stage s+AHEAD-1
-        const char *cur = smem + cur_b * TL::STAGE;
-        const char *nxt = smem + nxt_b * TL::STAGE;
+        const int nxt_b = cur_b + 1 == SG::NSTAGE ? 0 : cur_b + 1;
+        const int free_b = cur_b == 0 ? SG::NSTAGE - 1 : cur_b - 1;     // held stage s-1, takes stage s+AHEAD
+        const int fill_b = free_b == 0 ? SG::NSTAGE - 1 : free_b - 1;   // takes the rest of stage s+AHEAD-1
+        const char *cur = smem + cur_b * SG::BYTES;
+        const char *nxt = smem + nxt_b * SG::BYTES;
 #define MOLE_HALF(P, J0, N, S_LOAD, BUF, FR, STAGE_PTR, KK, FM)                                           \
         fd.template issue<(J0) + part_lo<P, NP, (N)>(), (J0) + part_lo<P + 1, NP, (N)>()>(S_LOAD, BUF);   \
         FR.template read_part<P, NP>(STAGE_PTR, wave, KK);                                                \
         FM.template mma_part<P, NP>(acc);                                                                 \
         __builtin_amdgcn_sched_barrier(0);
-        MOLE_HALF(0, SPLIT ? LH : 0, SPLIT ? LH : 0, s + AHEAD - 1, fill_b, f1, cur, 1, f0)
-        MOLE_HALF(1, SPLIT ? LH : 0, SPLIT ? LH : 0, s + AHEAD - 1, fill_b, f1, cur, 1, f0)
-        MOLE_HALF(2, SPLIT ? LH : 0, SPLIT ? LH : 0, s + AHEAD - 1, fill_b, f1, cur, 1, f0)
-        MOLE_HALF(3, SPLIT ? LH : 0, SPLIT ? LH : 0, s + AHEAD - 1, fill_b, f1, cur, 1, f0)
+        MOLE_HALF(0, SPLIT ? LH : 0, SPLIT ? L - LH : 0, s + AHEAD - 1, fill_b, f1, cur, 1, f0)
+        MOLE_HALF(1, SPLIT ? LH : 0, SPLIT ? L - LH : 0, s + AHEAD - 1, fill_b, f1, cur, 1, f0)
+        MOLE_HALF(2, SPLIT ? LH : 0, SPLIT ? L - LH : 0, s + AHEAD - 1, fill_b, f1, cur, 1, f0)
+        MOLE_HALF(3, SPLIT ? LH : 0, SPLIT ? L - LH : 0, s + AHEAD - 1, fill_b, f1, cur, 1, f0)
         __builtin_amdgcn_s_waitcnt(waitcnt_vm((AHEAD - 2) * L));
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
@@ -568,14 +584,17 @@ __global__ __launch_bounds__(Q_THREADS, Tile<TMB>::BLOCKS_PER_CU) void gemm256_k
         row0 = single ? 0 : (found < WAVE ? __shfl(off_lane, found, WAVE) : g.offsets[e]);
         k_ext = g.K;
     } else {
-        const int nblk = gridDim.x;
-        const int t = (blockIdx.x & 7) * (nblk >> 3) + (blockIdx.x >> 3);
-        if (t >= g.n_blocks) return;
+        // The contraction length differs from expert to expert, so experts are not handed to XCDs in
+        // contiguous ranges: the (expert, m-tile) units are dealt round-robin over the 8 XCDs, which gives
+        // every XCD the same share of every expert; the n-tiles of a unit stay together (they share the
+        // m-side operand in that XCD's L2).
         const int m_tiles = (g.M + Q_BM - 1) / Q_BM;
-        e = t / (m_tiles * n_tiles);
-        const int rem = t % (m_tiles * n_tiles);
-        mt = rem / n_tiles;
-        nt = rem % n_tiles;
+        const int slot = blockIdx.x >> 3;
+        const int unit = (slot / n_tiles) * 8 + (blockIdx.x & 7);
+        if (unit >= g.E * m_tiles) return;
+        e = unit / m_tiles;
+        mt = unit % m_tiles;
+        nt = slot % n_tiles;
         m_ext = g.M;
         k_ext = g.kept ? g.kept[e] : g.single_rows;
         row0 = g.offsets ? g.offsets[e] : 0;
@@ -638,7 +657,7 @@ static int dispatch256(const GemmArgs &g, bool b_ks, bool wg, int epi, int max_r
     constexpr int BM = Tile<TMB>::BM;
     const int n_tiles = ceil_div(g.N, Q_BN);
     if (wg) {
-        const int tiles = g.E * ceil_div(g.M, BM) * n_tiles;
+        const int tiles = 8 * ceil_div(g.E * ceil_div(g.M, BM), 8) * n_tiles;   // whole (expert, m-tile) units per XCD
         if (epi == EPI_WGRAD) return launch256<TMB, true, true, EPI_WGRAD>(g, tiles, st, kid);
         return -100;
     }
