@@ -27,17 +27,18 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 
 constexpr int Q_BN = 256, Q_BK = 32;
-constexpr int Q_THREADS = 256;
 constexpr int Q_N_OPERAND = Q_BN * Q_BK * 2;   // bytes of the n-side tile of one stage
 
-// geometry of a tile with TMB 32-row m-blocks
-template <int TMB> struct Tile {
+// Geometry of a BM x 256 tile of TMB 32-row m-blocks computed by 4 WM waves: WM wave rows of TMB/WM m-blocks
+// each, 4 wave columns of 64 columns each.  WM = 2 puts two waves on every SIMD: while one waits for
+// the memory pipeline to accept a load or for a barrier, the other issues MFMAs.
+template <int TMB, int WM> struct Tile {
+    static constexpr int NW = 4 * WM, THREADS = 64 * NW, TMW = TMB / WM;
     static constexpr int BM = TMB * 32;
     static constexpr int M_OPERAND = BM * Q_BK * 2;
     static constexpr int STAGE = M_OPERAND + Q_N_OPERAND;
     static constexpr int NSTAGE = TMB >= 8 ? 4 : 3;
-    static constexpr int LOADS = (M_OPERAND + Q_N_OPERAND) / 4096;   // asynchronous loads per wave per stage
-    static constexpr int SLABS = 4 * BM * 128;                       // the four waves' epilogue staging areas
+    static constexpr int SLABS = 4 * BM * 128;                       // the waves' epilogue staging areas
     static constexpr int LDS_BYTES = NSTAGE * STAGE > SLABS ? NSTAGE * STAGE : SLABS;
     static constexpr int BLOCKS_PER_CU = TMB >= 8 ? 1 : 2;
 };
@@ -46,12 +47,15 @@ template <int TMB> struct Tile {
 // m-side tile only the 64-row groups that hold live blocks are fetched and stored, so a light tile has
 // smaller stages and its ring, in the same LDS, is deeper: light tiles do little arithmetic per stage and
 // run at the memory latency divided by the stages in flight.
-template <int TMB, bool M_KS, int TMC> struct Stage {
-    static constexpr int LM = M_KS ? Tile<TMB>::BM / 64 : (TMC * 32 + 63) / 64;   // m-side loads per wave
-    static constexpr int L = LM + Q_BN / 64;                                       // loads per wave
-    static constexpr int M_OPERAND = LM * 64 * Q_BK * 2;
+template <int TMB, int WM, bool M_KS, int TMC> struct Stage {
+    typedef Tile<TMB, WM> TL;
+    static constexpr int RPL = 16 * TL::NW;                                       // rows (or 16-byte slot groups) one load of every wave covers
+    static constexpr int LM = M_KS ? TL::BM / RPL : (TMC * 32 + RPL - 1) / RPL;  // m-side loads per wave
+    static constexpr int LN = Q_BN / RPL;
+    static constexpr int L = LM + LN;                                             // loads per wave
+    static constexpr int M_OPERAND = LM * RPL * Q_BK * 2;
     static constexpr int BYTES = M_OPERAND + Q_N_OPERAND;
-    static constexpr int FIT = Tile<TMB>::NSTAGE * Tile<TMB>::STAGE / BYTES;
+    static constexpr int FIT = TL::NSTAGE * TL::STAGE / BYTES;
     static constexpr int NSTAGE = FIT > 6 ? 6 : FIT;
 };
 
@@ -132,19 +136,19 @@ __device__ __forceinline__ float fast_d_gelu_exact(float x) {
 // K-contiguous operand, element (r, k) at p[r*ld + k]: LDS [ROWS][4 x 16 B], the chunk index XORed
 // with swz4(row), chosen so that the 16 rows a ds_read_b128 pass touches (and any 8 aligned rows)
 // fall into distinct bank groups of the 64-bank LDS.
-// Wave w, load i fills LDS bytes [(4i+w)*1024, +1024) = rows 16(4i+w) .. +16.
+// With NW waves, wave w's load i fills LDS bytes [(NW i + w)*1024, +1024) = rows 16(NW i + w) .. +16.
 __device__ __forceinline__ int swz4(int row) { return (((row >> 1) ^ (row >> 3)) & 1) | ((row >> 1) & 2); }
-// Per-lane byte offsets of the ROWS/64 loads a wave issues for one stage of an operand tile, relative to
+// Per-lane byte offsets of the ROWS/(16 NW) loads a wave issues for one stage of an operand tile, relative to
 // the tile's first element at the stage's first k (what the scalar base points at).  r_left = rows of the
 // operand from the tile's first row on, k_left = k-rows from the stage's first k on (only the last stage
 // of a ragged contraction has fewer than 32).
-template <int ROWS> struct OffKC {
-    uint32_t off[ROWS / 64];
+template <int ROWS, int NW> struct OffKC {
+    uint32_t off[ROWS / (16 * NW)];
     __device__ __forceinline__ void init(long ld, int r_left) {
         const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
 #pragma unroll
-        for (int i = 0; i < ROWS / 64; ++i) {
-            const int row = (4 * i + w) * 16 + (lane >> 2);
+        for (int i = 0; i < ROWS / (16 * NW); ++i) {
+            const int row = (NW * i + w) * 16 + (lane >> 2);
             const int c = (lane & 3) ^ swz4(row);
             off[i] = (uint32_t)(min(row, r_left - 1) * ld * 2 + c * 16);
         }
@@ -153,27 +157,27 @@ template <int ROWS> struct OffKC {
 // K-strided operand, element (r, k) at p[k*ld + r]: LDS [32 k][ROWS x 2 B] as it lies in HBM, the
 // 32-byte granule index XORed with (k & 3) << 1 (conflict-free transpose reads, see frag_ks).
 // A k-row has ROWS/8 slots of 16 bytes; a wave load of 1 KiB covers 512/ROWS k-rows.
-template <int ROWS> struct OffKS {
-    uint32_t off[ROWS / 64];
+template <int ROWS, int NW> struct OffKS {
+    uint32_t off[ROWS / (16 * NW)];
     __device__ __forceinline__ void init(long ld, int r_left, int k_left) {
         constexpr int SPR = ROWS / 8;          // 16-byte slots per k-row
         constexpr int KPL = 64 / SPR;          // k-rows per wave load
         const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
 #pragma unroll
-        for (int i = 0; i < ROWS / 64; ++i) {
-            const int kr = (4 * i + w) * KPL + lane / SPR;
+        for (int i = 0; i < ROWS / (16 * NW); ++i) {
+            const int kr = (NW * i + w) * KPL + lane / SPR;
             const int pc = lane % SPR;                                        // physical 16-byte slot in the k-row
             const int c = ((((pc >> 1) ^ ((kr & 3) << 1)) << 1) | (pc & 1));  // logical 16-byte chunk
             off[i] = (uint32_t)(min(kr, k_left - 1) * ld * 2 + min(c * 8, r_left - 8) * 2);
         }
     }
 };
-template <int ROWS, bool KS> struct Off;
-template <int ROWS> struct Off<ROWS, false> : OffKC<ROWS> {};
-template <int ROWS> struct Off<ROWS, true> : OffKS<ROWS> {};
+template <int ROWS, int NW, bool KS> struct Off;
+template <int ROWS, int NW> struct Off<ROWS, NW, false> : OffKC<ROWS, NW> {};
+template <int ROWS, int NW> struct Off<ROWS, NW, true> : OffKS<ROWS, NW> {};
 // zero the k-rows [k_valid, 32) of a K-strided tile (the last, partial stage of a weight gradient)
-template <int ROWS> __device__ __forceinline__ void zero_k_tail(char *lds, int k_valid) {
-    for (int idx = threadIdx.x; idx < (Q_BK - k_valid) * (ROWS / 8); idx += Q_THREADS)
+template <int ROWS, int THREADS> __device__ __forceinline__ void zero_k_tail(char *lds, int k_valid) {
+    for (int idx = threadIdx.x; idx < (Q_BK - k_valid) * (ROWS / 8); idx += THREADS)
         *reinterpret_cast<uint4 *>(lds + k_valid * (ROWS * 2) + idx * 16) = make_uint4(0, 0, 0, 0);
 }
 
@@ -205,21 +209,26 @@ template <bool KS, int ROWS> __device__ __forceinline__ bf16x8 frag(const char *
 // first index of part P when N items are dealt to NP consecutive parts
 template <int P, int NP, int N> constexpr int part_lo() { return P * N / NP; }
 
-template <int TMB, bool M_KS, bool N_KS, int TMC> struct Frags {
-    bf16x8 m[TMC], n[2];
-    // the TMC + 2 fragment reads of a k-sub-step, n-side first, dealt to NP parts
-    template <int P, int NP> __device__ __forceinline__ void read_part(const char *stage, int wave, int kk) {
+// The fragments one wave needs for a k-sub-step: its TMCW live m-blocks (blocks wm*TMW .. of the tile, of which
+// the tile's first TMC are live) and its two 32-column n-blocks.  TMCW = 0: the wave has no live rows and
+// only takes part in the loads and barriers.
+template <int TMB, int WM, bool M_KS, bool N_KS, int TMC, int TMCW> struct Frags {
+    typedef Tile<TMB, WM> TL;
+    static constexpr int NR = TMCW ? TMCW + 2 : 0;
+    bf16x8 m[TMCW ? TMCW : 1], n[2];
+    // the fragment reads of a k-sub-step, n-side first, dealt to NP parts
+    template <int P, int NP> __device__ __forceinline__ void read_part(const char *stage, int wm, int wn, int kk) {
 #pragma unroll
-        for (int r = part_lo<P, NP, TMC + 2>(); r < part_lo<P + 1, NP, TMC + 2>(); ++r) {
-            if (r < 2) n[r] = frag<N_KS, Q_BN>(stage + Stage<TMB, M_KS, TMC>::M_OPERAND, wave * 2 + r, kk);
-            else m[r - 2] = frag<M_KS, Tile<TMB>::BM>(stage, r - 2, kk);
+        for (int r = part_lo<P, NP, NR>(); r < part_lo<P + 1, NP, NR>(); ++r) {
+            if (r < 2) n[r] = frag<N_KS, Q_BN>(stage + Stage<TMB, WM, M_KS, TMC>::M_OPERAND, wn * 2 + r, kk);
+            else m[r - 2] = frag<M_KS, TL::BM>(stage, wm * TL::TMW + r - 2, kk);
         }
     }
-    __device__ __forceinline__ void read(const char *stage, int wave, int kk) { read_part<0, 1>(stage, wave, kk); }
-    // the 2 TMC MFMAs of a k-sub-step dealt to NP parts
-    template <int P, int NP> __device__ __forceinline__ void mma_part(f32x16 (&acc)[TMB][2]) const {
+    __device__ __forceinline__ void read(const char *stage, int wm, int wn, int kk) { read_part<0, 1>(stage, wm, wn, kk); }
+    // the 2 TMCW MFMAs of a k-sub-step dealt to NP parts
+    template <int P, int NP> __device__ __forceinline__ void mma_part(f32x16 (&acc)[TL::TMW][2]) const {
 #pragma unroll
-        for (int i = part_lo<P, NP, 2 * TMC>(); i < part_lo<P + 1, NP, 2 * TMC>(); ++i)
+        for (int i = part_lo<P, NP, 2 * TMCW>(); i < part_lo<P + 1, NP, 2 * TMCW>(); ++i)
             acc[i >> 1][i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(n[i & 1], m[i >> 1], acc[i >> 1][i & 1], 0, 0, 0);
     }
 };
@@ -229,12 +238,12 @@ template <int TMB, bool M_KS, bool N_KS, int TMC> struct Frags {
 // fixed for the whole K loop.  Stages are fetched in order; past the last one the last is fetched again,
 // harmlessly: it keeps the number of loads per stage, which the vmcnt arithmetic of the loop relies on.
 // Of a K-contiguous m-side tile only the 64-row groups that hold live 32-row blocks (the first TMC) are fetched.
-template <int TMB, bool M_KS, bool N_KS, bool WG, int TMC> struct Feeder {
-    typedef Tile<TMB> TL;
-    typedef Stage<TMB, M_KS, TMC> SG;
+template <int TMB, int WM, bool M_KS, bool N_KS, bool WG, int TMC> struct Feeder {
+    typedef Tile<TMB, WM> TL;
+    typedef Stage<TMB, WM, M_KS, TMC> SG;
     static constexpr int LM = SG::LM, L = SG::L;
-    Off<TL::BM, M_KS> om, cm;
-    Off<Q_BN, N_KS> on, cn;
+    Off<TL::BM, TL::NW, M_KS> om, cm;
+    Off<Q_BN, TL::NW, N_KS> on, cn;
     const char *bm, *bn;
     long step_m, step_n;
     uint32_t lds_w;      // LDS address of ring buffer 0 + this wave's 1 KiB lane
@@ -265,11 +274,11 @@ template <int TMB, bool M_KS, bool N_KS, bool WG, int TMC> struct Feeder {
             if (j < LM) {
                 uint32_t o = om.off[j];
                 if constexpr (WG) o = clamp_k ? cm.off[j] : o;
-                dma16s(bm, o, dst + j * 4096);
+                dma16s(bm, o, dst + j * (TL::NW * 1024));
             } else {
                 uint32_t o = on.off[j - LM];
                 if constexpr (WG) o = clamp_k ? cn.off[j - LM] : o;
-                dma16s(bn, o, dst + SG::M_OPERAND + (j - LM) * 4096);
+                dma16s(bn, o, dst + SG::M_OPERAND + (j - LM) * (TL::NW * 1024));
             }
         }
         if (J1 == L && s + 1 < nk) { bm += step_m; bn += step_n; }
@@ -284,13 +293,14 @@ template <int TMB, bool M_KS, bool N_KS, bool WG, int TMC> struct Feeder {
 // iteration s+1 the rest, into the buffer that stage s-1 has left.  One synchronisation point per
 // iteration, between the halves: wait until this wave's share of stage s+1 has landed (newer stages may
 // still be in flight), then the barrier.
-template <int TMB, bool M_KS, bool N_KS, bool WG, int TMC>
+template <int TMB, int WM, bool M_KS, bool N_KS, bool WG, int TMC, int TMCW>
 __device__ __forceinline__ void main_loop(const bf16_t *Mp, long ldm, int m0, int m_ext, const bf16_t *Np, long ldn,
-                                          int n0, int n_ext, int k_ext, char *smem, int wave, f32x16 (&acc)[TMB][2]) {
-    typedef Tile<TMB> TL;
-    typedef Stage<TMB, M_KS, TMC> SG;
+                                          int n0, int n_ext, int k_ext, char *smem, int wave, int wm, int wn,
+                                          f32x16 (&acc)[Tile<TMB, WM>::TMW][2]) {
+    typedef Tile<TMB, WM> TL;
+    typedef Stage<TMB, WM, M_KS, TMC> SG;
     constexpr int AHEAD = SG::NSTAGE - 1, NP = 4;
-    typedef Feeder<TMB, M_KS, N_KS, WG, TMC> FD;
+    typedef Feeder<TMB, WM, M_KS, N_KS, WG, TMC> FD;
     constexpr int L = FD::L, LH = L / 2;      // loads per wave per stage; the halves are LH and L - LH
     const int nk = (k_ext + Q_BK - 1) / Q_BK;
     if (nk == 0) return;
@@ -299,8 +309,8 @@ __device__ __forceinline__ void main_loop(const bf16_t *Mp, long ldm, int m0, in
     auto fix_tail = [&](int s, int buf) __attribute__((always_inline)) {   // ragged contraction: zero what lies past it in the last stage
         if (WG && s == nk - 1 && (k_ext & (Q_BK - 1))) {
             char *b = smem + buf * SG::BYTES;
-            zero_k_tail<TL::BM>(b, k_ext & (Q_BK - 1));
-            zero_k_tail<Q_BN>(b + SG::M_OPERAND, k_ext & (Q_BK - 1));
+            zero_k_tail<TL::BM, TL::THREADS>(b, k_ext & (Q_BK - 1));
+            zero_k_tail<Q_BN, TL::THREADS>(b + SG::M_OPERAND, k_ext & (Q_BK - 1));
             __syncthreads();
         }
     };
@@ -313,8 +323,8 @@ __device__ __forceinline__ void main_loop(const bf16_t *Mp, long ldm, int m0, in
     __builtin_amdgcn_s_waitcnt(waitcnt_vm((AHEAD - 2) * L + (SPLIT ? LH : L)));
     __builtin_amdgcn_s_barrier();
     fix_tail(0, 0);
-    Frags<TMB, M_KS, N_KS, TMC> f0, f1;
-    f0.read(smem, wave, 0);
+    Frags<TMB, WM, M_KS, N_KS, TMC, TMCW> f0, f1;
+    f0.read(smem, wm, wn, 0);
     int cur_b = 0;                    // ring buffer of stage s
     for (int s = 0; s < nk; ++s) {
         const int nxt_b = cur_b + 1 == SG::NSTAGE ? 0 : cur_b + 1;
@@ -324,7 +334,7 @@ __device__ __forceinline__ void main_loop(const bf16_t *Mp, long ldm, int m0, in
         const char *nxt = smem + nxt_b * SG::BYTES;
 #define MOLE_HALF(P, J0, N, S_LOAD, BUF, FR, STAGE_PTR, KK, FM)                                           \
         fd.template issue<(J0) + part_lo<P, NP, (N)>(), (J0) + part_lo<P + 1, NP, (N)>()>(S_LOAD, BUF);   \
-        FR.template read_part<P, NP>(STAGE_PTR, wave, KK);                                                \
+        FR.template read_part<P, NP>(STAGE_PTR, wm, wn, KK);                                                \
         FM.template mma_part<P, NP>(acc);                                                                 \
         __builtin_amdgcn_sched_barrier(0);
         MOLE_HALF(0, SPLIT ? LH : 0, SPLIT ? L - LH : 0, s + AHEAD - 1, fill_b, f1, cur, 1, f0)
@@ -358,35 +368,37 @@ __device__ __forceinline__ void unpack4(uint2 u, float *f) {
 
 // The bias of the 8 x 4 columns a lane holds results for, as raw bf16 quadruples; fetched before the K loop
 // so that the epilogue does not wait for it (zero bits are 0.0 in bf16).
-template <int EPI> __device__ __forceinline__ void load_bias(const GemmArgs &g, int e, int n0, int lane, int wave, uint2 (&bias_raw)[8]) {
+template <int EPI> __device__ __forceinline__ void load_bias(const GemmArgs &g, int e, int n0, int lane, int wn, uint2 (&bias_raw)[8]) {
 #pragma unroll
     for (int c = 0; c < 8; ++c) {
         bias_raw[c] = make_uint2(0, 0);
         if constexpr (EPI == EPI_BIAS || EPI == EPI_BIAS_GELU) {
-            const int n = n0 + wave * 64 + (c >> 2) * 32 + 8 * (c & 3) + 4 * (lane >> 5);
+            const int n = n0 + wn * 64 + (c >> 2) * 32 + 8 * (c & 3) + 4 * (lane >> 5);
             if (n < g.N) bias_raw[c] = *reinterpret_cast<const uint2 *>((const bf16_t *)g.bias + (long)e * g.N + n);
         }
     }
 }
 
-// The epilogue of a tile whose first TMC 32-row blocks hold live rows.  acc[tm][tn][4q+j] = C[m, n] with
-// m = m0 + 32 tm + lane%32 and n = n0 + 64 wave + 32 tn + 8 q + 4 (lane/32) + j.  A wave owns a BM x 64 slab
-// of the tile.  bf16 results go through the wave's own BM x 128 bytes of LDS (the K loop is done with it) so
-// that global memory sees whole 128-byte rows: 8 bytes per lane into LDS, then 16 bytes per lane out, 8 rows
-// per store instruction.  The pre-activation that GELU' needs comes in the same way, in the opposite
-// direction.  TMC is a compile-time bound so that the work of different cells can be interleaved.
-template <int TMB, bool WG, int EPI, int TMC>
-__device__ __forceinline__ void epilogue(const GemmArgs &g, f32x16 (&acc)[TMB][2], char *smem, int lane, int wave, int e,
-                                         long row0, int m0, int n0, int m_ext, int live, const uint2 (&bias_raw)[8]) {
-    constexpr int Q_BM = Tile<TMB>::BM;
+// The epilogue of one wave, whose first TMCW 32-row blocks hold live rows.  acc[tm][tn][4q+j] = C[m, n] with
+// m = m0 + 32 tm + lane%32 (m0: the wave's first row) and n = n0 + 64 wn + 32 tn + 8 q + 4 (lane/32) + j.  A wave
+// owns a (32 TMW) x 64 slab of the tile.  bf16 results go through the wave's own slab of LDS (the K loop is
+// done with it) so that global memory sees whole 128-byte rows: 8 bytes per lane into LDS, then 16 bytes
+// per lane out, 8 rows per store instruction.  The pre-activation that GELU' needs comes in the same way,
+// in the opposite direction.  TMCW is a compile-time bound so that the work of different cells can be
+// interleaved.  live: the wave's live rows.
+template <int TMB, int WM, bool WG, int EPI, int TMC>
+__device__ __forceinline__ void epilogue(const GemmArgs &g, f32x16 (&acc)[Tile<TMB, WM>::TMW][2], char *smem, int lane, int wave,
+                                         int wn, int e, long row0, int m0, int n0, int m_ext, int live,
+                                         const uint2 (&bias_raw)[8]) {
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
     __syncthreads();
+    if constexpr (TMC == 0) return;
     const int lm = lane & 31, h = lane >> 5;
     bf16_t *Cb = (bf16_t *)g.C;
     long crow0 = row0;
     if constexpr (WG) { crow0 = 0; Cb += (long)e * g.strideC; }
-    const int nw0 = n0 + wave * 64;                 // first column of this wave's slab
-    char *slab = smem + wave * (Q_BM * 128);
+    const int nw0 = n0 + wn * 64;                   // first column of this wave's slab
+    char *slab = smem + wave * (Tile<TMB, WM>::TMW * 32 * 128);
     const int jr = lane >> 3, jc = lane & 7;        // row-in-group / 16-byte column of the wide accesses
     const bool col_ok = nw0 + jc * 8 < g.N;
 
@@ -505,10 +517,11 @@ __device__ __forceinline__ void epilogue(const GemmArgs &g, f32x16 (&acc)[TMB][2
 
 // Row-ragged (!WG): C[rows_e, N] = Mop[rows_e, K] . Nop_e ; Mop K-contiguous, Nop_e [N,K] or (N_KS) [K,N].
 // Weight gradient (WG): C_e[M, N] = sum_{r in rows_e} Mop[r, M]^T . Nop[r, N], both K-strided.
-template <int TMB, bool N_KS, bool WG, int EPI>
-__global__ __launch_bounds__(Q_THREADS, Tile<TMB>::BLOCKS_PER_CU) void gemm256_kernel(const GemmArgs g) {
+template <int TMB, int WM, bool N_KS, bool WG, int EPI>
+__global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PER_CU)) void gemm256_kernel(const GemmArgs g) {
+    typedef Tile<TMB, WM> TL;
     constexpr bool M_KS = WG;
-    constexpr int Q_BM = Tile<TMB>::BM;
+    constexpr int Q_BM = TL::BM, TMW = TL::TMW;
     extern __shared__ __align__(16) char smem[];
     // ---- which tile am I?  Blocks are dealt round-robin to the 8 XCDs (block b runs on XCD b mod 8):
     //      give each XCD a contiguous range of the REAL tiles, so that neighbours share operands in
@@ -611,9 +624,9 @@ __global__ __launch_bounds__(Q_THREADS, Tile<TMB>::BLOCKS_PER_CU) void gemm256_k
     const bf16_t *Mp = (const bf16_t *)g.A + row0 * g.lda;
     const bf16_t *Np = WG ? (const bf16_t *)g.B + row0 * g.ldb : (const bf16_t *)g.B + (long)e * g.strideB;
 
-    f32x16 acc[TMB][2];
+    f32x16 acc[TMW][2];
 #pragma unroll
-    for (int i = 0; i < TMB; ++i)
+    for (int i = 0; i < TMW; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -621,44 +634,57 @@ __global__ __launch_bounds__(Q_THREADS, Tile<TMB>::BLOCKS_PER_CU) void gemm256_k
 
     const int live = min(Q_BM, m_ext - m0);
     const int tmc = (live + 31) >> 5;
+    const int wu = __builtin_amdgcn_readfirstlane(wave);
+    const int wm = WM == 1 ? 0 : wu >> 2, wn = wu & 3;     // wave row / wave column
     uint2 bias_raw[8];
-    load_bias<EPI>(g, e, n0, lane, wave, bias_raw);
-    if (tmc > TMB / 2) {
-        main_loop<TMB, M_KS, N_KS, WG, TMB>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wave, acc);
-        epilogue<TMB, WG, EPI, TMB>(g, acc, smem, lane, wave, e, row0, m0, n0, m_ext, live, bias_raw);
-    } else if (tmc > TMB / 4) {
-        main_loop<TMB, M_KS, N_KS, WG, TMB / 2>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wave, acc);
-        epilogue<TMB, WG, EPI, TMB / 2>(g, acc, smem, lane, wave, e, row0, m0, n0, m_ext, live, bias_raw);
-    } else {
-        main_loop<TMB, M_KS, N_KS, WG, TMB / 4>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wave, acc);
-        epilogue<TMB, WG, EPI, TMB / 4>(g, acc, smem, lane, wave, e, row0, m0, n0, m_ext, live, bias_raw);
+    load_bias<EPI>(g, e, n0, lane, wn, bias_raw);
+    // K loop and epilogue for a tile whose first TMC blocks are live; the wave's share is CW of them
+#define MOLE_RUN_TILE(TMC)                                                                                                \
+    if (WM == 1 || wm == 0) {                                                                                             \
+        constexpr int CW = (TMC) < TMW ? (TMC) : TMW;                                                                     \
+        main_loop<TMB, WM, M_KS, N_KS, WG, (TMC), CW>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wu, 0, wn, acc); \
+        epilogue<TMB, WM, WG, EPI, CW>(g, acc, smem, lane, wu, wn, e, row0, m0, n0, m_ext, min(live, TMW * 32), bias_raw); \
+    } else {                                                                                                              \
+        constexpr int CW = (TMC) > TMW ? (TMC) - TMW : 0;                                                                 \
+        main_loop<TMB, WM, M_KS, N_KS, WG, (TMC), CW>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wu, 1, wn, acc); \
+        epilogue<TMB, WM, WG, EPI, CW>(g, acc, smem, lane, wu, wn, e, row0, m0 + TMW * 32, n0, m_ext, live - TMW * 32,    \
+                                       bias_raw);                                                                         \
     }
+    if (tmc > TMB / 2) {
+        MOLE_RUN_TILE(TMB)
+    } else if (tmc > TMB / 4) {
+        MOLE_RUN_TILE(TMB / 2)
+    } else {
+        MOLE_RUN_TILE(TMB / 4)
+    }
+#undef MOLE_RUN_TILE
 }
 
-template <int TMB, bool N_KS, bool WG, int EPI>
+template <int TMB, int WM, bool N_KS, bool WG, int EPI>
 static int launch256(GemmArgs g, int tiles, hipStream_t st, int kid) {
+    typedef Tile<TMB, WM> TL;
     if (tiles <= 0) return 0;
     ScopedTiming timing(kid, st);
     g.n_blocks = tiles;
     const int grid = (tiles + 7) & ~7;
-    auto kern = gemm256_kernel<TMB, N_KS, WG, EPI>;
+    auto kern = gemm256_kernel<TMB, WM, N_KS, WG, EPI>;
     static bool attr_done = false;
     if (!attr_done) {
-        MOLE_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, Tile<TMB>::LDS_BYTES));
+        MOLE_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, TL::LDS_BYTES));
         attr_done = true;
     }
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(Q_THREADS), Tile<TMB>::LDS_BYTES, st, g);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(TL::THREADS), TL::LDS_BYTES, st, g);
     MOLE_LAUNCH_CHECK();
     return 0;
 }
 
-template <int TMB>
+template <int TMB, int WM>
 static int dispatch256(const GemmArgs &g, bool b_ks, bool wg, int epi, int max_rows, hipStream_t st, int kid) {
-    constexpr int BM = Tile<TMB>::BM;
+    constexpr int BM = Tile<TMB, WM>::BM;
     const int n_tiles = ceil_div(g.N, Q_BN);
     if (wg) {
         const int tiles = 8 * ceil_div(g.E * ceil_div(g.M, BM), 8) * n_tiles;   // whole (expert, m-tile) units per XCD
-        if (epi == EPI_WGRAD) return launch256<TMB, true, true, EPI_WGRAD>(g, tiles, st, kid);
+        if (epi == EPI_WGRAD) return launch256<TMB, WM, true, true, EPI_WGRAD>(g, tiles, st, kid);
         return -100;
     }
     // block slots: worst-case number of heavy m-tiles (each has more than BM/2 rows; rounded to the
@@ -668,28 +694,27 @@ static int dispatch256(const GemmArgs &g, bool b_ks, bool wg, int epi, int max_r
     gg.full_blocks = ((rows_bound / (BM / 2)) * n_tiles + 7) & ~7;
     const int tiles = gg.full_blocks + (g.offsets ? g.E : 1) * n_tiles;
     if (!b_ks) {
-        if (epi == EPI_BIAS_GELU) return launch256<TMB, false, false, EPI_BIAS_GELU>(gg, tiles, st, kid);
-        if (epi == EPI_DGELU) return launch256<TMB, false, false, EPI_DGELU>(gg, tiles, st, kid);
-        if (epi == EPI_F32) return launch256<TMB, false, false, EPI_F32>(gg, tiles, st, kid);
+        if (epi == EPI_BIAS_GELU) return launch256<TMB, WM, false, false, EPI_BIAS_GELU>(gg, tiles, st, kid);
+        if (epi == EPI_DGELU) return launch256<TMB, WM, false, false, EPI_DGELU>(gg, tiles, st, kid);
+        if (epi == EPI_F32) return launch256<TMB, WM, false, false, EPI_F32>(gg, tiles, st, kid);
     } else {
-        if (epi == EPI_BIAS) return launch256<TMB, true, false, EPI_BIAS>(gg, tiles, st, kid);
-        if (epi == EPI_STORE) return launch256<TMB, true, false, EPI_STORE>(gg, tiles, st, kid);
+        if (epi == EPI_BIAS) return launch256<TMB, WM, true, false, EPI_BIAS>(gg, tiles, st, kid);
+        if (epi == EPI_STORE) return launch256<TMB, WM, true, false, EPI_STORE>(gg, tiles, st, kid);
     }
     return -100;
 }
 
-// Tile height per product: 128 rows (two blocks per CU) or 256 rows (one block per CU).
-// MOLE_TMB=4|8 in the environment overrides the choice (tuning aid).
+// Tile configuration: 256 rows on eight waves for every product (two waves per SIMD hide each other's
+// waits; one fetch of the n-side tile serves all 256 rows).  MOLE_TMB=4|8 in the environment selects the
+// four-wave variants with 128 or 256 rows instead (tuning aid).
 static int tile_blocks_for(int kid) {
     static const int forced = [] {
         const char *v = getenv("MOLE_TMB");
         return v ? atoi(v) : 0;
     }();
-    if (forced == 4 || forced == 8) return forced;
-    // the products with a heavy epilogue (GELU, GELU') and the weight gradients gain from two
-    // co-resident blocks that overlap one's epilogue with the other's K loop; the two K = F
-    // products are better off with the larger tile
-    return (kid == MOLE_K_FFN_FWD2 || kid == MOLE_K_FFN_GX) ? 8 : 4;
+    (void)kid;
+    if (forced == 4 || forced == 8 || forced == 16) return forced;
+    return 16;
 }
 
 int launch_gemm256(const GemmArgs &g, bool a_ks, bool b_ks, bool wg, int epi, int max_rows, hipStream_t st, int kid) {
@@ -698,8 +723,9 @@ int launch_gemm256(const GemmArgs &g, bool a_ks, bool b_ks, bool wg, int epi, in
     if (!wg && (a_ks || g.K % Q_BK)) return -100;
     if (wg && (!a_ks || !b_ks || g.M % 8)) return -100;
     const int tmb = tile_blocks_for(kid);
-    if (tmb == 4) return dispatch256<4>(g, b_ks, wg, epi, max_rows, st, kid);
-    return dispatch256<8>(g, b_ks, wg, epi, max_rows, st, kid);
+    if (tmb == 4) return dispatch256<4, 1>(g, b_ks, wg, epi, max_rows, st, kid);
+    if (tmb == 16) return dispatch256<8, 2>(g, b_ks, wg, epi, max_rows, st, kid);   // 256 rows, eight waves
+    return dispatch256<8, 1>(g, b_ks, wg, epi, max_rows, st, kid);
 }
 
 }  // namespace mole
