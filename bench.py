@@ -32,8 +32,8 @@ PEAK_HBM_GBS = 8000.0
 # WRITE_SIZE runs of this script scaled by the same counters' readings for a copy of known size
 # (profiles/bench_c2_hbm_traffic.txt); other workloads have no counter run and report null
 MEASURED_TRAFFIC_BYTES = {
-    "c2": {"ffn_fwd1": 894.3e6, "ffn_fwd2": 464.0e6, "ffn_gw2": 335.7e6, "ffn_da": 854.2e6, "ffn_gw1": 335.7e6,
-           "ffn_gx": 463.8e6},
+    "c2": {"ffn_fwd1": 758.2e6, "ffn_fwd2": 460.7e6, "ffn_gw2": 537.2e6, "ffn_da": 745.0e6, "ffn_gw1": 537.2e6,
+           "ffn_gx": 460.5e6},
 }
 
 
