@@ -35,10 +35,11 @@ constexpr int Q_N_OPERAND = Q_BN * Q_BK * 2;   // bytes of the n-side tile of on
 template <int TMB, int WM> struct Tile {
     static constexpr int NW = 4 * WM, THREADS = 64 * NW, TMW = TMB / WM;
     static constexpr int BM = TMB * 32;
-    static constexpr int M_OPERAND = BM * Q_BK * 2;
+    static constexpr int M_ROWS = (BM + 16 * NW - 1) / (16 * NW) * (16 * NW);   // rows the waves' loads cover
+    static constexpr int M_OPERAND = M_ROWS * Q_BK * 2;
     static constexpr int STAGE = M_OPERAND + Q_N_OPERAND;
     static constexpr int NSTAGE = TMB >= 8 ? 4 : 3;
-    static constexpr int SLABS = 4 * BM * 128;                       // the waves' epilogue staging areas
+    static constexpr int SLABS = NW * TMW * 32 * 128;                // the waves' epilogue staging areas
     static constexpr int LDS_BYTES = NSTAGE * STAGE > SLABS ? NSTAGE * STAGE : SLABS;
     static constexpr int BLOCKS_PER_CU = TMB >= 8 ? 1 : 2;
 };
@@ -50,6 +51,7 @@ template <int TMB, int WM> struct Tile {
 template <int TMB, int WM, bool M_KS, int TMC> struct Stage {
     typedef Tile<TMB, WM> TL;
     static constexpr int RPL = 16 * TL::NW;                                       // rows (or 16-byte slot groups) one load of every wave covers
+    static_assert(!M_KS || TL::BM % RPL == 0, "a K-strided m-side tile must be whole load rounds wide");
     static constexpr int LM = M_KS ? TL::BM / RPL : (TMC * 32 + RPL - 1) / RPL;  // m-side loads per wave
     static constexpr int LN = Q_BN / RPL;
     static constexpr int L = LM + LN;                                             // loads per wave
@@ -202,9 +204,8 @@ template <bool KS, int ROWS> __device__ __forceinline__ bf16x8 frag(const char *
 // first index of part P when N items are dealt to NP consecutive parts
 template <int P, int NP, int N> constexpr int part_lo() { return P * N / NP; }
 
-// The fragments one wave needs for a k-sub-step: its TMCW live m-blocks (blocks wm*TMW .. of the tile, of which
-// the tile's first TMC are live) and its two 32-column n-blocks.  TMCW = 0: the wave has no live rows and
-// only takes part in the loads and barriers.
+// The fragments one wave needs for a k-sub-step: its TMCW m-blocks (blocks wm*TMCW .. of the tile, of which
+// the tile's first TMC are fetched) and its two 32-column n-blocks.
 template <int TMB, int WM, bool M_KS, bool N_KS, int TMC, int TMCW> struct Frags {
     typedef Tile<TMB, WM> TL;
     static constexpr int NR = TMCW ? TMCW + 2 : 0;
@@ -214,7 +215,7 @@ template <int TMB, int WM, bool M_KS, bool N_KS, int TMC, int TMCW> struct Frags
 #pragma unroll
         for (int r = part_lo<P, NP, NR>(); r < part_lo<P + 1, NP, NR>(); ++r) {
             if (r < 2) n[r] = frag<N_KS, Q_BN>(stage + Stage<TMB, WM, M_KS, TMC>::M_OPERAND, wn * 2 + r, kk);
-            else m[r - 2] = frag<M_KS, TL::BM>(stage, wm * TL::TMW + r - 2, kk);
+            else m[r - 2] = frag<M_KS, TL::BM>(stage, wm * TMCW + r - 2, kk);
         }
     }
     __device__ __forceinline__ void read(const char *stage, int wm, int wn, int kk) { read_part<0, 1>(stage, wm, wn, kk); }
@@ -235,7 +236,7 @@ template <int TMB, int WM, bool M_KS, bool N_KS, bool WG, int TMC> struct Feeder
     typedef Tile<TMB, WM> TL;
     typedef Stage<TMB, WM, M_KS, TMC> SG;
     static constexpr int LM = SG::LM, L = SG::L;
-    Off<TL::BM, TL::NW, M_KS> om, cm;
+    Off<TL::M_ROWS, TL::NW, M_KS> om, cm;
     Off<Q_BN, TL::NW, N_KS> on, cn;
     const char *bm, *bn;
     long step_m, step_n;
@@ -561,13 +562,17 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
     //      tiles is only known here (the grid is sized for the worst case), hence the device-side sum.
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n_tiles = (g.N + Q_BN - 1) / Q_BN;
-    int e, mt, nt, m_ext, k_ext;
+    int e, mt, nt, m_ext, k_ext, tile_h = Q_BM;   // tile_h: rows of this tile's m-tiles (row-ragged products cut experts evenly)
     long row0;  // first row of the expert
     if constexpr (!WG) {
-        // Heavy m-tiles (more than BM/2 live rows) take the first g.full_blocks block slots, in
-        // contiguous per-XCD ranges; the light ones (an expert's last tile with at most BM/2 rows)
-        // take the slots after them in plain order.  The hardware starts blocks in index order, so
-        // the short tiles fill the end of the launch instead of holding CUs for a full tile's time.
+        // An expert with r rows is cut into t = ceil(r / BM) m-tiles.  Where a launch is a single round of
+        // tiles (the 320-row configuration of the two K = F products) they have equal height h = r / t
+        // rounded up to whole 32-row blocks, so that no expert leaves a short remainder tile behind, which
+        // would run as a second, nearly empty round; elsewhere they are BM rows high and the last one is
+        // the remainder, which costs fewer MFMA blocks in total and fills in among the many rounds.  The
+        // m-tiles of all experts are numbered in expert order and each XCD takes a contiguous range of the
+        // real (m-tile, n-tile) pairs, so that neighbours share operands in its L2 and every XCD gets the
+        // same share; their number is only known here (the grid is sized for the worst case).
         const bool single = g.offsets == nullptr;
         auto rows_of = [&](int ee) { return single ? g.single_rows : g.kept[ee]; };
         const int nE = single ? 1 : g.E;
@@ -575,40 +580,22 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
         // dependent loads (the scan itself re-reads rows_of through the cache)
         const int rows_lane = lane < nE ? rows_of(lane) : 0;
         const int off_lane = (!single && lane < nE) ? g.offsets[lane] : 0;
-        int n_full = 0, n_part = 0;
-        for (int ee = lane; ee < nE; ee += WAVE) {
-            const int r = ee < WAVE ? rows_lane : rows_of(ee);
-            n_full += r / Q_BM + ((r % Q_BM) > Q_BM / 2);
-            n_part += (r % Q_BM) != 0 && (r % Q_BM) <= Q_BM / 2;
-        }
-        for (int d = WAVE / 2; d >= 1; d >>= 1) {
-            n_full += __shfl_xor(n_full, d, WAVE);
-            n_part += __shfl_xor(n_part, d, WAVE);
-        }
-        int target;            // index among the full (or partial) m-tiles
-        bool want_full;
-        if ((int)blockIdx.x < g.full_blocks) {
-            const int total = n_full * n_tiles;
-            const int per_xcd = (total + 7) >> 3;
-            const int slot = blockIdx.x >> 3;
-            const int t = (blockIdx.x & 7) * per_xcd + slot;
-            if (slot >= per_xcd || t >= total) return;
-            target = t / n_tiles;
-            nt = t % n_tiles;
-            want_full = true;
-        } else {
-            const int p = blockIdx.x - g.full_blocks;
-            if (p >= n_part * n_tiles) return;
-            target = p / n_tiles;
-            nt = p % n_tiles;
-            want_full = false;
-        }
+        int n_mt = 0;
+        for (int ee = lane; ee < nE; ee += WAVE) n_mt += ((ee < WAVE ? rows_lane : rows_of(ee)) + Q_BM - 1) / Q_BM;
+        for (int d = WAVE / 2; d >= 1; d >>= 1) n_mt += __shfl_xor(n_mt, d, WAVE);
+        const int total = n_mt * n_tiles;
+        const int per_xcd = (total + 7) >> 3;
+        const int slot = blockIdx.x >> 3;
+        const int t = (blockIdx.x & 7) * per_xcd + slot;
+        if (slot >= per_xcd || t >= total) return;
+        const int target = t / n_tiles;        // index among all m-tiles
+        nt = t % n_tiles;
         // the expert whose running count passes `target`
         int run = 0, found = -1, before = 0;
         for (int base = 0; base < nE && found < 0; base += WAVE) {
             const int ee = base + lane;
             const int r = base == 0 ? rows_lane : (ee < nE ? rows_of(ee) : 0);
-            const int cnt = want_full ? r / Q_BM + ((r % Q_BM) > Q_BM / 2) : ((r % Q_BM) != 0 && (r % Q_BM) <= Q_BM / 2);
+            const int cnt = (r + Q_BM - 1) / Q_BM;
             int incl = cnt;
             for (int d = 1; d < WAVE; d <<= 1) {
                 const int y = __shfl_up(incl, d, WAVE);
@@ -625,7 +612,9 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
         if (found < 0) return;
         e = found;
         m_ext = found < WAVE ? __shfl(rows_lane, found, WAVE) : rows_of(e);
-        mt = want_full ? target - before : m_ext / Q_BM;
+        mt = target - before;
+        const int t_e = (m_ext + Q_BM - 1) / Q_BM;
+        tile_h = TMB == 10 ? ((((m_ext + t_e - 1) / t_e) + 31) & ~31) : Q_BM;
         row0 = single ? 0 : (found < WAVE ? __shfl(off_lane, found, WAVE) : g.offsets[e]);
         k_ext = g.K;
     } else {
@@ -648,11 +637,12 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
     // (operand bases, LDS destinations, loop bounds) lives in scalar registers
     e = __builtin_amdgcn_readfirstlane(e);
     mt = __builtin_amdgcn_readfirstlane(mt);
+    tile_h = __builtin_amdgcn_readfirstlane(tile_h);
     nt = __builtin_amdgcn_readfirstlane(nt);
     m_ext = __builtin_amdgcn_readfirstlane(m_ext);
     k_ext = __builtin_amdgcn_readfirstlane(k_ext);
     row0 = ((long)__builtin_amdgcn_readfirstlane((int)(row0 >> 32)) << 32) | (unsigned)__builtin_amdgcn_readfirstlane((int)row0);
-    const int m0 = mt * Q_BM, n0 = nt * Q_BN;
+    const int m0 = mt * tile_h, n0 = nt * Q_BN;
     const bf16_t *Mp = (const bf16_t *)g.A + row0 * g.lda;
     const bf16_t *Np = WG ? (const bf16_t *)g.B + row0 * g.ldb : (const bf16_t *)g.B + (long)e * g.strideB;
 
@@ -664,32 +654,33 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
 #pragma unroll
             for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
 
-    const int live = min(Q_BM, m_ext - m0);
+    const int live = min(tile_h, m_ext - m0);
     const int tmc = (live + 31) >> 5;
     const int wu = __builtin_amdgcn_readfirstlane(wave);
     const int wm = WM == 1 ? 0 : wu >> 2, wn = wu & 3;     // wave row / wave column
     uint2 bias_raw[8];
     load_bias<EPI>(g, e, n0, lane, wn, bias_raw);
+    // The live blocks are dealt evenly to the wave rows: c to each (the last row may find fewer live).
+    const int c = (tmc + WM - 1) / WM;
+    const int m0w = m0 + wm * c * 32, live_w = max(0, min(live - wm * c * 32, c * 32));
     PreAct<TMB, WM, EPI> pre;
-    pre.load(g, row0, m0 + wm * TMW * 32, n0, live - wm * TMW * 32, lane, wn);
-    // K loop and epilogue for a tile whose first TMC blocks are live; the wave's share is CW of them
-#define MOLE_RUN_TILE(TMC)                                                                                                \
-    if (WM == 1 || wm == 0) {                                                                                             \
-        constexpr int CW = (TMC) < TMW ? (TMC) : TMW;                                                                     \
-        main_loop<TMB, WM, M_KS, N_KS, WG, (TMC), CW>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wu, 0, wn, acc); \
-        epilogue<TMB, WM, WG, EPI, CW>(g, acc, smem, lane, wu, wn, e, row0, m0, n0, m_ext, min(live, TMW * 32), bias_raw, pre); \
-    } else {                                                                                                              \
-        constexpr int CW = (TMC) > TMW ? (TMC) - TMW : 0;                                                                 \
-        main_loop<TMB, WM, M_KS, N_KS, WG, (TMC), CW>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wu, 1, wn, acc); \
-        epilogue<TMB, WM, WG, EPI, CW>(g, acc, smem, lane, wu, wn, e, row0, m0 + TMW * 32, n0, m_ext, live - TMW * 32,    \
-                                       bias_raw, pre);                                                                    \
+    pre.load(g, row0, m0w, n0, live_w, lane, wn);
+    // K loop and epilogue with C blocks per wave row
+#define MOLE_RUN_TILE(C)                                                                                                  \
+    {                                                                                                                     \
+        main_loop<TMB, WM, M_KS, N_KS, WG, WM *(C), (C)>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wu, wm, wn, acc); \
+        epilogue<TMB, WM, WG, EPI, (C)>(g, acc, smem, lane, wu, wn, e, row0, m0w, n0, m_ext, live_w, bias_raw, pre);      \
     }
-    if (tmc > TMB / 2) {
-        MOLE_RUN_TILE(TMB)
-    } else if (tmc > TMB / 4) {
-        MOLE_RUN_TILE(TMB / 2)
+    if constexpr (WM == 1) {
+        if (c > TMB / 2) MOLE_RUN_TILE(TMB)
+        else if (c > TMB / 4) MOLE_RUN_TILE(TMB / 2)
+        else MOLE_RUN_TILE(TMB / 4)
     } else {
-        MOLE_RUN_TILE(TMB / 4)
+        if (c >= TMW) MOLE_RUN_TILE(TMW)
+        else if (TMW > 4 && c == 4) MOLE_RUN_TILE(TMW > 4 ? 4 : 1)
+        else if (c == 3) MOLE_RUN_TILE(3)
+        else if (c == 2) MOLE_RUN_TILE(2)
+        else MOLE_RUN_TILE(1)
     }
 #undef MOLE_RUN_TILE
 }
@@ -716,21 +707,24 @@ template <int TMB, int WM>
 static int dispatch256(const GemmArgs &g, bool b_ks, bool wg, int epi, int max_rows, hipStream_t st, int kid) {
     constexpr int BM = Tile<TMB, WM>::BM;
     const int n_tiles = ceil_div(g.N, Q_BN);
-    if (wg) {
-        const int tiles = 8 * ceil_div(g.E * ceil_div(g.M, BM), 8) * n_tiles;   // whole (expert, m-tile) units per XCD
-        if (epi == EPI_WGRAD) return launch256<TMB, WM, true, true, EPI_WGRAD>(g, tiles, st, kid);
-        return -100;
+    if constexpr (TMB != 10) {
+        if (wg) {
+            const int tiles = 8 * ceil_div(g.E * ceil_div(g.M, BM), 8) * n_tiles;   // whole (expert, m-tile) units per XCD
+            if (epi == EPI_WGRAD) return launch256<TMB, WM, true, true, EPI_WGRAD>(g, tiles, st, kid);
+            return -100;
+        }
     }
-    // block slots: worst-case number of heavy m-tiles (each has more than BM/2 rows; rounded to the
-    // 8 XCDs), then at most one light m-tile per expert
+    // block slots: the worst-case number of m-tiles (an expert with r rows has ceil(r / BM) of them)
     const int rows_bound = g.offsets ? max_rows : g.single_rows;
     GemmArgs gg = g;
-    gg.full_blocks = ((rows_bound / (BM / 2)) * n_tiles + 7) & ~7;
-    const int tiles = gg.full_blocks + (g.offsets ? g.E : 1) * n_tiles;
+    const int tiles = ((rows_bound / BM + (g.offsets ? g.E : 1)) * n_tiles + 7) & ~7;
+    if (wg) return -100;
     if (!b_ks) {
-        if (epi == EPI_BIAS_GELU) return launch256<TMB, WM, false, false, EPI_BIAS_GELU>(gg, tiles, st, kid);
-        if (epi == EPI_DGELU) return launch256<TMB, WM, false, false, EPI_DGELU>(gg, tiles, st, kid);
-        if (epi == EPI_F32) return launch256<TMB, WM, false, false, EPI_F32>(gg, tiles, st, kid);
+        if constexpr (TMB != 10) {
+            if (epi == EPI_BIAS_GELU) return launch256<TMB, WM, false, false, EPI_BIAS_GELU>(gg, tiles, st, kid);
+            if (epi == EPI_DGELU) return launch256<TMB, WM, false, false, EPI_DGELU>(gg, tiles, st, kid);
+            if (epi == EPI_F32) return launch256<TMB, WM, false, false, EPI_F32>(gg, tiles, st, kid);
+        }
     } else {
         if (epi == EPI_BIAS) return launch256<TMB, WM, true, false, EPI_BIAS>(gg, tiles, st, kid);
         if (epi == EPI_STORE) return launch256<TMB, WM, true, false, EPI_STORE>(gg, tiles, st, kid);
@@ -738,17 +732,19 @@ static int dispatch256(const GemmArgs &g, bool b_ks, bool wg, int epi, int max_r
     return -100;
 }
 
-// Tile configuration: 256 rows on eight waves for every product (two waves per SIMD hide each other's
-// waits; one fetch of the n-side tile serves all 256 rows).  MOLE_TMB=4|8 in the environment selects the
-// four-wave variants with 128 or 256 rows instead (tuning aid).
+// Tile configuration.  Eight waves (two per SIMD hide each other's waits; one fetch of the n-side tile
+// serves all rows of the tile) for every product: 256-row tiles, and tiles of up to 320 rows for the two
+// products with a light epilogue (out = a.w2 + b2 and gx = t.w1), whose register budget allows 160
+// accumulators a wave: with a capacity factor of 1.25 an expert then never needs more m-tiles than the
+// average one, and the launch stays one round of tiles.  MOLE_TMB=4|8 in the environment selects the
+// four-wave variants with 128 or 256 rows, 16 the 256-row eight-wave tile for everything (tuning aid).
 static int tile_blocks_for(int kid) {
     static const int forced = [] {
         const char *v = getenv("MOLE_TMB");
         return v ? atoi(v) : 0;
     }();
-    (void)kid;
     if (forced == 4 || forced == 8 || forced == 16) return forced;
-    return 16;
+    return (kid == MOLE_K_FFN_FWD2 || kid == MOLE_K_FFN_GX) ? 20 : 16;
 }
 
 int launch_gemm256(const GemmArgs &g, bool a_ks, bool b_ks, bool wg, int epi, int max_rows, hipStream_t st, int kid) {
@@ -759,6 +755,8 @@ int launch_gemm256(const GemmArgs &g, bool a_ks, bool b_ks, bool wg, int epi, in
     const int tmb = tile_blocks_for(kid);
     if (tmb == 4) return dispatch256<4, 1>(g, b_ks, wg, epi, max_rows, st, kid);
     if (tmb == 16) return dispatch256<8, 2>(g, b_ks, wg, epi, max_rows, st, kid);   // 256 rows, eight waves
+    if (tmb == 20 && !wg && b_ks) return dispatch256<10, 2>(g, b_ks, wg, epi, max_rows, st, kid);   // up to 320 rows, eight waves
+    if (tmb == 20) return dispatch256<8, 2>(g, b_ks, wg, epi, max_rows, st, kid);
     return dispatch256<8, 1>(g, b_ks, wg, epi, max_rows, st, kid);
 }
 
