@@ -84,6 +84,12 @@ int mole_kernel_timing_read(int n_ids, int *counts, float *ms_total);
  * ------------------------------------------------------------------------------------------ */
 int mole_softmax_fwd(const float *logits, const float *logit_bias, int S, int E, float *scores,
                      mole_stream_t stream);
+/* The whole of MOLETopk.forward (MOLE/utils/Ugate.py:11-14) in one kernel for bf16 tokens:
+ * scores[S,E] = softmax(x[S,M] . wg[E,M]^T + logit_bias), wg fp32 (rounded to bf16 for the products, fp32
+ * accumulation), logit_bias [E] or NULL.  Needs dtype == MOLE_BF16, M a multiple of 128, E <= 256; other
+ * cases use mole_gemm_nt + mole_softmax_fwd. */
+int mole_gate_fwd(const void *x, int dtype, const float *wg, const float *logit_bias, int S, int E, int M,
+                  float *scores, mole_stream_t stream);
 int mole_gate_bwd(const float *dgates, const float *scores, const int32_t *idx, int S, int E,
                   int k, int normalize_gate, int through_softmax, float *dout, mole_stream_t stream);
 /* Gradient of the gate's Linear (MOLE/utils/Ugate.py:12, run by autograd in the reference):

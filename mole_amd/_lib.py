@@ -28,6 +28,7 @@ _SIGNATURES = {
     "mole_kernel_timing_enable": (c_int, [c_int]),
     "mole_kernel_timing_read": (c_int, [c_int, POINTER(c_int), POINTER(c_float)]),
     "mole_softmax_fwd": (c_int, [_P, _P, c_int, c_int, _P, _P]),
+    "mole_gate_fwd": (c_int, [_P, c_int, _P, _P, c_int, c_int, c_int, _P, _P]),
     "mole_gate_bwd": (c_int, [_P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P, _P]),
     "mole_gate_wgrad_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "mole_gate_wgrad": (c_int, [_P, _P, c_int, c_int, c_int, c_int, _P, _P, c_size_t, _P]),

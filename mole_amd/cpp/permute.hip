@@ -230,15 +230,16 @@ __global__ __launch_bounds__(256) void gate_wgrad_partial_kernel(const float *__
         if (e < E)
             *reinterpret_cast<float2 *>(part + ((size_t)blockIdx.x * E + e) * M + m) = make_float2(acc[e][0], acc[e][1]);
 }
-// sums the partials in a fixed order: 4 slices of the block list per output, then the slices in order
+// sums the partials in a fixed order: 16 slices of the block list per group of four outputs, then the
+// slices in order
 __global__ __launch_bounds__(256) void gate_wgrad_reduce_kernel(const float *__restrict__ part, int nblocks, int EM,
                                                                 float *__restrict__ dwg) {
-    __shared__ float4 s_acc[4][64];
-    const int o = threadIdx.x & 63, slice = threadIdx.x >> 6;
-    const int idx = (blockIdx.x * 64 + o) * 4;
+    __shared__ float4 s_acc[16][16];
+    const int o = threadIdx.x & 15, slice = threadIdx.x >> 4;
+    const int idx = (blockIdx.x * 16 + o) * 4;
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
     if (idx < EM) {
-        const int per = (nblocks + 3) / 4;
+        const int per = (nblocks + 15) / 16;
         const int b1 = min(nblocks, (slice + 1) * per);
         for (int b = slice * per; b < b1; ++b) {
             const float4 v = *reinterpret_cast<const float4 *>(part + (size_t)b * EM + idx);
@@ -250,7 +251,7 @@ __global__ __launch_bounds__(256) void gate_wgrad_reduce_kernel(const float *__r
     if (slice == 0 && idx < EM) {
         float4 r = s_acc[0][o];
 #pragma unroll
-        for (int sl = 1; sl < 4; ++sl) { r.x += s_acc[sl][o].x; r.y += s_acc[sl][o].y; r.z += s_acc[sl][o].z; r.w += s_acc[sl][o].w; }
+        for (int sl = 1; sl < 16; ++sl) { r.x += s_acc[sl][o].x; r.y += s_acc[sl][o].y; r.z += s_acc[sl][o].z; r.w += s_acc[sl][o].w; }
         *reinterpret_cast<float4 *>(dwg + idx) = r;
     }
 }
@@ -442,7 +443,7 @@ extern "C" int mole_gate_wgrad(const float *dlogits, const void *x, int dtype, i
     }
 #undef MOLE_GW
     MOLE_LAUNCH_CHECK();
-    hipLaunchKernelGGL(gate_wgrad_reduce_kernel, dim3(ceil_div(E * M, 256)), dim3(256), 0, st, part, nb, E * M, dwg);
+    hipLaunchKernelGGL(gate_wgrad_reduce_kernel, dim3(ceil_div(E * M, 64)), dim3(256), 0, st, part, nb, E * M, dwg);
     MOLE_LAUNCH_CHECK();
     return 0;
 }

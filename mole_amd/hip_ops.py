@@ -46,6 +46,21 @@ def softmax_fwd(logits: torch.Tensor, logit_bias: Optional[torch.Tensor] = None)
     return scores
 
 
+def gate_fwd(x: torch.Tensor, wg: torch.Tensor, logit_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """scores [S,E] fp32 = softmax(x @ wg.T + logit_bias): one fused kernel for bf16 tokens (M % 128 == 0, E <= 256),
+    the NT GEMM followed by the softmax kernel otherwise."""
+    _dev(x), _dev(wg)
+    S, M = x.shape
+    E = wg.shape[0]
+    if x.dtype == torch.bfloat16 and wg.dtype == torch.float32 and M % 128 == 0 and E <= 256:
+        scores = torch.empty(S, E, dtype=torch.float32, device=x.device)
+        L.check(L.lib().mole_gate_fwd(L.ptr(x), L.dtype_code(x.dtype), L.ptr(wg), L.ptr(logit_bias), S, E, M, L.ptr(scores),
+                                      L.stream()), "mole_gate_fwd")
+        return scores
+    w = wg if wg.dtype == x.dtype else wg.to(x.dtype)
+    return softmax_fwd(gemm_nt(x, w.contiguous()), logit_bias)
+
+
 def gate_bwd(dgates: torch.Tensor, scores: torch.Tensor, idx: torch.Tensor, normalize_gate: bool,
              through_softmax: bool = True) -> torch.Tensor:
     """d(logits) (through_softmax) or d(scores) from d(gates)."""

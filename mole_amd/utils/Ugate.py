@@ -1,8 +1,9 @@
 """Gate of the MoE layer: Linear without bias, softmax over experts.
 
-Mirror of MOLE/utils/Ugate.py:5-14 (same class name, same `linear` attribute).  The logits come from
-the MFMA NT GEMM of the C ABI (mole_gemm_nt), the softmax from mole_softmax_fwd; the backward is the
-textbook softmax/linear backward on device tensors.  `logit_bias` ([E], optional, not trained) is
+Mirror of MOLE/utils/Ugate.py:5-14 (same class name, same `linear` attribute).  For bf16 tokens the scores
+come from one fused kernel of the C ABI (mole_gate_fwd); otherwise the logits come from the MFMA NT GEMM
+(mole_gemm_nt) and the softmax from mole_softmax_fwd.  The backward is the textbook softmax/linear
+backward on device tensors.  `logit_bias` ([E], optional, not trained) is
 added to the logits before the softmax - the reference gate has none.
 """
 import torch
@@ -28,11 +29,7 @@ class _GateFn(torch.autograd.Function):
 
 def gate_scores(x: torch.Tensor, weight: torch.Tensor, logit_bias=None) -> torch.Tensor:
     """softmax(x @ weight.T + logit_bias) in fp32; x [S,M] fp32 or bf16, weight [E,M] fp32."""
-    w = weight.detach()
-    if w.dtype != x.dtype:
-        w = w.to(x.dtype)
-    logits = H.gemm_nt(x.detach().contiguous(), w.contiguous())
-    return H.softmax_fwd(logits, logit_bias)
+    return H.gate_fwd(x.detach().contiguous(), weight.detach().contiguous(), logit_bias)
 
 
 class MOLETopk(torch.nn.Module):

@@ -94,3 +94,23 @@ def test_gate_wgrad(S, E, M, dtype):
     got = H.gate_wgrad(dl.cuda(), x.cuda())
     want = dl.double().t() @ x.double()
     assert rel_err(got, want) < 1e-5       # fp32 sums of exact products in both dtypes
+
+
+@pytest.mark.parametrize("S,E,M,bias", [(100, 16, 128, False), (1000, 8, 256, True), (513, 64, 384, False),
+                                        (300, 256, 1024, True), (64, 100, 128, True), (16384, 16, 1024, False)])
+def test_fused_gate_forward(S, E, M, bias):
+    """mole_gate_fwd (bf16 tokens) against the oracle's gate on the same rounded operands, and against the
+    unfused GEMM + softmax path it replaces."""
+    from mole_amd import hip_ops as H
+    print(f"gate_fwd S={S} E={E} M={M} bias={bias}", flush=True)
+    g = torch.Generator().manual_seed(S + E)
+    x = torch.randn(S, M, generator=g).bfloat16()
+    wg = torch.randn(E, M, generator=g) * 0.05
+    b = torch.log(torch.arange(1, E + 1, dtype=torch.float32) ** -1.2) if bias else None
+    got = H.gate_fwd(x.cuda(), wg.cuda(), b.cuda() if bias else None).cpu()
+    want = O.gate_scores(x.float(), wg.bfloat16().float(), b)
+    assert got.shape == (S, E)
+    assert rel_err(got, want) < 1e-4
+    assert float((got.sum(-1) - 1).abs().max()) < 1e-5
+    unfused = H.softmax_fwd(H.gemm_nt(x.cuda(), wg.bfloat16().cuda()), b.cuda() if bias else None).cpu()
+    assert rel_err(got, unfused) < 1e-5
