@@ -144,35 +144,54 @@ __global__ __launch_bounds__(256) void dispatch_bwd_gate_kernel(const T *__restr
         w[e][0] = v.x; w[e][1] = v.y; w[e][2] = v.z; w[e][3] = v.w;
     }
     const int i0 = blockIdx.x * DB_TOKENS, i1 = min(i0 + DB_TOKENS, S);
-    for (int i = i0; i < i1; ++i) {
-        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    constexpr int U = 8;      // tokens whose row gathers are in flight together: one at a time runs at the memory latency
+    for (int ib = i0; ib < i1; ib += U) {
+        float acc[U][4];
+#pragma unroll
+        for (int u = 0; u < U; ++u) acc[u][0] = acc[u][1] = acc[u][2] = acc[u][3] = 0.f;
         for (int j = 0; j < k; ++j) {
-            const int r = row[(size_t)j * S + i];
-            if (r < 0) continue;
+            int r[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) r[u] = ib + u < i1 ? row[(size_t)j * S + ib + u] : -1;
             if constexpr (sizeof(T) == 2) {
-                const uint2 v = *reinterpret_cast<const uint2 *>(dxd + (size_t)r * M + m);
-                acc[0] += __uint_as_float(v.x << 16); acc[1] += __uint_as_float(v.x & 0xffff0000u);
-                acc[2] += __uint_as_float(v.y << 16); acc[3] += __uint_as_float(v.y & 0xffff0000u);
+                uint2 v[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    v[u] = r[u] >= 0 ? *reinterpret_cast<const uint2 *>(dxd + (size_t)r[u] * M + m) : make_uint2(0, 0);
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    acc[u][0] += __uint_as_float(v[u].x << 16); acc[u][1] += __uint_as_float(v[u].x & 0xffff0000u);
+                    acc[u][2] += __uint_as_float(v[u].y << 16); acc[u][3] += __uint_as_float(v[u].y & 0xffff0000u);
+                }
             } else {
-                const float4 v = *reinterpret_cast<const float4 *>(dxd + (size_t)r * M + m);
-                acc[0] += v.x; acc[1] += v.y; acc[2] += v.z; acc[3] += v.w;
+                float4 v[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    v[u] = r[u] >= 0 ? *reinterpret_cast<const float4 *>(dxd + (size_t)r[u] * M + m) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+                for (int u = 0; u < U; ++u) { acc[u][0] += v[u].x; acc[u][1] += v[u].y; acc[u][2] += v[u].z; acc[u][3] += v[u].w; }
             }
         }
-        const float *dl = dlogits + (size_t)i * E;
 #pragma unroll
-        for (int e = 0; e < EB; ++e) {
-            const float d = e < E ? dl[e] : 0.f;
+        for (int u = 0; u < U; ++u) {
+            const int i = ib + u;
+            if (i >= i1) break;
+            const float *dl = dlogits + (size_t)i * E;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) acc[q] += d * w[e][q];
-        }
-        if constexpr (sizeof(T) == 2) {
-            const bf16_t b0 = (bf16_t)acc[0], b1 = (bf16_t)acc[1], b2 = (bf16_t)acc[2], b3 = (bf16_t)acc[3];
-            uint2 o;
-            o.x = (uint32_t)__builtin_bit_cast(uint16_t, b0) | ((uint32_t)__builtin_bit_cast(uint16_t, b1) << 16);
-            o.y = (uint32_t)__builtin_bit_cast(uint16_t, b2) | ((uint32_t)__builtin_bit_cast(uint16_t, b3) << 16);
-            *reinterpret_cast<uint2 *>(dx + (size_t)i * M + m) = o;
-        } else {
-            *reinterpret_cast<float4 *>(dx + (size_t)i * M + m) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+            for (int e = 0; e < EB; ++e) {
+                const float d = e < E ? dl[e] : 0.f;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) acc[u][q] += d * w[e][q];
+            }
+            if constexpr (sizeof(T) == 2) {
+                const bf16_t b0 = (bf16_t)acc[u][0], b1 = (bf16_t)acc[u][1], b2 = (bf16_t)acc[u][2], b3 = (bf16_t)acc[u][3];
+                uint2 o;
+                o.x = (uint32_t)__builtin_bit_cast(uint16_t, b0) | ((uint32_t)__builtin_bit_cast(uint16_t, b1) << 16);
+                o.y = (uint32_t)__builtin_bit_cast(uint16_t, b2) | ((uint32_t)__builtin_bit_cast(uint16_t, b3) << 16);
+                *reinterpret_cast<uint2 *>(dx + (size_t)i * M + m) = o;
+            } else {
+                *reinterpret_cast<float4 *>(dx + (size_t)i * M + m) = make_float4(acc[u][0], acc[u][1], acc[u][2], acc[u][3]);
+            }
         }
     }
 }
