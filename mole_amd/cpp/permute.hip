@@ -7,6 +7,8 @@
 // written k times (dispatch), or k rows are read and one written (combine); all sums are fp32.
 #include "common.h"
 
+#include <type_traits>
+
 namespace mole {
 
 template <typename T> struct Vec;  // 16 bytes of T
@@ -144,33 +146,38 @@ __global__ __launch_bounds__(256) void dispatch_bwd_gate_kernel(const T *__restr
         w[e][0] = v.x; w[e][1] = v.y; w[e][2] = v.z; w[e][3] = v.w;
     }
     const int i0 = blockIdx.x * DB_TOKENS, i1 = min(i0 + DB_TOKENS, S);
-    constexpr int U = 8;      // tokens whose row gathers are in flight together: one at a time runs at the memory latency
-    for (int ib = i0; ib < i1; ib += U) {
+    // Eight tokens per batch; the first choice's row gathers of the next batch are in flight while the
+    // current batch is finished: one token at a time, or one batch at a time, runs at the memory latency.
+    constexpr int U = 8;
+    typedef typename std::conditional<sizeof(T) == 2, uint2, float4>::type Raw;
+    auto gather = [&](Raw (&v)[U], int ib, int j) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int r = ib + u < i1 ? row[(size_t)j * S + ib + u] : -1;
+            if constexpr (sizeof(T) == 2) v[u] = r >= 0 ? *reinterpret_cast<const uint2 *>(dxd + (size_t)r * M + m) : make_uint2(0, 0);
+            else v[u] = r >= 0 ? *reinterpret_cast<const float4 *>(dxd + (size_t)r * M + m) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    };
+    auto add = [&](float (&acc)[U][4], const Raw (&v)[U]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if constexpr (sizeof(T) == 2) {
+                acc[u][0] += __uint_as_float(v[u].x << 16); acc[u][1] += __uint_as_float(v[u].x & 0xffff0000u);
+                acc[u][2] += __uint_as_float(v[u].y << 16); acc[u][3] += __uint_as_float(v[u].y & 0xffff0000u);
+            } else {
+                acc[u][0] += v[u].x; acc[u][1] += v[u].y; acc[u][2] += v[u].z; acc[u][3] += v[u].w;
+            }
+        }
+    };
+    auto finish = [&](const Raw (&first)[U], int ib) __attribute__((always_inline)) {
         float acc[U][4];
 #pragma unroll
         for (int u = 0; u < U; ++u) acc[u][0] = acc[u][1] = acc[u][2] = acc[u][3] = 0.f;
-        for (int j = 0; j < k; ++j) {
-            int r[U];
-#pragma unroll
-            for (int u = 0; u < U; ++u) r[u] = ib + u < i1 ? row[(size_t)j * S + ib + u] : -1;
-            if constexpr (sizeof(T) == 2) {
-                uint2 v[U];
-#pragma unroll
-                for (int u = 0; u < U; ++u)
-                    v[u] = r[u] >= 0 ? *reinterpret_cast<const uint2 *>(dxd + (size_t)r[u] * M + m) : make_uint2(0, 0);
-#pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    acc[u][0] += __uint_as_float(v[u].x << 16); acc[u][1] += __uint_as_float(v[u].x & 0xffff0000u);
-                    acc[u][2] += __uint_as_float(v[u].y << 16); acc[u][3] += __uint_as_float(v[u].y & 0xffff0000u);
-                }
-            } else {
-                float4 v[U];
-#pragma unroll
-                for (int u = 0; u < U; ++u)
-                    v[u] = r[u] >= 0 ? *reinterpret_cast<const float4 *>(dxd + (size_t)r[u] * M + m) : make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll
-                for (int u = 0; u < U; ++u) { acc[u][0] += v[u].x; acc[u][1] += v[u].y; acc[u][2] += v[u].z; acc[u][3] += v[u].w; }
-            }
+        add(acc, first);
+        for (int j = 1; j < k; ++j) {
+            Raw v[U];
+            gather(v, ib, j);
+            add(acc, v);
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -193,6 +200,14 @@ __global__ __launch_bounds__(256) void dispatch_bwd_gate_kernel(const T *__restr
                 *reinterpret_cast<float4 *>(dx + (size_t)i * M + m) = make_float4(acc[u][0], acc[u][1], acc[u][2], acc[u][3]);
             }
         }
+    };
+    Raw va[U], vb[U];
+    gather(va, i0, 0);
+    for (int ib = i0; ib < i1; ib += 2 * U) {
+        gather(vb, ib + U, 0);
+        finish(va, ib);
+        gather(va, ib + 2 * U, 0);
+        if (ib + U < i1) finish(vb, ib + U);
     }
 }
 
@@ -218,10 +233,10 @@ __global__ __launch_bounds__(256) void gate_wgrad_partial_kernel(const float *__
 #pragma unroll
     for (int e = 0; e < EB; ++e) acc[e][0] = acc[e][1] = 0.f;
     const T *px = x + (size_t)i0 * M + m;
-    for (int t0 = 0; t0 < nt; t0 += 8) {
-        float xv[8][2];
+    // eight rows per batch, the next batch's loads in flight while the current one is used
+    auto load8 = [&](float (&xv)[8][2], int t0) __attribute__((always_inline)) {
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {       // 8 rows in flight
+        for (int u = 0; u < 8; ++u) {
             const int t = min(t0 + u, nt - 1);
             if constexpr (sizeof(T) == 2) {
                 const uint32_t v = *reinterpret_cast<const uint32_t *>(px + (size_t)t * M);
@@ -231,6 +246,8 @@ __global__ __launch_bounds__(256) void gate_wgrad_partial_kernel(const float *__
                 xv[u][0] = v.x; xv[u][1] = v.y;
             }
         }
+    };
+    auto use8 = [&](const float (&xv)[8][2], int t0) __attribute__((always_inline)) {
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             if (t0 + u >= nt) break;
@@ -243,6 +260,14 @@ __global__ __launch_bounds__(256) void gate_wgrad_partial_kernel(const float *__
                 acc[e + 3][0] += d.w * xv[u][0]; acc[e + 3][1] += d.w * xv[u][1];
             }
         }
+    };
+    float xa[8][2], xb[8][2];
+    load8(xa, 0);
+    for (int t0 = 0; t0 < nt; t0 += 16) {
+        load8(xb, t0 + 8);
+        use8(xa, t0);
+        load8(xa, t0 + 16);
+        use8(xb, t0 + 8);
     }
 #pragma unroll
     for (int e = 0; e < EB; ++e)
