@@ -118,10 +118,12 @@ int mole_gate_wgrad(const float *dlogits, const void *x, int dtype, int S, int E
  *   l_aux    [1]   fp32  out   E/S^2 * sum_e (sum_i scores[i,e]) * counts[0,e]; may be NULL
  *
  * capacity_factor > 0: C = k*int(cf*ceil(S/E)); == 0: C = max(loc)+1; < 0: the smaller of both;
- * C is then rounded up to `alignment`.  k is clipped to E by the caller (k <= E required).
+ * C is then rounded up to `alignment`.  The factor is a double and the product is taken in double precision,
+ * like the Python expression it replaces (0.02 * 50 must give 1, which single precision does not).
+ * k is clipped to E by the caller (k <= E required).
  * ------------------------------------------------------------------------------------------ */
 size_t mole_route_workspace_bytes(int S, int E, int k);
-int mole_route(const float *scores, int S, int E, int k, float capacity_factor, int normalize_gate,
+int mole_route(const float *scores, int S, int E, int k, double capacity_factor, int normalize_gate,
                int alignment, int layout, int32_t *idx, int32_t *loc, float *gates, int32_t *row,
                int32_t *counts, int32_t *kept_rows, int32_t *offsets, int32_t *capacity,
                float *l_aux, void *workspace, size_t workspace_bytes, mole_stream_t stream);

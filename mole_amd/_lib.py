@@ -8,7 +8,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import POINTER, c_char_p, c_float, c_int, c_int32, c_int64, c_size_t, c_uint64, c_void_p
+from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_int32, c_int64, c_size_t, c_uint64, c_void_p
 
 import torch  # noqa: F401  (must precede the dlopen below)
 
@@ -33,7 +33,7 @@ _SIGNATURES = {
     "mole_gate_wgrad_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "mole_gate_wgrad": (c_int, [_P, _P, c_int, c_int, c_int, c_int, _P, _P, c_size_t, _P]),
     "mole_route_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
-    "mole_route": (c_int, [_P, c_int, c_int, c_int, c_float, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P,
+    "mole_route": (c_int, [_P, c_int, c_int, c_int, c_double, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P,
                            _P, _P, c_size_t, _P]),
     "mole_dispatch_fwd": (c_int, [_P, c_int, _P, c_int, c_int, c_int, _P, _P]),
     "mole_dispatch_bwd": (c_int, [_P, c_int, _P, c_int, c_int, c_int, _P, _P, c_int, _P, _P, _P]),

@@ -293,7 +293,7 @@ static void launch_topk(const float *scores, int S, int E, int k, int logG, int 
                        normalize, idx, loc, gates, hist, colsum, nb);
 }
 
-extern "C" int mole_route(const float *scores, int S, int E, int k, float capacity_factor, int normalize_gate,
+extern "C" int mole_route(const float *scores, int S, int E, int k, double capacity_factor, int normalize_gate,
                           int alignment, int layout, int32_t *idx, int32_t *loc, float *gates, int32_t *row,
                           int32_t *counts, int32_t *kept_rows, int32_t *offsets, int32_t *capacity,
                           float *l_aux, void *workspace, size_t workspace_bytes, mole_stream_t stream) {
@@ -335,9 +335,9 @@ extern "C" int mole_route(const float *scores, int S, int E, int k, float capaci
     MOLE_LAUNCH_CHECK();
 
     const int spe = (S + E - 1) / E;
-    const int cf_sign = capacity_factor > 0.f ? 1 : (capacity_factor < 0.f ? -1 : 0);
+    const int cf_sign = capacity_factor > 0. ? 1 : (capacity_factor < 0. ? -1 : 0);
     // int(cf * spe) of the Python reference: the product is taken in double precision
-    const double prod = (double)(capacity_factor < 0.f ? -capacity_factor : capacity_factor) * (double)spe;
+    const double prod = (capacity_factor < 0. ? -capacity_factor : capacity_factor) * (double)spe;
     const int cap_bound = k * (int)prod;
     hipLaunchKernelGGL(route_finish_kernel, dim3(1), dim3(FIN_THREADS), 0, st, counts, colsum, nb, S, E, k, cf_sign,
                        cap_bound, alignment, layout, basej, kept_rows, offsets, capacity, l_aux);

@@ -140,6 +140,8 @@ def dispatch_fwd(x: torch.Tensor, row: torch.Tensor, total_rows: int, out: Optio
     S, M = x.shape
     k = row.shape[0]
     xd = out if out is not None else torch.empty(total_rows, M, dtype=x.dtype, device=x.device)
+    if xd.numel() == 0:          # every pair was dropped: nothing to scatter
+        return xd
     L.check(L.lib().mole_dispatch_fwd(L.ptr(x), L.dtype_code(x.dtype), L.ptr(row), S, M, k, L.ptr(xd), L.stream()),
             "mole_dispatch_fwd")
     return xd
@@ -173,6 +175,8 @@ def combine_fwd(o: torch.Tensor, row: torch.Tensor, gates: torch.Tensor) -> torc
     _dev(o), _dev(row), _dev(gates)
     k, S = row.shape
     M = o.shape[-1]
+    if o.numel() == 0:           # every pair was dropped: all tokens output zeros
+        return torch.zeros(S, M, dtype=o.dtype, device=o.device)
     y = torch.empty(S, M, dtype=o.dtype, device=o.device)
     L.check(L.lib().mole_combine_fwd(L.ptr(o), L.dtype_code(o.dtype), L.ptr(row), L.ptr(gates), S, M, k, L.ptr(y), L.stream()),
             "mole_combine_fwd")
@@ -186,6 +190,8 @@ def combine_bwd(dy: torch.Tensor, o: torch.Tensor, row: torch.Tensor, gates: tor
     M = o.shape[-1]
     if d_o is None:
         d_o = torch.empty_like(o)
+    if o.numel() == 0:
+        return d_o, torch.zeros(k, S, dtype=torch.float32, device=o.device)
     dgates = torch.empty(k, S, dtype=torch.float32, device=o.device)
     L.check(L.lib().mole_combine_bwd(L.ptr(dy), L.ptr(o), L.dtype_code(o.dtype), L.ptr(row), L.ptr(gates), S, M, k,
                                      L.ptr(d_o), L.ptr(dgates), L.stream()), "mole_combine_bwd")

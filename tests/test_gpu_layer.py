@@ -172,3 +172,27 @@ def test_fast_assign_prefetch_matches_oracle():
         n = int(rng.integers(1, 8)); P = int(rng.integers(1, 12))
         Fv = [int(v) for v in rng.integers(0, 12, n)]; Ev = [int(v) for v in rng.integers(0, 9, n)]
         assert core.fast_assign_prefetch(P, Fv, Ev) == tuple(O.fast_assign_prefetch(P, Fv, Ev))
+
+
+def test_layer_degenerate_inputs():
+    """No tokens at all; fewer tokens than experts; every pair beyond the capacity dropped but one per expert."""
+    from mole_amd.moe.layer import MOLEModule
+    print("layer degenerate", flush=True)
+    for dtype in (torch.float32, torch.bfloat16):
+        m, x, ref = _build(0, 64, 4, 2, 128, dtype)
+        xe = torch.zeros(0, 64, dtype=dtype, device="cuda", requires_grad=True)
+        y = m(xe, capacity_factor=1.0)
+        assert y.shape == (0, 64)
+        y.sum().backward()
+        assert xe.grad.shape == (0, 64)
+        # 3 tokens, 8 experts, top-2: most experts receive nothing
+        m, x, ref = _build(3, 64, 8, 2, 128, dtype, seed=5)
+        _run_and_compare(m, x, ref, 2, 0.0, dtype)
+        # capacity 1 row per expert and choice: nearly everything is dropped, dropped tokens output zeros
+        m, x, ref = _build(200, 64, 4, 1, 128, dtype, seed=6)
+        res = _run_and_compare(m, x, ref, 1, 0.02, dtype)
+        assert res.crit.capacity == 1 and int(res.crit.kept_rows.sum()) <= 4
+        # a capacity of zero drops everything: zeros out, zero gradients, no error
+        m, x, ref = _build(50, 64, 4, 2, 128, dtype, seed=7)
+        res = _run_and_compare(m, x, ref, 2, 0.001, dtype)
+        assert res.crit.capacity == 0 and float(res.y.abs().max()) == 0.0

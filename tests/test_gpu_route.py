@@ -33,6 +33,7 @@ def _compare(scores, k, cf, layout_ragged, normalize=True, alignment=1):
     (1, 1, 1, 1.0), (5, 3, 2, 0.0), (255, 8, 2, 1.0), (256, 8, 2, 1.0), (257, 8, 2, 0.5),
     (1000, 16, 1, 1.25), (777, 5, 5, 0.0), (4096, 64, 2, 0.0), (3000, 100, 4, -0.5),
     (2048, 256, 8, 0.0), (600, 1024, 16, 0.0), (4096, 8, 2, 1.0),
+    (200, 4, 1, 0.02),      # 0.02 * 50 is 1 in double precision and 0.99999998 in single: the capacity must be 1
 ])
 @pytest.mark.parametrize("ragged", [True, False])
 def test_route_matches_oracle(S, E, k, cf, ragged):
