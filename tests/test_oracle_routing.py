@@ -135,6 +135,9 @@ def test_capacity_special_cases_of_the_benchmark_configs():
     assert O.compute_capacity(4096, 8, 2, 1.0, 0) == 1024
     assert O.compute_capacity(10, 4, 2, 0.0, 7, alignment=4) == 8
     assert O.compute_capacity(10, 4, 1, -1.0, 7) == 3
+    # the product is a Python (double precision) one: int(0.02 * 50) is 1; in single precision it would be 0
+    assert O.compute_capacity(200, 4, 1, 0.02, 0) == 1
+    assert O.compute_capacity(200, 4, 1, 0.001, 0) == 0
 
 
 def test_capacity_drop_is_lowest_index_first_and_first_choice_first():
