@@ -115,3 +115,17 @@ def test_fused_gate_forward(S, E, M, bias):
     assert float((got.sum(-1) - 1).abs().max()) < 1e-5
     unfused = H.softmax_fwd(H.gemm_nt(x.cuda(), wg.bfloat16().cuda()), b.cuda() if bias else None).cpu()
     assert rel_err(got, unfused) < 1e-5
+
+
+def test_route_random_sweep():
+    """Sixty seeded random (S, E, k, capacity factor, alignment) combinations, both layouts, bit for bit."""
+    rng = np.random.default_rng(2024)
+    cfs = [0.0, 0.01, 0.02, 0.05, 0.1, 0.3, 0.5, 0.7, 1.0, 1.25, 2.0, 3.3, -0.3, -1.0]
+    for case in range(60):
+        E = int(rng.choice([1, 2, 3, 4, 7, 8, 16, 17, 32, 60, 64, 128]))
+        k = int(rng.integers(1, min(E, 8) + 1))
+        S = int(rng.integers(1, 1500))
+        cf = float(rng.choice(cfs))
+        align = int(rng.choice([1, 1, 1, 2, 8]))
+        print(f"route sweep {case}: S={S} E={E} k={k} cf={cf} align={align}", flush=True)
+        _compare(zipf_scores(S, E, seed=case, ties=(case % 5 == 0)), k, cf, bool(case % 2), normalize=bool(case % 3), alignment=align)
