@@ -109,18 +109,21 @@ __device__ __forceinline__ float fast_gelu_erf(float x) {
     const float hx = 0.5f * x;
     return fmaf(hx, odd_poly(x, 0.25f, c), hx);
 }
-// derivative of the tanh form of GELU, what the reference's backward multiplies by (MOLE/cpp/gelu.cu:3-14)
-__device__ __forceinline__ float fast_d_gelu_tanh(float x) {
-    constexpr float c[10] = {3.58895016f, -24.237009f, 110.279869f, -345.395355f, 772.538513f,
-                             -1226.4845f, 1338.11902f, -946.521179f, 388.703674f, -70.0920258f};
-    return 0.5f + odd_poly(x, 1.0f / 4.5f, c);
-}
-// derivative of the erf form: Phi(x) + x phi(x)
-__device__ __forceinline__ float fast_d_gelu_exact(float x) {
-    constexpr float c[10] = {3.58931732f, -24.1413288f, 108.150215f, -329.418243f, 711.674683f,
-                             -1091.27979f, 1154.8053f, -796.700195f, 320.776367f, -56.9563408f};
-    return 0.5f + odd_poly(x, 1.0f / 4.5f, c);
-}
+// The two GELU derivatives share the clamp (4.5) and the degree, so the variant is a choice of coefficients,
+// made once per tile, not a branch per element: tanh form = what the reference's backward multiplies by
+// (MOLE/cpp/gelu.cu:3-14), exact form = Phi(x) + x phi(x).
+struct DGeluCoef {
+    float c[10];
+    __device__ __forceinline__ void select(bool tanh_form) {
+        constexpr float ct[10] = {3.58895016f, -24.237009f, 110.279869f, -345.395355f, 772.538513f,
+                                  -1226.4845f, 1338.11902f, -946.521179f, 388.703674f, -70.0920258f};
+        constexpr float ce[10] = {3.58931732f, -24.1413288f, 108.150215f, -329.418243f, 711.674683f,
+                                  -1091.27979f, 1154.8053f, -796.700195f, 320.776367f, -56.9563408f};
+#pragma unroll
+        for (int i = 0; i < 10; ++i) c[i] = tanh_form ? ct[i] : ce[i];
+    }
+    __device__ __forceinline__ float operator()(float x) const { return 0.5f + odd_poly(x, 1.0f / 4.5f, c); }
+};
 
 // ---- operand tiles in LDS -------------------------------------------------------------------------
 // A stage holds 32 of K.  Every lane always issues its load (no divergent branches in the K loop):
@@ -373,28 +376,6 @@ template <int EPI> __device__ __forceinline__ void load_bias(const GemmArgs &g, 
     }
 }
 
-// The wave's (32 TMW) x 64 piece of the pre-activation that GELU' needs, 16 bytes per lane per 8 rows, fetched
-// before the K loop into registers where the register budget allows it (two waves per SIMD leave 256
-// registers a wave, of which the K loop needs under 200; half of the piece fits): the epilogue then starts
-// on data that is already there while the loads of the other half are in flight.
-template <int TMB, int WM, int EPI> struct PreAct {
-    static constexpr bool ON = EPI == EPI_DGELU && WM == 2;
-    static constexpr int N = ON ? Tile<TMB, WM>::TMW * 2 : 1;      // the first half of the rows; the rest would spill
-    uint4 v[N];
-    __device__ __forceinline__ void load(const GemmArgs &g, long row0, int m0, int n0, int live, int lane, int wn) {
-        if constexpr (ON) {
-            const int jr = lane >> 3, jc = lane & 7, nw0 = n0 + wn * 64;
-#pragma unroll
-            for (int it = 0; it < N; ++it) {
-                const int row = it * 8 + jr;
-                v[it] = make_uint4(0, 0, 0, 0);
-                if (row < live && nw0 + jc * 8 < g.N)
-                    v[it] = *reinterpret_cast<const uint4 *>((const bf16_t *)g.H + (row0 + m0 + row) * g.ldc + nw0 + jc * 8);
-            }
-        }
-    }
-};
-
 // The epilogue of one wave, whose first TMCW 32-row blocks hold live rows.  acc[tm][tn][4q+j] = C[m, n] with
 // m = m0 + 32 tm + lane%32 (m0: the wave's first row) and n = n0 + 64 wn + 32 tn + 8 q + 4 (lane/32) + j.  A wave
 // owns a (32 TMW) x 64 slab of the tile.  bf16 results go through the wave's own slab of LDS (the K loop is
@@ -405,7 +386,7 @@ template <int TMB, int WM, int EPI> struct PreAct {
 template <int TMB, int WM, bool WG, int EPI, int TMC>
 __device__ __forceinline__ void epilogue(const GemmArgs &g, f32x16 (&acc)[Tile<TMB, WM>::TMW][2], char *smem, int lane, int wave,
                                          int wn, int e, long row0, int m0, int n0, int m_ext, int live,
-                                         const uint2 (&bias_raw)[8], const PreAct<TMB, WM, EPI> &pre) {
+                                         const uint2 (&bias_raw)[8]) {
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
     __syncthreads();
     if constexpr (TMC == 0) return;
@@ -474,26 +455,11 @@ __device__ __forceinline__ void epilogue(const GemmArgs &g, f32x16 (&acc)[Tile<T
             }
         return;
     }
-    if constexpr (PreAct<TMB, WM, EPI>::ON) {
-        constexpr int NPRE = PreAct<TMB, WM, EPI>::N, NREST = TMC * 4 > NPRE ? TMC * 4 - NPRE : 0;
-        uint4 rest[NREST ? NREST : 1];
-#pragma unroll
-        for (int it = 0; it < NREST; ++it) {
-            const int row = (NPRE + it) * 8 + jr;
-            rest[it] = make_uint4(0, 0, 0, 0);
-            if (row < live && col_ok)
-                rest[it] = *reinterpret_cast<const uint4 *>((const bf16_t *)g.H + (crow0 + m0 + row) * g.ldc + nw0 + jc * 8);
-        }
-#pragma unroll
-        for (int it = 0; it < TMC * 4; ++it) {
-            const int row = it * 8 + jr;
-            *reinterpret_cast<uint4 *>(slab_at(row, jc, (row >> 4) & 1)) = fix16(it < NPRE ? pre.v[it < NPRE ? it : 0] : rest[it >= NPRE ? it - NPRE : 0], row);
-        }
-    } else if constexpr (EPI == EPI_DGELU) {
-        fill((const bf16_t *)g.H);
-    }
+    if constexpr (EPI == EPI_DGELU) fill((const bf16_t *)g.H);
     if constexpr (EPI == EPI_WGRAD) { if (g.accumulate) fill(Cb); }
 
+    DGeluCoef dgelu;
+    if constexpr (EPI == EPI_DGELU) dgelu.select(g.gelu_bwd == MOLE_GELU_BWD_TANH);
     // pass 0 writes C; for EPI_BIAS_GELU pass 1 writes C2 = gelu(h)
     constexpr int PASSES = EPI == EPI_BIAS_GELU ? 2 : 1;
 #pragma unroll
@@ -525,13 +491,8 @@ __device__ __forceinline__ void epilogue(const GemmArgs &g, f32x16 (&acc)[Tile<T
                     } else if constexpr (EPI == EPI_DGELU) {
                         float hv[4];
                         unpack4(*reinterpret_cast<const uint2 *>(cell), hv);
-                        if (g.gelu_bwd == MOLE_GELU_BWD_TANH) {
 #pragma unroll
-                            for (int j = 0; j < 4; ++j) v[j] *= fast_d_gelu_tanh(hv[j]);
-                        } else {
-#pragma unroll
-                            for (int j = 0; j < 4; ++j) v[j] *= fast_d_gelu_exact(hv[j]);
-                        }
+                        for (int j = 0; j < 4; ++j) v[j] *= dgelu(hv[j]);
                     } else if constexpr (EPI == EPI_WGRAD) {
                         if (g.accumulate) {
                             float old[4];
@@ -663,13 +624,11 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
     // The live blocks are dealt evenly to the wave rows: c to each (the last row may find fewer live).
     const int c = (tmc + WM - 1) / WM;
     const int m0w = m0 + wm * c * 32, live_w = max(0, min(live - wm * c * 32, c * 32));
-    PreAct<TMB, WM, EPI> pre;
-    pre.load(g, row0, m0w, n0, live_w, lane, wn);
     // K loop and epilogue with C blocks per wave row
 #define MOLE_RUN_TILE(C)                                                                                                  \
     {                                                                                                                     \
         main_loop<TMB, WM, M_KS, N_KS, WG, WM *(C), (C)>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wu, wm, wn, acc); \
-        epilogue<TMB, WM, WG, EPI, (C)>(g, acc, smem, lane, wu, wn, e, row0, m0w, n0, m_ext, live_w, bias_raw, pre);      \
+        epilogue<TMB, WM, WG, EPI, (C)>(g, acc, smem, lane, wu, wn, e, row0, m0w, n0, m_ext, live_w, bias_raw);      \
     }
     if constexpr (WM == 1) {
         if (c > TMB / 2) MOLE_RUN_TILE(TMB)
