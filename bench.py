@@ -111,7 +111,11 @@ def bench_offloaded_stack(args):
     layers = []
     for i in range(n_layers):
         print(f"[c4] building layer {i} (pinned host weights)", file=sys.stderr, flush=True)
-        layers.append(MOLEModule(E, 0, M, F, pool, k, ebatch, dist, "gelu", 1, False, True, dtype=torch.bfloat16))
+        try:
+            layers.append(MOLEModule(E, 0, M, F, pool, k, ebatch, dist, "gelu", 1, False, True, dtype=torch.bfloat16))
+        except RuntimeError as exc:     # pinned host memory is capped well below the machine's RAM on some boxes
+            print(f"[c4] layer {i} could not be built ({str(exc).splitlines()[0]}): lower --layers", file=sys.stderr)
+            sys.exit(3)
     for m in layers:
         m.set_prefetch(E, E)
     g = torch.Generator().manual_seed(0)
