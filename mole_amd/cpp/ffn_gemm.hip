@@ -332,19 +332,37 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kernel(const GemmArgs g) {
 
 // column sums over an expert's rows: out[e, n] (+)= sum_{r in rows_e} in[r, n]
 // (torch::sum_out(g_b2, go, {1}) / (g_b1, t, {1}), MOLE/cpp/core.cpp:399, 408).
+// Both sums run in one launch: blocks [0, nbx0) of a grid row take the first matrix, the rest the
+// second, so the narrow one (M columns) does not leave most of the chip idle on its own.
 // A block of 16 waves owns 64*VEC columns of one expert; wave w sums rows w, w+16, ... with 8-byte
-// loads per lane (4 rows in flight), then the 16 partial rows are folded through LDS in a fixed order.
+// loads per lane (8 rows in flight), then the 16 partial rows are folded through LDS in a fixed order.
 constexpr int BG_WAVES = 16;
+constexpr int BG_FLY = 8;
 template <typename T>
-__global__ __launch_bounds__(BG_WAVES * 64) void bias_grad_kernel(const T *__restrict__ in,
+__device__ __forceinline__ void bias_acc(float *acc, uint2 v) {
+    if constexpr (sizeof(T) == 2) {
+        acc[0] += __uint_as_float(v.x << 16); acc[1] += __uint_as_float(v.x & 0xffff0000u);
+        acc[2] += __uint_as_float(v.y << 16); acc[3] += __uint_as_float(v.y & 0xffff0000u);
+    } else {
+        acc[0] += __uint_as_float(v.x); acc[1] += __uint_as_float(v.y);
+    }
+}
+template <typename T>
+__global__ __launch_bounds__(BG_WAVES * 64) void bias_grad_kernel(const T *__restrict__ in0, int N0, T *__restrict__ out0,
+                                                                   int nbx0, const T *__restrict__ in1, int N1,
+                                                                   T *__restrict__ out1,
                                                                    const int32_t *__restrict__ offsets,
-                                                                   const int32_t *__restrict__ kept, int N,
-                                                                   int accumulate, T *__restrict__ out) {
+                                                                   const int32_t *__restrict__ kept, int accumulate) {
     constexpr int VEC = 8 / sizeof(T);   // elements per 8-byte load: 4 bf16 or 2 fp32
     __shared__ float s_part[BG_WAVES][64 * VEC];
+    const bool first = (int)blockIdx.x < nbx0;
+    const T *__restrict__ in = first ? in0 : in1;
+    T *__restrict__ out = first ? out0 : out1;
+    const int N = first ? N0 : N1;
+    const int bx = first ? blockIdx.x : blockIdx.x - nbx0;
     const int e = blockIdx.y;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    const int n = (blockIdx.x * 64 + lane) * VEC;
+    const int n = (bx * 64 + lane) * VEC;
     const long r0 = offsets[e];
     const int rows = kept[e];
     float acc[VEC];
@@ -353,35 +371,20 @@ __global__ __launch_bounds__(BG_WAVES * 64) void bias_grad_kernel(const T *__res
     if (n < N) {
         const T *p = in + r0 * (long)N + n;
         int r = w;
-        for (; r + 3 * BG_WAVES < rows; r += 4 * BG_WAVES) {
-            uint2 v[4];
+        for (; r + (BG_FLY - 1) * BG_WAVES < rows; r += BG_FLY * BG_WAVES) {
+            uint2 v[BG_FLY];
 #pragma unroll
-            for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const uint2 *>(p + (long)(r + u * BG_WAVES) * N);
+            for (int u = 0; u < BG_FLY; ++u) v[u] = *reinterpret_cast<const uint2 *>(p + (long)(r + u * BG_WAVES) * N);
 #pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                if constexpr (sizeof(T) == 2) {
-                    acc[0] += __uint_as_float(v[u].x << 16); acc[1] += __uint_as_float(v[u].x & 0xffff0000u);
-                    acc[2] += __uint_as_float(v[u].y << 16); acc[3] += __uint_as_float(v[u].y & 0xffff0000u);
-                } else {
-                    acc[0] += __uint_as_float(v[u].x); acc[1] += __uint_as_float(v[u].y);
-                }
-            }
+            for (int u = 0; u < BG_FLY; ++u) bias_acc<T>(acc, v[u]);
         }
-        for (; r < rows; r += BG_WAVES) {
-            const uint2 v = *reinterpret_cast<const uint2 *>(p + (long)r * N);
-            if constexpr (sizeof(T) == 2) {
-                acc[0] += __uint_as_float(v.x << 16); acc[1] += __uint_as_float(v.x & 0xffff0000u);
-                acc[2] += __uint_as_float(v.y << 16); acc[3] += __uint_as_float(v.y & 0xffff0000u);
-            } else {
-                acc[0] += __uint_as_float(v.x); acc[1] += __uint_as_float(v.y);
-            }
-        }
+        for (; r < rows; r += BG_WAVES) bias_acc<T>(acc, *reinterpret_cast<const uint2 *>(p + (long)r * N));
     }
 #pragma unroll
     for (int q = 0; q < VEC; ++q) s_part[w][lane * VEC + q] = acc[q];
     __syncthreads();
     for (int c = threadIdx.x; c < 64 * VEC; c += BG_WAVES * 64) {
-        const int nn = blockIdx.x * 64 * VEC + c;
+        const int nn = bx * 64 * VEC + c;
         if (nn >= N) continue;
         float v = 0.f;
 #pragma unroll
@@ -469,11 +472,10 @@ static int ffn_bwd_t(const void *go, const void *xd, const void *h, const void *
     // g_b2 = sum go ; g_b1 = sum t
     {
     ScopedTiming timing(MOLE_K_FFN_GB, st);
-    hipLaunchKernelGGL(bias_grad_kernel<T>, dim3(ceil_div(M, 512 / (int)sizeof(T)), E), dim3(BG_WAVES * 64), 0, st, (const T *)go, offsets, kept, M,
-                       accumulate, (T *)g_b2);
-    MOLE_LAUNCH_CHECK();
-    hipLaunchKernelGGL(bias_grad_kernel<T>, dim3(ceil_div(F, 512 / (int)sizeof(T)), E), dim3(BG_WAVES * 64), 0, st, (const T *)t, offsets, kept, F,
-                       accumulate, (T *)g_b1);
+    const int cols_per_block = 512 / (int)sizeof(T);
+    const int nb2 = ceil_div(M, cols_per_block), nb1 = ceil_div(F, cols_per_block);
+    hipLaunchKernelGGL(bias_grad_kernel<T>, dim3(nb2 + nb1, E), dim3(BG_WAVES * 64), 0, st, (const T *)go, M, (T *)g_b2, nb2,
+                       (const T *)t, F, (T *)g_b1, offsets, kept, accumulate);
     MOLE_LAUNCH_CHECK();
     }
     // g_w1[e] = t^T . xd
