@@ -70,7 +70,8 @@ enum {
     MOLE_K_COMBINE_BWD = 10,
     MOLE_K_ROUTE = 11,    /* the four routing kernels together */
     MOLE_K_GEMM_NT = 12,
-    MOLE_K_COUNT = 13
+    MOLE_K_ADAM = 13,
+    MOLE_K_COUNT = 14
 };
 int mole_kernel_timing_enable(int on);
 int mole_kernel_timing_read(int n_ids, int *counts, float *ms_total);
@@ -241,6 +242,33 @@ int mole_unimem_store_grads(void *handle, void *const host_dst[4], const void *c
 int mole_unimem_sync_tranback(void *handle);
 int mole_unimem_tranback_stream(void *handle, mole_stream_t *out);
 int mole_unimem_writeback_stats(void *handle, uint64_t *bytes, float *busy_ms);
+
+/* Optimizer state of offloaded experts in the backward pipeline; replaces the moment fetches and the
+ * parameter / moment stores of _MOLECore::instant_adam (MOLE/cpp/core.cpp:864-935:
+ * fetch_batch_cpu_mome/vari/grad + _ParamProxy::fetch on the tran stream after comp_event,
+ * store_batch_cpu_para/mome/vari on the tranback stream).
+ * mole_unimem_load_state: count host->device copies of bytes[i] from pinned host_src[i] to dev_dst[i] on
+ * the library's copy stream, which first waits for the work already enqueued on compute_stream (the
+ * previous users of dev_dst); compute_stream then waits for the copies.
+ * mole_unimem_store_state: count device->host copies on the write-back stream once the work already
+ * enqueued on compute_stream has finished; lifetime and synchronisation rules as for
+ * mole_unimem_store_grads. */
+int mole_unimem_load_state(void *handle, void *const dev_dst[], const void *const host_src[], const size_t bytes[],
+                           int count, mole_stream_t compute_stream);
+int mole_unimem_store_state(void *handle, void *const host_dst[], const void *const dev_src[], const size_t bytes[],
+                            int count, mole_stream_t compute_stream);
+
+/* Fused Adam / AdamW step on a flat array of n elements; replaces _MOLECore::adam
+ * (MOLE/cpp/define.hpp:543-579) as called four times per expert batch by instant_adam
+ * (MOLE/cpp/core.cpp:917-920).  p, g: dtype (fp32 or bf16); m, v: fp32, updated in place; p_out: dtype, may
+ * be p itself or a separate buffer (the reference's write-back variant keeps p and returns p_back).
+ * t is the step count already incremented (the reference uses its stored counter + 1); lam is the weight
+ * decay: adamw != 0 scales p by (1 - lam lr) first, otherwise g += lam p.  In the reference's order:
+ * m = b1 m + (1-b1) g;  v = b2 v + (1-b2) g g;  p_out = p - lr (m / (1-b1^t)) / (sqrt(v / (1-b2^t)) + eps).
+ * All pointers 16-byte aligned. */
+int mole_adam_step(const void *p, const void *g, float *m, float *v, void *p_out, size_t n, int dtype,
+                   float beta1, float beta2, int t, float lr, float lam, float eps, int adamw,
+                   mole_stream_t stream);
 
 /* Greedy cross-layer prefetch assignment; replaces fast_assign_prefetch
  * (MOLE/cpp/core.cpp:1302-1345).  lp_out [n]; gp_out holds up to gp_cap triples

@@ -19,7 +19,7 @@ LAYOUT_PADDED, LAYOUT_RAGGED = 0, 1
 GELU_BWD_TANH, GELU_BWD_EXACT = 0, 1
 MAX_TOPK, MAX_EXPERTS = 16, 1024
 KERNEL_IDS = ("ffn_fwd1", "ffn_fwd2", "ffn_gw2", "ffn_da", "ffn_gw1", "ffn_gx", "ffn_gb", "dispatch_fwd", "dispatch_bwd",
-              "combine_fwd", "combine_bwd", "route", "gemm_nt")
+              "combine_fwd", "combine_bwd", "route", "gemm_nt", "adam")
 
 _P = c_void_p
 _SIGNATURES = {
@@ -63,6 +63,10 @@ _SIGNATURES = {
     "mole_unimem_sync_tranback": (c_int, [_P]),
     "mole_unimem_tranback_stream": (c_int, [_P, POINTER(_P)]),
     "mole_unimem_writeback_stats": (c_int, [_P, POINTER(c_uint64), POINTER(c_float)]),
+    "mole_unimem_load_state": (c_int, [_P, POINTER(_P), POINTER(_P), POINTER(c_size_t), c_int, _P]),
+    "mole_unimem_store_state": (c_int, [_P, POINTER(_P), POINTER(_P), POINTER(c_size_t), c_int, _P]),
+    "mole_adam_step": (c_int, [_P, _P, _P, _P, _P, c_size_t, c_int, c_float, c_float, c_int, c_float, c_float, c_float,
+                               c_int, _P]),
     "mole_fast_assign_prefetch": (c_int, [c_int, POINTER(c_int), POINTER(c_int), c_int, POINTER(c_int),
                                           POINTER(c_int), c_int, POINTER(c_int)]),
 }

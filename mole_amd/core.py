@@ -101,6 +101,46 @@ class UniMem:
         for g in dev_grads:           # the allocator must not hand these blocks out again before the copy has run
             g.record_stream(wb)
 
+    @staticmethod
+    def _arrays(tensors):
+        n = len(tensors)
+        ptrs, sizes = (c_void_p * n)(), (ctypes.c_size_t * n)()
+        for i, t in enumerate(tensors):
+            ptrs[i], sizes[i] = t.data_ptr(), t.numel() * t.element_size()
+        return ptrs, sizes
+
+    def _side_stream(self, getter: str, device) -> torch.cuda.Stream:
+        out = c_void_p()
+        L.check(getattr(L.lib(), getter)(self._h, ctypes.byref(out)), getter)
+        return torch.cuda.ExternalStream(int(out.value), device=device)
+
+    def load_state(self, dev_tensors, host_tensors):
+        """Pinned host arrays -> device tensors of the same sizes on the copy stream (after the compute already
+        enqueued on the current stream, which then waits for the copies): optimizer moments and accumulated
+        gradients of an expert batch (core.cpp:864-915)."""
+        dp, sizes = self._arrays(dev_tensors)
+        hp, hs = self._arrays(host_tensors)
+        if list(sizes) != list(hs):
+            raise RuntimeError("UniMem.load_state: host and device sizes differ")
+        L.check(L.lib().mole_unimem_load_state(self._h, dp, hp, sizes, len(dev_tensors), L.stream()),
+                "mole_unimem_load_state")
+        tran = self._side_stream("mole_unimem_tran_stream", dev_tensors[0].device)
+        for t in dev_tensors:
+            t.record_stream(tran)
+
+    def store_state(self, host_tensors, dev_tensors):
+        """Device tensors -> pinned host arrays on the write-back stream, after the compute already enqueued on
+        the current stream (core.cpp:925-935)."""
+        hp, hs = self._arrays(host_tensors)
+        dp, sizes = self._arrays(dev_tensors)
+        if list(sizes) != list(hs):
+            raise RuntimeError("UniMem.store_state: host and device sizes differ")
+        L.check(L.lib().mole_unimem_store_state(self._h, hp, dp, sizes, len(dev_tensors), L.stream()),
+                "mole_unimem_store_state")
+        wb = self._side_stream("mole_unimem_tranback_stream", dev_tensors[0].device)
+        for t in dev_tensors:
+            t.record_stream(wb)
+
     def writeback_stats(self):
         b, ms = c_uint64(), c_float()
         L.check(L.lib().mole_unimem_writeback_stats(self._h, ctypes.byref(b), ctypes.byref(ms)),
@@ -198,8 +238,9 @@ class MOLECore:
             raise NotImplementedError("this build covers the single-GPU hot path (world_size == 1)")
         if act_name != "gelu":
             raise NotImplementedError("only act='gelu' is on the hot path")
-        if adv_adam:
-            raise NotImplementedError("in-pipeline Adam (adv_adam) is outside the hot path")
+        self.adv_adam = bool(adv_adam)
+        self.adam = None            # set_adam(): (beta1, beta2, t, lr, lam, eps, adamW)
+        self.hybrid_adam_count = d_experts
         self.use_pool, self.acc_step, self.step = bool(use_pool), int(acc_step), int(step)
         self.device, self.moe_id, self.total_experts = device, moe_id, total_experts
         self.s_experts, self.d_experts, self.ebatch_size = s_experts, d_experts, max(int(ebatch_size), 1)
@@ -215,7 +256,16 @@ class MOLECore:
         self.gpu[p_id] = (all_tensors, grad_tensors)
 
     def set_CPUParamCore(self, p_id, all_tensors, grad_, momentum, variance, bias, p_id2=None):
-        self.cpu[p_id] = (all_tensors, grad_)
+        self.cpu[p_id] = (all_tensors, grad_, momentum, variance)
+
+    def set_adam(self, beta1, beta2, t, lr, lam, eps, adamW, hybrid_adam_count=-1):
+        """Hyper-parameters of the in-pipeline Adam (define.hpp:524-541); t is the optimizer's step counter
+        before this step, hybrid_adam_count the number of leading offloaded experts updated on the GPU (-1: all)."""
+        self.adam = (float(beta1), float(beta2), int(t), float(lr), float(lam), float(eps), bool(adamW))
+        self.hybrid_adam_count = self.d_experts if hybrid_adam_count == -1 else int(hybrid_adam_count)
+
+    def set_hybrid_adam_count(self, hybrid_adam_count):
+        self.hybrid_adam_count = self.d_experts if hybrid_adam_count == -1 else int(hybrid_adam_count)
 
     def _host(self):
         return [c[0] for c in self.cpu]
@@ -332,6 +382,7 @@ class MOLECore:
                 raise RuntimeError(f"prefetch stack out of order: top holds {prefetched}, layer expects {self.bwd_base}")
             self.bwd_base = 0
             host_grads = [c[1] for c in self.cpu]
+            adam_now = self.adv_adam and (self.step + 1) % self.acc_step == 0
             for (base, size, pref, view_base) in self._chunks(prefetched):
                 p = um.fetch(self._host(), view_base, base, size, pref)   # weights are fetched again (core.cpp:1203)
                 um.wait_params()
@@ -339,8 +390,17 @@ class MOLECore:
                 g = [torch.empty((size, *hg.shape[1:]), dtype=hg.dtype, device=x2.device) for hg in host_grads]
                 H.ffn_bwd_into(go, x2, h, a, offsets[e0:], kept_rows[e0:], size, rows, M, F, p[0], p[2], t, g[0], g[1],
                                g[2], g[3], gx, False, self.gelu_bwd)
-                um.release(view_base, size)
-                self._store_grad(host_grads, g, base, size)
+                if adam_now:
+                    # the update reads the parameters in their pool slots, so the slots are released after it
+                    self._instant_adam(p, g, base, size)
+                    um.release(view_base, size)
+                else:
+                    um.release(view_base, size)
+                    self._store_grad(host_grads, g, base, size)
+            if adam_now:
+                # the next prefetch reads the host parameters that the write-back stream is still filling
+                # (the reference ends its backward with a synchronisation of the copy stream, core.cpp:1287)
+                um.sync_tran()
         self.step += 1
         for c in self.cpu:
             if c is not None and hasattr(c[1], "lazy_zero"):
@@ -356,6 +416,53 @@ class MOLECore:
                 hg[base:base + size] += gg.to("cpu")
         else:
             get_UniMem().store_grads(host_grads, g, base, size)
+
+
+    def _instant_adam(self, p_slots, g, base, size):
+        """Adam on the GPU for experts [base, base+size) of the offloaded set, inside the backward pipeline
+        (core.cpp:848-943): fetch their moments (and, when accumulating, the gradients of the earlier
+        micro-steps) from pinned host memory, one fused update per parameter array, write parameters and
+        moments back.  Only the first hybrid_adam_count experts are updated here; the gradients of the others
+        go to the host for the CPU optimizer.  The reference narrows the second weight from the first one when
+        it cuts a batch at hybrid_adam_count (core.cpp:859); this follows the evident intent instead."""
+        if self.adam is None:
+            raise RuntimeError("in-pipeline Adam needs set_adam() before backward")
+        if any(c[2] is None or c[3] is None for c in self.cpu):
+            raise RuntimeError("in-pipeline Adam needs momentum and variance arrays (set_CPUParamCore)")
+        um = get_UniMem()
+        host_grads = [c[1] for c in self.cpu]
+        n = max(0, min(size, self.hybrid_adam_count - base))
+        if n < size:          # experts beyond the GPU-updated prefix: gradients only
+            rest = [gg[n:] for gg in g]
+            if self.acc_step > 1 and not getattr(host_grads[0], "lazy_zero", True):
+                um.sync_tran()
+                for hg, gg in zip(host_grads, rest):
+                    hg[base + n:base + size] += gg.to("cpu")
+            else:
+                um.store_state([hg[base + n:base + size] for hg in host_grads], rest)
+        if n == 0:
+            return
+        beta1, beta2, t, lr, lam, eps, adamw = self.adam
+        dev = g[0].device
+        m_host = [c[2][base:base + n] for c in self.cpu]
+        v_host = [c[3][base:base + n] for c in self.cpu]
+        m = [torch.empty(mh.shape, dtype=torch.float32, device=dev) for mh in m_host]
+        v = [torch.empty(vh.shape, dtype=torch.float32, device=dev) for vh in v_host]
+        loads_dev, loads_host = m + v, m_host + v_host
+        acc = self.acc_step > 1 and not getattr(host_grads[0], "lazy_zero", True)
+        if acc:
+            g_prev = [torch.empty((n, *hg.shape[1:]), dtype=hg.dtype, device=dev) for hg in host_grads]
+            loads_dev, loads_host = loads_dev + g_prev, loads_host + [hg[base:base + n] for hg in host_grads]
+        um.load_state(loads_dev, loads_host)
+        p_new = []
+        for k in range(4):
+            gk = g[k][:n]
+            if acc:
+                gk += g_prev[k]
+            out = torch.empty_like(gk)
+            H.adam_step(p_slots[k], gk, m[k], v[k], beta1, beta2, t + 1, lr, lam, eps, adamw, p_out=out)
+            p_new.append(out)
+        um.store_state([c[0][base:base + n] for c in self.cpu] + m_host + v_host, p_new + m + v)
 
 
 class BatchFusedFWD(torch.autograd.Function):

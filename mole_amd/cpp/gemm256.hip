@@ -679,9 +679,9 @@ static int dispatch256(const GemmArgs &g, bool b_ks, bool wg, int epi, int max_r
     const int tiles = ((rows_bound / BM + (g.offsets ? g.E : 1)) * n_tiles + 7) & ~7;
     if (wg) return -100;
     if (!b_ks) {
+        if (epi == EPI_DGELU) return launch256<TMB, WM, false, false, EPI_DGELU>(gg, tiles, st, kid);
         if constexpr (TMB != 10) {
             if (epi == EPI_BIAS_GELU) return launch256<TMB, WM, false, false, EPI_BIAS_GELU>(gg, tiles, st, kid);
-            if (epi == EPI_DGELU) return launch256<TMB, WM, false, false, EPI_DGELU>(gg, tiles, st, kid);
             if (epi == EPI_F32) return launch256<TMB, WM, false, false, EPI_F32>(gg, tiles, st, kid);
         }
     } else {
@@ -692,10 +692,11 @@ static int dispatch256(const GemmArgs &g, bool b_ks, bool wg, int epi, int max_r
 }
 
 // Tile configuration.  Eight waves (two per SIMD hide each other's waits; one fetch of the n-side tile
-// serves all rows of the tile) for every product: 256-row tiles, and tiles of up to 320 rows for the two
-// products with a light epilogue (out = a.w2 + b2 and gx = t.w1), whose register budget allows 160
-// accumulators a wave: with a capacity factor of 1.25 an expert then never needs more m-tiles than the
-// average one, and the launch stays one round of tiles.  MOLE_TMB=4|8 in the environment selects the
+// serves all rows of the tile) for every product.  256-row tiles by default; tiles of up to 320 rows for
+// the three products whose register budget allows 160 accumulators a wave (out = a.w2 + b2, gx = t.w1 and
+// t = (go.w2^T) gelu'(h)): with a capacity factor of 1.25 an expert then never needs more m-tiles than
+// the average one, and the launch stays one round of tiles.  h = xd.w1^T + b1 with the GELU epilogue
+// spills at 160 accumulators and stays at 256 rows.  MOLE_TMB=4|8 in the environment selects the
 // four-wave variants with 128 or 256 rows, 16 the 256-row eight-wave tile for everything (tuning aid).
 static int tile_blocks_for(int kid) {
     static const int forced = [] {
@@ -703,7 +704,7 @@ static int tile_blocks_for(int kid) {
         return v ? atoi(v) : 0;
     }();
     if (forced == 4 || forced == 8 || forced == 16) return forced;
-    return (kid == MOLE_K_FFN_FWD2 || kid == MOLE_K_FFN_GX) ? 20 : 16;
+    return (kid == MOLE_K_FFN_FWD2 || kid == MOLE_K_FFN_GX || kid == MOLE_K_FFN_DA) ? 20 : 16;
 }
 
 int launch_gemm256(const GemmArgs &g, bool a_ks, bool b_ks, bool wg, int epi, int max_rows, hipStream_t st, int kid) {
@@ -714,7 +715,7 @@ int launch_gemm256(const GemmArgs &g, bool a_ks, bool b_ks, bool wg, int epi, in
     const int tmb = tile_blocks_for(kid);
     if (tmb == 4) return dispatch256<4, 1>(g, b_ks, wg, epi, max_rows, st, kid);
     if (tmb == 16) return dispatch256<8, 2>(g, b_ks, wg, epi, max_rows, st, kid);   // 256 rows, eight waves
-    if (tmb == 20 && !wg && b_ks) return dispatch256<10, 2>(g, b_ks, wg, epi, max_rows, st, kid);   // up to 320 rows, eight waves
+    if (tmb == 20 && !wg && (b_ks || epi == EPI_DGELU)) return dispatch256<10, 2>(g, b_ks, wg, epi, max_rows, st, kid);   // up to 320 rows, eight waves
     if (tmb == 20) return dispatch256<8, 2>(g, b_ks, wg, epi, max_rows, st, kid);
     return dispatch256<8, 1>(g, b_ks, wg, epi, max_rows, st, kid);
 }

@@ -22,7 +22,7 @@ struct UniMem {
     size_t slot_bytes[4] = {0, 0, 0, 0};
     char *pool[4] = {nullptr, nullptr, nullptr, nullptr};
     hipStream_t tran = nullptr, tranback = nullptr;
-    hipEvent_t para_event = nullptr, grads_ready = nullptr;
+    hipEvent_t para_event = nullptr, grads_ready = nullptr, state_free = nullptr, state_ready = nullptr, wb_done = nullptr;
     bool para_recorded = false;
     std::vector<hipEvent_t> slot_event;
     std::vector<char> slot_pending;  // slot_event[s] was recorded and not yet waited on
@@ -118,6 +118,9 @@ extern "C" int mole_unimem_create(int device, int pool_size, int dtype, int64_t 
     MOLE_HIP(hipStreamCreateWithFlags(&u->tranback, hipStreamNonBlocking));
     MOLE_HIP(hipEventCreateWithFlags(&u->para_event, hipEventDisableTiming));
     MOLE_HIP(hipEventCreateWithFlags(&u->grads_ready, hipEventDisableTiming));
+    MOLE_HIP(hipEventCreateWithFlags(&u->state_free, hipEventDisableTiming));
+    MOLE_HIP(hipEventCreateWithFlags(&u->state_ready, hipEventDisableTiming));
+    MOLE_HIP(hipEventCreateWithFlags(&u->wb_done, hipEventDisableTiming));
     u->slot_event.resize(pool_size);
     u->slot_pending.assign(pool_size, 0);
     for (int s = 0; s < pool_size; ++s) MOLE_HIP(hipEventCreateWithFlags(&u->slot_event[s], hipEventDisableTiming));
@@ -135,6 +138,9 @@ extern "C" int mole_unimem_destroy(void *handle) {
     for (auto &t : u->wb_timers) { (void)hipEventDestroy(t[0]); (void)hipEventDestroy(t[1]); }
     (void)hipEventDestroy(u->para_event);
     (void)hipEventDestroy(u->grads_ready);
+    (void)hipEventDestroy(u->state_free);
+    (void)hipEventDestroy(u->state_ready);
+    (void)hipEventDestroy(u->wb_done);
     (void)hipStreamDestroy(u->tran);
     (void)hipStreamDestroy(u->tranback);
     for (int p = 0; p < 4; ++p)
@@ -271,6 +277,59 @@ extern "C" int mole_unimem_store_grads(void *handle, void *const host_dst[4], co
         MOLE_HIP(hipMemcpyAsync((char *)host_dst[p] + (size_t)base * sb, dev_src[p], (size_t)n * sb, hipMemcpyDeviceToHost,
                                 u->tranback));
         u->wb_bytes_open += (uint64_t)n * sb;
+    }
+    MOLE_HIP(hipEventRecord(tm[1], u->tranback));
+    return 0;
+}
+
+extern "C" int mole_unimem_load_state(void *handle, void *const dev_dst[], const void *const host_src[],
+                                      const size_t bytes[], int count, mole_stream_t compute_stream) {
+    UM(handle);
+    MOLE_REQUIRE(dev_dst && host_src && bytes && count >= 0, "mole_unimem_load_state: bad arguments count=%d", count);
+    if (count == 0) return 0;
+    for (int i = 0; i < count; ++i)
+        MOLE_REQUIRE(bytes[i] == 0 || (dev_dst[i] && host_src[i]), "mole_unimem_load_state: null buffer %d", i);
+    // the destination may have been in use by work already enqueued on the compute stream
+    MOLE_HIP(hipEventRecord(u->state_free, (hipStream_t)compute_stream));
+    MOLE_HIP(hipStreamWaitEvent(u->tran, u->state_free, 0));
+    // and the host arrays may still be the target of an earlier write-back (gradients of the previous micro-step)
+    MOLE_HIP(hipEventRecord(u->wb_done, u->tranback));
+    MOLE_HIP(hipStreamWaitEvent(u->tran, u->wb_done, 0));
+    std::array<hipEvent_t, 2> *tm;
+    if (int rc = next_timer(u, &tm)) return rc;
+    MOLE_HIP(hipEventRecord((*tm)[0], u->tran));
+    for (int i = 0; i < count; ++i) {
+        if (bytes[i] == 0) continue;
+        MOLE_HIP(hipMemcpyAsync(dev_dst[i], host_src[i], bytes[i], hipMemcpyHostToDevice, u->tran));
+        u->bytes_open += bytes[i];
+    }
+    MOLE_HIP(hipEventRecord((*tm)[1], u->tran));
+    MOLE_HIP(hipEventRecord(u->state_ready, u->tran));
+    MOLE_HIP(hipStreamWaitEvent((hipStream_t)compute_stream, u->state_ready, 0));
+    return 0;
+}
+
+extern "C" int mole_unimem_store_state(void *handle, void *const host_dst[], const void *const dev_src[],
+                                       const size_t bytes[], int count, mole_stream_t compute_stream) {
+    UM(handle);
+    MOLE_REQUIRE(host_dst && dev_src && bytes && count >= 0, "mole_unimem_store_state: bad arguments count=%d", count);
+    if (count == 0) return 0;
+    for (int i = 0; i < count; ++i)
+        MOLE_REQUIRE(bytes[i] == 0 || (host_dst[i] && dev_src[i]), "mole_unimem_store_state: null buffer %d", i);
+    MOLE_HIP(hipEventRecord(u->grads_ready, (hipStream_t)compute_stream));
+    MOLE_HIP(hipStreamWaitEvent(u->tranback, u->grads_ready, 0));
+    if (u->wb_timers_used == u->wb_timers.size()) {
+        std::array<hipEvent_t, 2> p;
+        MOLE_HIP(hipEventCreate(&p[0]));
+        MOLE_HIP(hipEventCreate(&p[1]));
+        u->wb_timers.push_back(p);
+    }
+    auto &tm = u->wb_timers[u->wb_timers_used++];
+    MOLE_HIP(hipEventRecord(tm[0], u->tranback));
+    for (int i = 0; i < count; ++i) {
+        if (bytes[i] == 0) continue;
+        MOLE_HIP(hipMemcpyAsync(host_dst[i], dev_src[i], bytes[i], hipMemcpyDeviceToHost, u->tranback));
+        u->wb_bytes_open += bytes[i];
     }
     MOLE_HIP(hipEventRecord(tm[1], u->tranback));
     return 0;

@@ -249,3 +249,32 @@ def ffn_bwd(go, xd, h, a, offsets, kept_rows, w1, w2, g_w1, g_b1, g_w2, g_b2, ne
     ffn_bwd_into(go, xd, h, a, offsets, kept_rows, E, max_rows, M, F, w1, w2, t, g_w1, g_b1, g_w2, g_b2, gx, accumulate,
                  gelu_bwd)
     return gx
+
+
+def adam_step(p, g, m, v, beta1: float, beta2: float, t: int, lr: float, lam: float, eps: float, adamw: bool,
+              p_out=None) -> None:
+    """One fused Adam / AdamW step (define.hpp:543-579) over all elements of p: m and v (fp32) are updated in
+    place, the new parameters go to p_out (p itself when None).  t is the step count already incremented.
+    p may be a raw device address (a slot of the parameter pool) holding g.numel() elements of g's dtype."""
+    for x in (g, m, v):
+        _dev(x)
+    if isinstance(p, int):
+        if p_out is None:
+            p_out = p
+    else:
+        _dev(p)
+        if p.dtype != g.dtype or p.numel() != g.numel():
+            raise RuntimeError("mole_amd.adam_step: p and g must agree in dtype and size")
+        p_out = p if p_out is None else p_out
+    if not isinstance(p_out, int):
+        _dev(p_out)
+        if p_out.dtype != g.dtype or p_out.numel() != g.numel():
+            raise RuntimeError("mole_amd.adam_step: p_out and g must agree in dtype and size")
+    if m.dtype != torch.float32 or v.dtype != torch.float32:
+        raise RuntimeError("mole_amd.adam_step: m and v are fp32")
+    n = g.numel()
+    if not (m.numel() == v.numel() == n):
+        raise RuntimeError("mole_amd.adam_step: g, m, v must have the same number of elements")
+    L.check(L.lib().mole_adam_step(L.ptr(p), L.ptr(g), L.ptr(m), L.ptr(v), L.ptr(p_out), n, L.dtype_code(g.dtype),
+                                   float(beta1), float(beta2), int(t), float(lr), float(lam), float(eps), int(bool(adamw)),
+                                   L.stream()), "mole_adam_step")

@@ -63,9 +63,16 @@ class CPUHostBatchedParameter(object):
             self.all_tensors.adam_state = self.adam_state
             self.all_tensors.grad_ = torch.zeros((count, *list(size)), dtype=dtype, pin_memory=pin)
             self.all_tensors.grad_.lazy_zero = True
-            self.all_tensors.momentum = None   # optimizer state: allocated by the optimizer side
-            self.all_tensors.variance = None
-            moe.set_CPUParamCore(p_id, self.all_tensors, self.all_tensors.grad_, None, None, self.bias, self.p_id)
+            # Adam moments (Uparam.py:178-181), fp32 whatever the parameter dtype.  Pinned memory is
+            # scarce, so they exist only when the core runs the in-pipeline Adam that reads them.
+            if getattr(moe, "adv_adam", False):
+                self.all_tensors.momentum = torch.zeros((count, *list(size)), dtype=torch.float32, pin_memory=pin)
+                self.all_tensors.variance = torch.zeros((count, *list(size)), dtype=torch.float32, pin_memory=pin)
+            else:
+                self.all_tensors.momentum = None
+                self.all_tensors.variance = None
+            moe.set_CPUParamCore(p_id, self.all_tensors, self.all_tensors.grad_, self.all_tensors.momentum,
+                                 self.all_tensors.variance, self.bias, self.p_id)
         else:
             self.all_tensors = None
 

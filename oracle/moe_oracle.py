@@ -24,6 +24,8 @@ Sources followed, function by function (paths are inside the reference tree):
   d_gelu_tanh          MOLE/cpp/gelu.cu:3-14
   UniMemModel          MOLE/cpp/umemory.cpp:92-183, MOLE/cpp/core.cpp:41-75, 1017-1051
   fast_assign_prefetch MOLE/cpp/core.cpp:1302-1345
+  adam_step            MOLE/cpp/define.hpp:543-579 (_MOLECore::adam, used by instant_adam,
+                       MOLE/cpp/core.cpp:848-943)
 
 Parity status.
   * ffn_fwd / ffn_bwd / d_gelu_tanh / gate_scores reduce to torch library routines and closed
@@ -35,6 +37,8 @@ Parity status.
     for locations, integer closed form for capacity, permutation invariants, adjointness of
     encode/decode backward, torch autograd on a dense one-hot formulation.
   * UniMemModel / fast_assign_prefetch are integer state machines restated from the C++.
+  * adam_step is pinned against torch.optim.Adam and torch.optim.AdamW over several steps in fp64
+    and against hand-computed first-step values (tests/test_oracle_adam.py).
 
 Floating point: everything is evaluated in the dtype of the inputs (fp32 by default; pass fp64
 tensors for an error budget).  bf16 inputs are compared by up-casting the *same rounded values*
@@ -541,3 +545,30 @@ def fast_assign_prefetch(P: int, Fv: Sequence[int], Ev: Sequence[int]):
             stk.append([i, new_gp])
             lp[i] = Ev[i]
     return gp, lp
+
+
+# ---------------------------------------------------------------------------------------------
+# in-pipeline Adam (MOLE/cpp/define.hpp:543-579)
+# ---------------------------------------------------------------------------------------------
+def adam_step(p: torch.Tensor, m: torch.Tensor, v: torch.Tensor, g: torch.Tensor, beta1: float, beta2: float,
+              t_stored: int, lr: float, lam: float, eps: float, adamW: bool, scalar=np.float32):
+    """One update as _MOLECore::adam evaluates it, tensor op by tensor op, in the dtype of the inputs.
+    t_stored is the counter set_adam() stored; the update uses t_stored + 1 (define.hpp:547).
+    The hyper-parameters are C++ floats in the reference (define.hpp:521), so 1 - beta, lam * lr and
+    1 - lam * lr are formed in single precision (scalar=np.float32); std::pow(float, int) promotes to double,
+    and so does 1 - pow.  scalar=np.float64 gives the textbook double-precision constants.
+    Returns (p_new, m_new, v_new); the inputs are left untouched."""
+    f = scalar
+    beta1, beta2, lr, lam, eps = f(beta1), f(beta2), f(lr), f(lam), f(eps)
+    one = f(1)
+    t = t_stored + 1
+    if adamW:
+        p = p * float(one - lam * lr)
+    else:
+        g = g + float(lam) * p
+    m = float(beta1) * m + float(one - beta1) * g
+    v = float(beta2) * v + float(one - beta2) * g * g
+    mt = m / (1.0 - float(beta1) ** t)
+    vt = v / (1.0 - float(beta2) ** t)
+    p = p - float(lr) * mt / (vt.sqrt() + float(eps))
+    return p, m, v

@@ -10,7 +10,7 @@ from tests.util import rel_err, tol
 pytestmark = pytest.mark.gpu
 
 
-def _build(S, M, E, k, Fd, dtype, d_experts=0, pool=0, ebatch=4, seed=0, **kw):
+def _build(S, M, E, k, Fd, dtype, d_experts=0, pool=0, ebatch=4, seed=0, acc_step=1, adv_adam=False, **kw):
     from mole_amd.moe.layer import MOLEModule
     MOLEModule.reset_instances()
     g = torch.Generator().manual_seed(seed)
@@ -19,7 +19,7 @@ def _build(S, M, E, k, Fd, dtype, d_experts=0, pool=0, ebatch=4, seed=0, **kw):
     w1, b1 = torch.randn(E, Fd, M, generator=g) * 0.02, torch.randn(E, Fd, generator=g) * 0.02
     w2, b2 = torch.randn(E, Fd, M, generator=g) * 0.02, torch.randn(E, M, generator=g) * 0.02
     m = MOLEModule(d_experts, E - d_experts, M, Fd, pool if d_experts else -1, k, ebatch,
-                   {"local_rank": 0, "world_size": 1, "rank": 0}, "gelu", 1, False, d_experts > 0, dtype=dtype, **kw)
+                   {"local_rank": 0, "world_size": 1, "rank": 0}, "gelu", acc_step, adv_adam, d_experts > 0, dtype=dtype, **kw)
     s = E - d_experts
     with torch.no_grad():
         m.gate[0].linear.weight.copy_(wg)
