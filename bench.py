@@ -32,8 +32,8 @@ PEAK_HBM_GBS = 8000.0
 # WRITE_SIZE runs of this script scaled by the same counters' readings for a copy of known size
 # (profiles/bench_c2_hbm_traffic.txt); other workloads have no counter run and report null
 MEASURED_TRAFFIC_BYTES = {
-    "c2": {"ffn_fwd1": 758.2e6, "ffn_fwd2": 460.7e6, "ffn_gw2": 537.2e6, "ffn_da": 745.0e6, "ffn_gw1": 537.2e6,
-           "ffn_gx": 460.5e6},
+    "c2": {"ffn_fwd1": 771.5e6, "ffn_fwd2": 360.9e6, "ffn_gw2": 537.1e6, "ffn_da": 689.9e6, "ffn_gw1": 537.1e6,
+           "ffn_gx": 381.5e6},
 }
 
 
@@ -219,6 +219,25 @@ def main():
     timing = L.kernel_timing_read()
     L.kernel_timing_enable(False)
 
+    # the fused Adam update on one weight array of this layer ([E, F, M] parameters and gradients in the
+    # layer's dtype, fp32 moments): not part of the step above, measured for its own HBM roofline
+    from mole_amd import hip_ops as H
+    pdt = torch.bfloat16 if w["dtype"] == "bf16" else torch.float32
+    n_adam = w["E"] * w["F"] * w["M"]
+    ap_, ag_ = (torch.randn(n_adam, device="cuda") * 0.02).to(pdt), (torch.randn(n_adam, device="cuda") * 1e-3).to(pdt)
+    am_, av_ = torch.zeros(n_adam, device="cuda"), torch.zeros(n_adam, device="cuda")
+    H.adam_step(ap_, ag_, am_, av_, 0.9, 0.999, 1, 1e-3, 0.0, 1e-8, False)
+    torch.cuda.synchronize()
+    L.kernel_timing_enable(True)
+    for i in range(5):
+        H.adam_step(ap_, ag_, am_, av_, 0.9, 0.999, 2 + i, 1e-3, 0.0, 1e-8, False)
+    torch.cuda.synchronize()
+    adam_cnt, adam_ms = L.kernel_timing_read()["adam"]
+    L.kernel_timing_enable(False)
+    del ap_, ag_, am_, av_
+    adam_bytes = n_adam * (22.0 if pdt == torch.bfloat16 else 28.0)   # read p, g, m, v; write p, m, v
+    adam_gbs = adam_bytes / (adam_ms / adam_cnt * 1e-3) / 1e9
+
     R = int(m.last_route.offsets[-1].item())       # kept (token, choice) rows
     S, M, F, k = w["S"], w["M"], w["F"], w["k"]
     b = 2 if w["dtype"] == "bf16" else 4
@@ -260,6 +279,9 @@ def main():
         "hbm_permutes": {n: {"achieved": kernels[n]["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
                              "frac": round(kernels[n]["gbs"] / PEAK_HBM_GBS, 4)}
                          for n in ("dispatch_fwd", "combine_fwd", "combine_bwd", "dispatch_bwd") if n in kernels},
+        "hbm_optimizer": {"adam_step": {"achieved": round(adam_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                        "frac": round(adam_gbs / PEAK_HBM_GBS, 4), "elements": n_adam,
+                                        "avg_us": round(adam_ms / adam_cnt * 1e3, 2)}},
         "kernels": kernels,
     }
     if not args.no_cpu_baseline:
