@@ -463,24 +463,35 @@ static int ffn_bwd_t(const void *go, const void *xd, const void *h, const void *
     g.offsets = offsets; g.kept = kept; g.E = E; g.m_tiles_bound = m_tiles;
     g.accumulate = accumulate; g.gelu_bwd = gelu_bwd;
     const int wg_tiles = E * ceil_div(F, TBM) * ceil_div(M, TBN);
-    // g_w2[e] = a^T . go          (contract over the expert's rows)
-    g.A = a; g.lda = F; g.B = go; g.ldb = M; g.M = F; g.N = M; g.C = g_w2; g.ldc = M; g.strideC = (long)F * M;
-    if (int rc = run_gemm<T, true, true, true, EPI_WGRAD>(g, max_rows, wg_tiles, st, MOLE_K_FFN_GW2)) return rc;
+    // The bias gradients are sums of go and of t over every expert's rows: go and t are operands of the two
+    // weight-gradient products, whose 256-wide kernel sums an operand on the side (one more MFMA against a
+    // block of ones in the blocks that see the whole operand).  Other kernels leave them to bias_grad_kernel.
+    GemmArgs gw2{};
+    gw2 = g;
+    gw2.A = a; gw2.lda = F; gw2.B = go; gw2.ldb = M; gw2.M = F; gw2.N = M; gw2.C = g_w2; gw2.ldc = M; gw2.strideC = (long)F * M;
+    bool fused_sums = false;
+    if constexpr (sizeof(T) == 2)
+        fused_sums = fast_path_enabled() && gemm256_sums_operand(gw2, MOLE_K_FFN_GW2) && gemm256_sums_operand(gw2, MOLE_K_FFN_GW1);
+    // g_w2[e] = a^T . go          (contract over the expert's rows); g_b2 = sum go
+    if (fused_sums) { gw2.colsum = g_b2; gw2.colsum_side = 2; }
+    if (int rc = run_gemm<T, true, true, true, EPI_WGRAD>(gw2, max_rows, wg_tiles, st, MOLE_K_FFN_GW2)) return rc;
     // t = (go . w2^T) * gelu'(h)   (w2 [F,M]: K = M contiguous)
     g.A = go; g.lda = M; g.B = w2; g.ldb = M; g.strideB = (long)F * M; g.N = F; g.K = M; g.C = t; g.ldc = F; g.H = h;
     if (int rc = run_gemm<T, false, false, false, EPI_DGELU>(g, max_rows, m_tiles * ceil_div(F, TBN), st, MOLE_K_FFN_DA)) return rc;
-    // g_b2 = sum go ; g_b1 = sum t
-    {
-    ScopedTiming timing(MOLE_K_FFN_GB, st);
-    const int cols_per_block = 512 / (int)sizeof(T);
-    const int nb2 = ceil_div(M, cols_per_block), nb1 = ceil_div(F, cols_per_block);
-    hipLaunchKernelGGL(bias_grad_kernel<T>, dim3(nb2 + nb1, E), dim3(BG_WAVES * 64), 0, st, (const T *)go, M, (T *)g_b2, nb2,
-                       (const T *)t, F, (T *)g_b1, offsets, kept, accumulate);
-    MOLE_LAUNCH_CHECK();
+    if (!fused_sums) {
+        // g_b2 = sum go ; g_b1 = sum t
+        ScopedTiming timing(MOLE_K_FFN_GB, st);
+        const int cols_per_block = 512 / (int)sizeof(T);
+        const int nb2 = ceil_div(M, cols_per_block), nb1 = ceil_div(F, cols_per_block);
+        hipLaunchKernelGGL(bias_grad_kernel<T>, dim3(nb2 + nb1, E), dim3(BG_WAVES * 64), 0, st, (const T *)go, M, (T *)g_b2, nb2,
+                           (const T *)t, F, (T *)g_b1, offsets, kept, accumulate);
+        MOLE_LAUNCH_CHECK();
     }
-    // g_w1[e] = t^T . xd
+    // g_w1[e] = t^T . xd ; g_b1 = sum t
     g.A = t; g.lda = F; g.B = xd; g.ldb = M; g.M = F; g.N = M; g.C = g_w1; g.ldc = M; g.strideC = (long)F * M;
+    if (fused_sums) { g.colsum = g_b1; g.colsum_side = 1; }
     if (int rc = run_gemm<T, true, true, true, EPI_WGRAD>(g, max_rows, wg_tiles, st, MOLE_K_FFN_GW1)) return rc;
+    g.colsum = nullptr; g.colsum_side = 0;
     // gx = t . w1                  (w1 [F,M]: K = F strided)
     if (gx != nullptr) {
         g.A = t; g.lda = F; g.B = w1; g.ldb = M; g.strideB = (long)F * M; g.N = M; g.K = F; g.C = gx; g.ldc = M;

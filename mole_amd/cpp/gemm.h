@@ -53,11 +53,14 @@ struct GemmArgs {
     int gelu_bwd;           // EPI_DGELU: MOLE_GELU_BWD_*
     int n_blocks;           // real number of tiles in the launch (grid is rounded up to 8)
     int full_blocks;        // 256-wide kernel, row-ragged: block slots reserved for full m-tiles
+    void *colsum;           // weight gradients, 256-wide kernel: [E][M] (side 1) or [E][N] (side 2) sums of an operand
+    int colsum_side;        //   over the expert's rows: 1 = the m-side operand (A), 2 = the n-side operand (B)
 };
 
 
 // 256x256 bf16 tiles with direct-to-LDS loads (gemm256.hip).  Returns -100 when the shape does not
 // meet its alignment requirements; the caller then uses the generic kernel.
 int launch_gemm256(const GemmArgs &g, bool a_ks, bool b_ks, bool wg, int epi, int max_rows, hipStream_t st, int kid);
+bool gemm256_sums_operand(const GemmArgs &g, int kid);
 
 }  // namespace mole

@@ -222,11 +222,25 @@ template <int TMB, int WM, bool M_KS, bool N_KS, int TMC, int TMCW> struct Frags
         }
     }
     __device__ __forceinline__ void read(const char *stage, int wm, int wn, int kk) { read_part<0, 1>(stage, wm, wn, kk); }
-    // the 2 TMCW MFMAs of a k-sub-step dealt to NP parts
-    template <int P, int NP> __device__ __forceinline__ void mma_part(f32x16 (&acc)[TL::TMW][2]) const {
+    // the 2 TMCW MFMAs of a k-sub-step dealt to NP parts.  SUM: the last part adds one MFMA against a block of
+    // ones, which sums one operand block over k: of the m-side (SUM 1; wave column i takes the wave row's
+    // m-block i) or of the n-side (SUM 2; wave row j takes the wave column's n-block j).
+    template <int P, int NP, int SUM> __device__ __forceinline__ void mma_part(f32x16 (&acc)[TL::TMW][2], f32x16 &sums, int wm, int wn) const {
 #pragma unroll
         for (int i = part_lo<P, NP, 2 * TMCW>(); i < part_lo<P + 1, NP, 2 * TMCW>(); ++i)
             acc[i >> 1][i & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(n[i & 1], m[i >> 1], acc[i >> 1][i & 1], 0, 0, 0);
+        if constexpr (SUM != 0 && P == NP - 1) {
+            const bf16_t one = (bf16_t)1.0f;
+            const bf16x8 ones = {one, one, one, one, one, one, one, one};
+            if constexpr (SUM == 1) {
+#pragma unroll
+                for (int i = 0; i < TMCW; ++i)
+                    if (wn == i) sums = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, m[i], sums, 0, 0, 0);
+            } else {
+                if (wm == 0) sums = __builtin_amdgcn_mfma_f32_32x32x16_bf16(n[0], ones, sums, 0, 0, 0);
+                else sums = __builtin_amdgcn_mfma_f32_32x32x16_bf16(n[1], ones, sums, 0, 0, 0);
+            }
+        }
     }
 };
 
@@ -290,10 +304,10 @@ template <int TMB, int WM, bool M_KS, bool N_KS, bool WG, int TMC> struct Feeder
 // iteration s+1 the rest, into the buffer that stage s-1 has left.  One synchronisation point per
 // iteration, between the halves: wait until this wave's share of stage s+1 has landed (newer stages may
 // still be in flight), then the barrier.
-template <int TMB, int WM, bool M_KS, bool N_KS, bool WG, int TMC, int TMCW>
+template <int TMB, int WM, bool M_KS, bool N_KS, bool WG, int TMC, int TMCW, int SUM>
 __device__ __forceinline__ void main_loop(const bf16_t *Mp, long ldm, int m0, int m_ext, const bf16_t *Np, long ldn,
                                           int n0, int n_ext, int k_ext, char *smem, int wave, int wm, int wn,
-                                          f32x16 (&acc)[Tile<TMB, WM>::TMW][2]) {
+                                          f32x16 (&acc)[Tile<TMB, WM>::TMW][2], f32x16 &sums) {
     typedef Tile<TMB, WM> TL;
     typedef Stage<TMB, WM, M_KS, TMC> SG;
     constexpr int AHEAD = SG::NSTAGE - 1, NP = 4;
@@ -332,7 +346,7 @@ __device__ __forceinline__ void main_loop(const bf16_t *Mp, long ldm, int m0, in
 #define MOLE_HALF(P, J0, N, S_LOAD, BUF, FR, STAGE_PTR, KK, FM)                                           \
         fd.template issue<(J0) + part_lo<P, NP, (N)>(), (J0) + part_lo<P + 1, NP, (N)>()>(S_LOAD, BUF);   \
         FR.template read_part<P, NP>(STAGE_PTR, wm, wn, KK);                                                \
-        FM.template mma_part<P, NP>(acc);                                                                 \
+        FM.template mma_part<P, NP, SUM>(acc, sums, wm, wn);                                              \
         __builtin_amdgcn_sched_barrier(0);
         MOLE_HALF(0, SPLIT ? LH : 0, SPLIT ? L - LH : 0, s + AHEAD - 1, fill_b, f1, cur, 1, f0)
         MOLE_HALF(1, SPLIT ? LH : 0, SPLIT ? L - LH : 0, s + AHEAD - 1, fill_b, f1, cur, 1, f0)
@@ -509,6 +523,40 @@ __device__ __forceinline__ void epilogue(const GemmArgs &g, f32x16 (&acc)[Tile<T
     }
 }
 
+// Writes the operand sums of a weight-gradient block (see Frags::mma_part): colsum[e][i] (+)= sum over the
+// expert's rows of operand column i.  SUM 1: every register of lane l < 32 holds the sum for row l of the wave's
+// summed m-block (block wn of wave row wm); SUM 2: register 4q+j of a lane holds the sum for column
+// 8q + 4 (lane/32) + j of the wave's summed n-block (block wm of wave column wn).
+template <int SUM, int C>
+__device__ __forceinline__ void store_sums(const GemmArgs &g, const f32x16 &sums, int e, int m0, int n0, int m_ext, int wm,
+                                           int wn, int lane) {
+    bf16_t *out = (bf16_t *)g.colsum;
+    if constexpr (SUM == 1) {
+        const int m = m0 + (wm * C + wn) * 32 + (lane & 31);
+        if (lane < 32 && wn < C && m < m_ext) {
+            bf16_t *p = out + (long)e * g.M + m;
+            float v = sums[0];
+            if (g.accumulate) v += (float)*p;
+            *p = (bf16_t)v;
+        }
+    } else {
+        if ((lane & 31) == 0) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int n = n0 + wn * 64 + wm * 32 + 8 * q + 4 * (lane >> 5) + j;
+                    if (n < g.N) {
+                        bf16_t *p = out + (long)e * g.N + n;
+                        float v = sums[4 * q + j];
+                        if (g.accumulate) v += (float)*p;
+                        *p = (bf16_t)v;
+                    }
+                }
+        }
+    }
+}
+
 // Row-ragged (!WG): C[rows_e, N] = Mop[rows_e, K] . Nop_e ; Mop K-contiguous, Nop_e [N,K] or (N_KS) [K,N].
 // Weight gradient (WG): C_e[M, N] = sum_{r in rows_e} Mop[r, M]^T . Nop[r, N], both K-strided.
 template <int TMB, int WM, bool N_KS, bool WG, int EPI>
@@ -523,6 +571,7 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
     //      tiles is only known here (the grid is sized for the worst case), hence the device-side sum.
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n_tiles = (g.N + Q_BN - 1) / Q_BN;
+    int sum_nt = 0, sum_mt = 0;   // weight gradients: the n-tile / m-tile whose block also sums the m-side / n-side operand
     int e, mt, nt, m_ext, k_ext, tile_h = Q_BM;   // tile_h: rows of this tile's m-tiles (row-ragged products cut experts evenly)
     long row0;  // first row of the expert
     if constexpr (!WG) {
@@ -590,6 +639,13 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
         e = unit / m_tiles;
         mt = unit % m_tiles;
         nt = slot % n_tiles;
+        // Blocks that also sum an operand run an eighth longer.  Consecutive slots of an XCD go to its four
+        // shader engines in turn and are handed out in order, so an engine that always gets the long blocks
+        // holds up the other three: the summing n-tile moves on from unit to unit, which gives every engine the
+        // same number of long blocks in every round; the summing m-tile moves on from expert to expert, which
+        // spreads those blocks over the XCDs.
+        sum_nt = (slot / n_tiles) % n_tiles;
+        sum_mt = e % m_tiles;
         m_ext = g.M;
         k_ext = g.kept ? g.kept[e] : g.single_rows;
         row0 = g.offsets ? g.offsets[e] : 0;
@@ -600,6 +656,8 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
     mt = __builtin_amdgcn_readfirstlane(mt);
     tile_h = __builtin_amdgcn_readfirstlane(tile_h);
     nt = __builtin_amdgcn_readfirstlane(nt);
+    sum_nt = __builtin_amdgcn_readfirstlane(sum_nt);
+    sum_mt = __builtin_amdgcn_readfirstlane(sum_mt);
     m_ext = __builtin_amdgcn_readfirstlane(m_ext);
     k_ext = __builtin_amdgcn_readfirstlane(k_ext);
     row0 = ((long)__builtin_amdgcn_readfirstlane((int)(row0 >> 32)) << 32) | (unsigned)__builtin_amdgcn_readfirstlane((int)row0);
@@ -621,14 +679,30 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
     const int wm = WM == 1 ? 0 : wu >> 2, wn = wu & 3;     // wave row / wave column
     uint2 bias_raw[8];
     load_bias<EPI>(g, e, n0, lane, wn, bias_raw);
+    // Operand sums ride along in the weight-gradient blocks that see the whole operand once: one n-tile
+    // of every m-tile for the m-side, one m-tile of every n-tile for the n-side.  These blocks run the
+    // full tile shape (blocks past the operand's end repeat its last row and are not stored).
+    int sum_side = 0;
+    if constexpr (WG && WM == 2 && TMW == 4) {
+        if (g.colsum != nullptr && ((g.colsum_side == 1 && nt == sum_nt) || (g.colsum_side == 2 && mt == sum_mt))) sum_side = g.colsum_side;
+    }
     // The live blocks are dealt evenly to the wave rows: c to each (the last row may find fewer live).
-    const int c = (tmc + WM - 1) / WM;
+    const int c = sum_side ? TMW : (tmc + WM - 1) / WM;
     const int m0w = m0 + wm * c * 32, live_w = max(0, min(live - wm * c * 32, c * 32));
     // K loop and epilogue with C blocks per wave row
-#define MOLE_RUN_TILE(C)                                                                                                  \
+    f32x16 sums;
+#pragma unroll
+    for (int q = 0; q < 16; ++q) sums[q] = 0.f;
+#define MOLE_RUN_TILE_SUM(C, SUM)                                                                                         \
     {                                                                                                                     \
-        main_loop<TMB, WM, M_KS, N_KS, WG, WM *(C), (C)>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wu, wm, wn, acc); \
+        main_loop<TMB, WM, M_KS, N_KS, WG, WM *(C), (C), SUM>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wu, wm, wn, acc, sums); \
+        if constexpr (SUM != 0) store_sums<SUM, (C)>(g, sums, e, m0, n0, m_ext, wm, wn, lane);                            \
         epilogue<TMB, WM, WG, EPI, (C)>(g, acc, smem, lane, wu, wn, e, row0, m0w, n0, m_ext, live_w, bias_raw);      \
+    }
+#define MOLE_RUN_TILE(C) MOLE_RUN_TILE_SUM(C, 0)
+    if constexpr (WG && WM == 2 && TMW == 4) {
+        if (sum_side == 1) { MOLE_RUN_TILE_SUM(TMW, 1) return; }
+        if (sum_side == 2) { MOLE_RUN_TILE_SUM(TMW, 2) return; }
     }
     if constexpr (WM == 1) {
         if (c > TMB / 2) MOLE_RUN_TILE(TMB)
@@ -642,6 +716,7 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
         else MOLE_RUN_TILE(1)
     }
 #undef MOLE_RUN_TILE
+#undef MOLE_RUN_TILE_SUM
 }
 
 template <int TMB, int WM, bool N_KS, bool WG, int EPI>
@@ -705,6 +780,16 @@ static int tile_blocks_for(int kid) {
     }();
     if (forced == 4 || forced == 8 || forced == 16) return forced;
     return (kid == MOLE_K_FFN_FWD2 || kid == MOLE_K_FFN_GX || kid == MOLE_K_FFN_DA) ? 20 : 16;
+}
+
+// Whether the weight-gradient launch for g will also produce the operand sums asked for in g.colsum
+// (the eight-wave 256-row tile does; the tuning variants and the generic kernel do not).
+bool gemm256_sums_operand(const GemmArgs &g, int kid) {
+    if (g.lda % 8 || g.ldb % 8 || g.ldc % 8 || g.N % 8 || g.M % 8) return false;
+    const int tmb = tile_blocks_for(kid);
+    static const bool off = getenv("MOLE_NO_SUMS") != nullptr;   // tuning aid: bias gradients from their own kernel
+    if (off) return false;
+    return tmb == 16 || tmb == 20;
 }
 
 int launch_gemm256(const GemmArgs &g, bool a_ks, bool b_ks, bool wg, int epi, int max_rows, hipStream_t st, int kid) {

@@ -81,10 +81,10 @@ def test_ffn_fwd_bwd_matches_oracle(E, M, Fd, rows, gap, gelu_bwd, dtype):
     assert rel_err(g_w1, w_gw1) < t
     assert rel_err(g_b1, w_gb1) < t
     # accumulate variant (bffn_bwd_acc): a second call adds the same gradients again
-    if dtype == torch.float32:
-        H.ffn_bwd(c["go"], c["xd"], h, a, off, n, c["w1"], c["w2"], g_w1, g_b1, g_w2, g_b2, False, True, mode)
-        assert rel_err(g_w1, 2 * w_gw1) < t and rel_err(g_b2, 2 * w_gb2) < t
-        assert rel_err(g_w2, 2 * w_gw2) < t and rel_err(g_b1, 2 * w_gb1) < t
+    # (bf16: the running sum is rounded to bf16 after every call)
+    H.ffn_bwd(c["go"], c["xd"], h, a, off, n, c["w1"], c["w2"], g_w1, g_b1, g_w2, g_b2, False, True, mode)
+    assert rel_err(g_w1, 2 * w_gw1) < t and rel_err(g_b2, 2 * w_gb2) < t
+    assert rel_err(g_w2, 2 * w_gw2) < t and rel_err(g_b1, 2 * w_gb1) < t
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
