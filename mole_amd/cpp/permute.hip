@@ -468,7 +468,11 @@ extern "C" int mole_gate_wgrad(const float *dlogits, const void *x, int dtype, i
     MOLE_REQUIRE(dwg != nullptr, "mole_gate_wgrad: null output");
     hipStream_t st = (hipStream_t)stream;
     if (S == 0) {
-        MOLE_HIP(hipMemsetAsync(dwg, 0, (size_t)E * M * sizeof(float), st));
+        // no tokens: the reduction over zero partials writes the zeros (a kernel, not a memset, so that a
+        // caller may capture the call in a graph)
+        MOLE_REQUIRE(aligned16(dwg), "mole_gate_wgrad: misaligned output");
+        hipLaunchKernelGGL(gate_wgrad_reduce_kernel, dim3(ceil_div(E * M, 64)), dim3(256), 0, st, (const float *)dwg, 0, E * M, dwg);
+        MOLE_LAUNCH_CHECK();
         return 0;
     }
     MOLE_REQUIRE(dlogits && x && workspace && aligned16(x) && aligned16(dwg) && aligned16(workspace), "mole_gate_wgrad: null or misaligned pointer");
