@@ -48,6 +48,10 @@ CASES = [
     (3, 136, 264, [257, 31, 129], 3),
     (8, 256, 512, [100, 200, 0, 1, 300, 128, 127, 129], 0),
     (2, 512, 2048, [1024, 1000], 24),
+    # more experts than one wave of the tile search covers, most of them nearly empty
+    (150, 64, 256, [(7 * e) % 23 if e % 3 else 0 for e in range(149)] + [700], 0),
+    # an expert with more rows than four 320-row tiles, and column counts that are not whole tiles
+    (3, 264, 520, [1500, 3, 321], 5),
 ]
 
 
@@ -97,3 +101,39 @@ def test_gemm_nt_gate_logits(dtype):
         c = H.gemm_nt(a.cuda(), b.cuda())
         want = a.float() @ b.float().t()
         assert rel_err(c, want) < (1e-5 if dtype == torch.float32 else 1e-4)   # fp32 accumulation of exact products
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_ffn_random_shapes_bf16(seed):
+    """Random expert counts, loads and (8-aligned) widths through the bf16 grouped kernels."""
+    from mole_amd import hip_ops as H, _lib as L
+    rng = np.random.default_rng(100 + seed)
+    E = int(rng.integers(1, 40))
+    M = int(rng.integers(1, 40)) * 8
+    Fd = int(rng.integers(1, 80)) * 8
+    rows = [int(r) for r in rng.choice([0, 1, 31, 32, 33, 255, 256, 257, 320, 321, 640, 700], size=E)]
+    gap = int(rng.integers(0, 3))
+    print(f"ffn random seed={seed} E={E} M={M} F={Fd} rows={rows} gap={gap}", flush=True)
+    dtype = torch.bfloat16
+    d = _make(E, M, Fd, rows, dtype, seed=seed, pad_between=gap)
+    c = {k: (v.cuda() if torch.is_tensor(v) else v) for k, v in d.items()}
+    off = torch.from_numpy(d["off"]).cuda(); n = torch.from_numpy(d["n"]).cuda()
+    out, h, a = H.ffn_fwd(c["xd"], off, n, c["w1"], c["b1"], c["w2"], c["b2"])
+    w_out, w_h, w_gx, w_gw1, w_gb1, w_gw2, w_gb2 = _oracle_fwd_bwd(d, "tanh")
+    t = tol(dtype)
+    mask = torch.zeros(max(d["R"], 1), dtype=torch.bool)
+    for e in range(E):
+        mask[int(d["off"][e]):int(d["off"][e]) + int(d["n"][e])] = True
+    if mask.any():
+        assert rel_err(h.cpu()[mask], w_h[mask]) < t
+        assert rel_err(out.cpu()[mask], w_out[mask]) < t
+    g_w1 = torch.full_like(c["w1"], 9.0); g_w2 = torch.full_like(c["w2"], 9.0)
+    g_b1 = torch.full_like(c["b1"], 9.0); g_b2 = torch.full_like(c["b2"], 9.0)
+    gx = H.ffn_bwd(c["go"], c["xd"], h, a, off, n, c["w1"], c["w2"], g_w1, g_b1, g_w2, g_b2, True, False, L.GELU_BWD_TANH)
+    if mask.any():
+        assert rel_err(gx.cpu()[mask], w_gx[mask]) < t
+        assert rel_err(g_w2, w_gw2) < t and rel_err(g_b2, w_gb2) < t
+        assert rel_err(g_w1, w_gw1) < t and rel_err(g_b1, w_gb1) < t
+    else:   # no rows at all: every gradient is exactly zero
+        for gt in (g_w1, g_b1, g_w2, g_b2):
+            assert float(gt.float().abs().max()) == 0.0
