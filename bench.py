@@ -112,7 +112,7 @@ def bench_offloaded_stack(args):
     for i in range(n_layers):
         print(f"[c4] building layer {i} (pinned host weights)", file=sys.stderr, flush=True)
         try:
-            layers.append(MOLEModule(E, 0, M, F, pool, k, ebatch, dist, "gelu", 1, False, True, dtype=torch.bfloat16))
+            layers.append(MOLEModule(E, 0, M, F, pool, k, ebatch, dist, "gelu", 1, bool(args.adam), True, dtype=torch.bfloat16))
         except RuntimeError as exc:     # pinned host memory is capped well below the machine's RAM on some boxes
             print(f"[c4] layer {i} could not be built ({str(exc).splitlines()[0]}): lower --layers", file=sys.stderr)
             sys.exit(3)
@@ -123,7 +123,13 @@ def bench_offloaded_stack(args):
     dy = (torch.randn(S, M, generator=g) * 1e-3).to(torch.bfloat16).cuda()
     um = core.get_UniMem()
 
+    step_no = [0]
+
     def one_step():
+        if args.adam:     # the optimizer hands the hyper-parameters and its step counter to every layer
+            for m in layers:
+                m.MOLECore.set_adam(0.9, 0.999, step_no[0], 1e-4, 0.01, 1e-8, True, -1)
+            step_no[0] += 1
         layers[0].prefetch_fwd(E)                 # what the scheduler does before the first layer
         h = x
         for m in layers:
@@ -137,6 +143,7 @@ def bench_offloaded_stack(args):
         print(f"[c4] warm-up step {i}", file=sys.stderr, flush=True)
         one_step()
     torch.cuda.synchronize(); core.synchronize_tran()
+    um.copy_stats(); um.writeback_stats()         # forget the warm-up's copies
     t0 = time.perf_counter()
     for i in range(args.steps):
         print(f"[c4] timed step {i}", file=sys.stderr, flush=True)
@@ -161,11 +168,12 @@ def bench_offloaded_stack(args):
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall * 1e3, 2),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"c4: {n_layers}-layer offloaded-expert stack fwd+bwd, S={S} M={M} E={E} top-{k} F={F}, "
-                               f"experts in pinned host memory, pool {pool} slots, chunks of {ebatch} experts"},
+                               f"experts in pinned host memory, pool {pool} slots, chunks of {ebatch} experts"
+                               + (", in-pipeline AdamW on the GPU (fp32 moments in pinned host memory)" if args.adam else "")},
         "prefetch": {"h2d_bytes_per_step": int(h2d_bytes), "h2d_busy_ms": round(h2d_ms, 2),
                      "h2d_gbs": round(h2d_bytes / (h2d_ms * 1e-3) / 1e9, 2),
                      "h2d_busy_frac_of_step": round(h2d_ms / (wall * 1e3), 4),
-                     "expected_h2d_bytes": 2 * n_layers * E * expert_bytes,
+                     "expected_h2d_bytes": (2 + (4 if args.adam else 0)) * n_layers * E * expert_bytes,
                      "d2h_gradient_bytes_per_step": int(d2h_bytes), "d2h_busy_ms": round(d2h_ms, 2),
                      "d2h_gbs": round(d2h_bytes / (d2h_ms * 1e-3) / 1e9, 2)},
         "kernel_ms_per_step": round(kernel_ms, 2),
@@ -183,6 +191,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c4"])
     ap.add_argument("--layers", type=int, default=2, help="depth of the c4 stack (12 in the configuration)")
+    ap.add_argument("--adam", action="store_true",
+                    help="c4 only: update the offloaded experts with the in-pipeline Adam (adds 30 GB of pinned moments per layer)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:

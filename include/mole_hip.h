@@ -225,8 +225,9 @@ int mole_unimem_wait_params(void *handle, mole_stream_t compute_stream);
 int mole_unimem_release(void *handle, int view_base, int n, mole_stream_t compute_stream);
 int mole_unimem_sync_tran(void *handle);
 int mole_unimem_tran_stream(void *handle, mole_stream_t *out);
-/* bytes moved host->device and the copy stream's busy time between the two most recent
- * mole_unimem_sync_tran() calls, measured with events on the copy stream */
+/* bytes moved host->device and the copy stream's busy time (events on the copy stream), summed over the copies
+ * that mole_unimem_sync_tran() calls have waited for since the previous mole_unimem_copy_stats(); reading
+ * resets the sums */
 int mole_unimem_copy_stats(void *handle, uint64_t *bytes, float *busy_ms);
 
 /* Gradient write-back of offloaded experts; replaces _MOLECore::store_grad / _CPUParamCore::store_grad
@@ -236,7 +237,8 @@ int mole_unimem_copy_stats(void *handle, uint64_t *bytes, float *busy_ms);
  * second library-owned stream once the work already enqueued on compute_stream has finished.  The caller
  * keeps dev_src alive until that stream has passed the copy (mole_unimem_tranback_stream tells which) and
  * reads the host arrays only after mole_unimem_sync_tranback().  Overwrites; accumulation is the caller's.
- * mole_unimem_writeback_stats: bytes and copy time between the two most recent sync_tranback calls. */
+ * mole_unimem_writeback_stats: bytes and copy time of the write-backs that sync_tranback calls have waited for
+ * since the previous read; reading resets the sums. */
 int mole_unimem_store_grads(void *handle, void *const host_dst[4], const void *const dev_src[4], int base,
                             int n, mole_stream_t compute_stream);
 int mole_unimem_sync_tranback(void *handle);
@@ -249,12 +251,14 @@ int mole_unimem_writeback_stats(void *handle, uint64_t *bytes, float *busy_ms);
  * store_batch_cpu_para/mome/vari on the tranback stream).
  * mole_unimem_load_state: count host->device copies of bytes[i] from pinned host_src[i] to dev_dst[i] on
  * the library's copy stream, which first waits for the work already enqueued on compute_stream (the
- * previous users of dev_dst); compute_stream then waits for the copies.
+ * previous users of dev_dst) and, when after_writeback != 0, for the write-backs enqueued so far (set it when
+ * host_src may be the target of one, e.g. gradients stored by the previous micro-step; it serialises the two
+ * copy directions); compute_stream then waits for the copies.
  * mole_unimem_store_state: count device->host copies on the write-back stream once the work already
  * enqueued on compute_stream has finished; lifetime and synchronisation rules as for
  * mole_unimem_store_grads. */
 int mole_unimem_load_state(void *handle, void *const dev_dst[], const void *const host_src[], const size_t bytes[],
-                           int count, mole_stream_t compute_stream);
+                           int count, int after_writeback, mole_stream_t compute_stream);
 int mole_unimem_store_state(void *handle, void *const host_dst[], const void *const dev_src[], const size_t bytes[],
                             int count, mole_stream_t compute_stream);
 

@@ -63,7 +63,7 @@ _SIGNATURES = {
     "mole_unimem_sync_tranback": (c_int, [_P]),
     "mole_unimem_tranback_stream": (c_int, [_P, POINTER(_P)]),
     "mole_unimem_writeback_stats": (c_int, [_P, POINTER(c_uint64), POINTER(c_float)]),
-    "mole_unimem_load_state": (c_int, [_P, POINTER(_P), POINTER(_P), POINTER(c_size_t), c_int, _P]),
+    "mole_unimem_load_state": (c_int, [_P, POINTER(_P), POINTER(_P), POINTER(c_size_t), c_int, c_int, _P]),
     "mole_unimem_store_state": (c_int, [_P, POINTER(_P), POINTER(_P), POINTER(c_size_t), c_int, _P]),
     "mole_adam_step": (c_int, [_P, _P, _P, _P, _P, c_size_t, c_int, c_float, c_float, c_int, c_float, c_float, c_float,
                                c_int, _P]),

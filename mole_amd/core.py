@@ -114,15 +114,16 @@ class UniMem:
         L.check(getattr(L.lib(), getter)(self._h, ctypes.byref(out)), getter)
         return torch.cuda.ExternalStream(int(out.value), device=device)
 
-    def load_state(self, dev_tensors, host_tensors):
+    def load_state(self, dev_tensors, host_tensors, after_writeback: bool = False):
         """Pinned host arrays -> device tensors of the same sizes on the copy stream (after the compute already
         enqueued on the current stream, which then waits for the copies): optimizer moments and accumulated
-        gradients of an expert batch (core.cpp:864-915)."""
+        gradients of an expert batch (core.cpp:864-915).  after_writeback: the host arrays may still be the target
+        of a write-back in flight (gradients of the previous micro-step), so the copies wait for that stream too."""
         dp, sizes = self._arrays(dev_tensors)
         hp, hs = self._arrays(host_tensors)
         if list(sizes) != list(hs):
             raise RuntimeError("UniMem.load_state: host and device sizes differ")
-        L.check(L.lib().mole_unimem_load_state(self._h, dp, hp, sizes, len(dev_tensors), L.stream()),
+        L.check(L.lib().mole_unimem_load_state(self._h, dp, hp, sizes, len(dev_tensors), int(after_writeback), L.stream()),
                 "mole_unimem_load_state")
         tran = self._side_stream("mole_unimem_tran_stream", dev_tensors[0].device)
         for t in dev_tensors:
@@ -453,7 +454,7 @@ class MOLECore:
         if acc:
             g_prev = [torch.empty((n, *hg.shape[1:]), dtype=hg.dtype, device=dev) for hg in host_grads]
             loads_dev, loads_host = loads_dev + g_prev, loads_host + [hg[base:base + n] for hg in host_grads]
-        um.load_state(loads_dev, loads_host)
+        um.load_state(loads_dev, loads_host, after_writeback=acc)
         p_new = []
         for k in range(4):
             gk = g[k][:n]

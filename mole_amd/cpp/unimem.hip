@@ -248,8 +248,8 @@ extern "C" int mole_unimem_sync_tran(void *handle) {
         MOLE_HIP(hipEventElapsedTime(&ms, u->timers[i][0], u->timers[i][1]));
         total += ms;
     }
-    u->ms_last = total;
-    u->bytes_last = u->bytes_open;
+    u->ms_last += total;
+    u->bytes_last += u->bytes_open;
     u->bytes_open = 0;
     u->timers_used = 0;
     return 0;
@@ -283,7 +283,8 @@ extern "C" int mole_unimem_store_grads(void *handle, void *const host_dst[4], co
 }
 
 extern "C" int mole_unimem_load_state(void *handle, void *const dev_dst[], const void *const host_src[],
-                                      const size_t bytes[], int count, mole_stream_t compute_stream) {
+                                      const size_t bytes[], int count, int after_writeback,
+                                      mole_stream_t compute_stream) {
     UM(handle);
     MOLE_REQUIRE(dev_dst && host_src && bytes && count >= 0, "mole_unimem_load_state: bad arguments count=%d", count);
     if (count == 0) return 0;
@@ -292,9 +293,12 @@ extern "C" int mole_unimem_load_state(void *handle, void *const dev_dst[], const
     // the destination may have been in use by work already enqueued on the compute stream
     MOLE_HIP(hipEventRecord(u->state_free, (hipStream_t)compute_stream));
     MOLE_HIP(hipStreamWaitEvent(u->tran, u->state_free, 0));
-    // and the host arrays may still be the target of an earlier write-back (gradients of the previous micro-step)
-    MOLE_HIP(hipEventRecord(u->wb_done, u->tranback));
-    MOLE_HIP(hipStreamWaitEvent(u->tran, u->wb_done, 0));
+    // the host arrays may still be the target of an earlier write-back (gradients of the previous micro-step):
+    // then the copies also wait for the write-back stream, which costs the overlap of the two directions
+    if (after_writeback) {
+        MOLE_HIP(hipEventRecord(u->wb_done, u->tranback));
+        MOLE_HIP(hipStreamWaitEvent(u->tran, u->wb_done, 0));
+    }
     std::array<hipEvent_t, 2> *tm;
     if (int rc = next_timer(u, &tm)) return rc;
     MOLE_HIP(hipEventRecord((*tm)[0], u->tran));
@@ -344,8 +348,8 @@ extern "C" int mole_unimem_sync_tranback(void *handle) {
         MOLE_HIP(hipEventElapsedTime(&ms, u->wb_timers[i][0], u->wb_timers[i][1]));
         total += ms;
     }
-    u->wb_ms_last = total;
-    u->wb_bytes_last = u->wb_bytes_open;
+    u->wb_ms_last += total;
+    u->wb_bytes_last += u->wb_bytes_open;
     u->wb_bytes_open = 0;
     u->wb_timers_used = 0;
     return 0;
@@ -361,6 +365,8 @@ extern "C" int mole_unimem_writeback_stats(void *handle, uint64_t *bytes, float 
     UM(handle);
     if (bytes) *bytes = u->wb_bytes_last;
     if (busy_ms) *busy_ms = u->wb_ms_last;
+    u->wb_bytes_last = 0;
+    u->wb_ms_last = 0.f;
     return 0;
 }
 
@@ -374,6 +380,8 @@ extern "C" int mole_unimem_copy_stats(void *handle, uint64_t *bytes, float *busy
     UM(handle);
     if (bytes) *bytes = u->bytes_last;
     if (busy_ms) *busy_ms = u->ms_last;
+    u->bytes_last = 0;
+    u->ms_last = 0.f;
     return 0;
 }
 
