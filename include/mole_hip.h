@@ -88,7 +88,8 @@ int mole_softmax_fwd(const float *logits, const float *logit_bias, int S, int E,
 /* The whole of MOLETopk.forward (MOLE/utils/Ugate.py:11-14) in one kernel for bf16 tokens:
  * scores[S,E] = softmax(x[S,M] . wg[E,M]^T + logit_bias), wg fp32 (rounded to bf16 for the products, fp32
  * accumulation), logit_bias [E] or NULL.  Needs dtype == MOLE_BF16, M a multiple of 128, E <= 256; other
- * cases use mole_gemm_nt + mole_softmax_fwd. */
+ * cases use mole_gemm_nt + mole_softmax_fwd.  Every block of 16 tokens reads all of wg, so beyond a few dozen
+ * experts the two-kernel path is the faster one (the Python host side switches at E = 32). */
 int mole_gate_fwd(const void *x, int dtype, const float *wg, const float *logit_bias, int S, int E, int M,
                   float *scores, mole_stream_t stream);
 int mole_gate_bwd(const float *dgates, const float *scores, const int32_t *idx, int S, int E,

@@ -46,13 +46,17 @@ def softmax_fwd(logits: torch.Tensor, logit_bias: Optional[torch.Tensor] = None)
     return scores
 
 
-def gate_fwd(x: torch.Tensor, wg: torch.Tensor, logit_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """scores [S,E] fp32 = softmax(x @ wg.T + logit_bias): one fused kernel for bf16 tokens (M % 128 == 0, E <= 256),
-    the NT GEMM followed by the softmax kernel otherwise."""
+def gate_fwd(x: torch.Tensor, wg: torch.Tensor, logit_bias: Optional[torch.Tensor] = None,
+             fused: Optional[bool] = None) -> torch.Tensor:
+    """scores [S,E] fp32 = softmax(x @ wg.T + logit_bias): one fused kernel for bf16 tokens and small gates
+    (M % 128 == 0, E <= 32: a block of 16 tokens re-reads all of wg, which only pays while wg is small), the NT
+    GEMM followed by the softmax kernel otherwise.  fused=True asks for the one-kernel path at any E <= 256."""
     _dev(x), _dev(wg)
     S, M = x.shape
     E = wg.shape[0]
-    if x.dtype == torch.bfloat16 and wg.dtype == torch.float32 and M % 128 == 0 and E <= 256:
+    if fused is None:
+        fused = x.dtype == torch.bfloat16 and wg.dtype == torch.float32 and M % 128 == 0 and E <= 32
+    if fused:
         scores = torch.empty(S, E, dtype=torch.float32, device=x.device)
         L.check(L.lib().mole_gate_fwd(L.ptr(x), L.dtype_code(x.dtype), L.ptr(wg), L.ptr(logit_bias), S, E, M, L.ptr(scores),
                                       L.stream()), "mole_gate_fwd")

@@ -108,7 +108,7 @@ def test_fused_gate_forward(S, E, M, bias):
     x = torch.randn(S, M, generator=g).bfloat16()
     wg = torch.randn(E, M, generator=g) * 0.05
     b = torch.log(torch.arange(1, E + 1, dtype=torch.float32) ** -1.2) if bias else None
-    got = H.gate_fwd(x.cuda(), wg.cuda(), b.cuda() if bias else None).cpu()
+    got = H.gate_fwd(x.cuda(), wg.cuda(), b.cuda() if bias else None, fused=True).cpu()
     want = O.gate_scores(x.float(), wg.bfloat16().float(), b)
     assert got.shape == (S, E)
     assert rel_err(got, want) < 1e-4
