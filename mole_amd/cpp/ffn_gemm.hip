@@ -432,6 +432,8 @@ static int run_gemm(const GemmArgs &g, int max_rows, int tiles_generic, hipStrea
             if (rc != -100) return rc;
         }
     }
+    // only the 256-wide kernel sums an operand on the side: the caller asks gemm256_sums_operand() first
+    MOLE_REQUIRE(g.colsum == nullptr, "grouped GEMM: operand sums requested from a kernel that does not produce them");
     return launch_gemm<T, A_KS, B_KS, WG, TBM, TBN, EPI>(g, tiles_generic, st, kid);
 }
 

@@ -39,16 +39,22 @@ struct UniMem {
     float wb_ms_last = 0.f;
 };
 
-static int next_timer(UniMem *u, std::array<hipEvent_t, 2> **out) {
-    if (u->timers_used == u->timers.size()) {
+// The next event pair of a copy stream's statistics.  A caller that never synchronises the stream would
+// grow the list without bound: past MAX_TIMERS pairs the last one is reused (the statistics then miss the
+// copies in between; nothing else depends on them).
+constexpr size_t MAX_TIMERS = 4096;
+static int next_timer(std::vector<std::array<hipEvent_t, 2>> &timers, size_t &used, std::array<hipEvent_t, 2> **out) {
+    if (used == MAX_TIMERS) --used;
+    if (used == timers.size()) {
         std::array<hipEvent_t, 2> p;
         MOLE_HIP(hipEventCreate(&p[0]));
         MOLE_HIP(hipEventCreate(&p[1]));
-        u->timers.push_back(p);
+        timers.push_back(p);
     }
-    *out = &u->timers[u->timers_used++];
+    *out = &timers[used++];
     return 0;
 }
+static int next_timer(UniMem *u, std::array<hipEvent_t, 2> **out) { return next_timer(u->timers, u->timers_used, out); }
 
 // Host -> pool copy of experts [base, base+n) into slots [slot0, slot0+n).  The copy is cut at every
 // slot whose previous user has not been waited for yet, so that a prefetch trails the compute that
@@ -264,13 +270,9 @@ extern "C" int mole_unimem_store_grads(void *handle, void *const host_dst[4], co
         MOLE_REQUIRE(host_dst[p] && dev_src[p], "mole_unimem_store_grads: null buffer for parameter kind %d", p);
     MOLE_HIP(hipEventRecord(u->grads_ready, (hipStream_t)compute_stream));
     MOLE_HIP(hipStreamWaitEvent(u->tranback, u->grads_ready, 0));
-    if (u->wb_timers_used == u->wb_timers.size()) {
-        std::array<hipEvent_t, 2> p;
-        MOLE_HIP(hipEventCreate(&p[0]));
-        MOLE_HIP(hipEventCreate(&p[1]));
-        u->wb_timers.push_back(p);
-    }
-    auto &tm = u->wb_timers[u->wb_timers_used++];
+    std::array<hipEvent_t, 2> *tmp;
+    if (int rc = next_timer(u->wb_timers, u->wb_timers_used, &tmp)) return rc;
+    auto &tm = *tmp;
     MOLE_HIP(hipEventRecord(tm[0], u->tranback));
     for (int p = 0; p < 4; ++p) {
         const size_t sb = u->slot_bytes[p];
@@ -322,13 +324,9 @@ extern "C" int mole_unimem_store_state(void *handle, void *const host_dst[], con
         MOLE_REQUIRE(bytes[i] == 0 || (host_dst[i] && dev_src[i]), "mole_unimem_store_state: null buffer %d", i);
     MOLE_HIP(hipEventRecord(u->grads_ready, (hipStream_t)compute_stream));
     MOLE_HIP(hipStreamWaitEvent(u->tranback, u->grads_ready, 0));
-    if (u->wb_timers_used == u->wb_timers.size()) {
-        std::array<hipEvent_t, 2> p;
-        MOLE_HIP(hipEventCreate(&p[0]));
-        MOLE_HIP(hipEventCreate(&p[1]));
-        u->wb_timers.push_back(p);
-    }
-    auto &tm = u->wb_timers[u->wb_timers_used++];
+    std::array<hipEvent_t, 2> *tmp;
+    if (int rc = next_timer(u->wb_timers, u->wb_timers_used, &tmp)) return rc;
+    auto &tm = *tmp;
     MOLE_HIP(hipEventRecord(tm[0], u->tranback));
     for (int i = 0; i < count; ++i) {
         if (bytes[i] == 0) continue;

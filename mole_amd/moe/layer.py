@@ -258,6 +258,68 @@ class MOLEModule(torch.nn.Module):
                 MOLEModule._instance[-1].local_prefetch_bwd()
         return out
 
+    # ---- optimizer hooks (layer.py:135-136, 343-348) --------------------------------------------
+    def set_hybrid_adam_count(self, hybrid_adam_count):
+        self.MOLECore.set_hybrid_adam_count(hybrid_adam_count)
+
+    def unset_lazy_zero(self):
+        for p in (self.FC1_W_CPU, self.FC1_B_CPU, self.FC2_W_CPU, self.FC2_B_CPU):
+            p.unset_lazy_zero()
+
+    # ---- layer state for checkpoints (layer.py:350-427) ------------------------------------------
+    def _expert_stores(self):
+        """(parameter store of kind p for the GPU-resident experts, for the offloaded ones), p = 0..3"""
+        return ((self.FC1_W_GPU, self.FC1_W_CPU), (self.FC1_B_GPU, self.FC1_B_CPU),
+                (self.FC2_W_GPU, self.FC2_W_CPU), (self.FC2_B_GPU, self.FC2_B_CPU))
+
+    @torch.no_grad()
+    def get_layer_state(self, grad):
+        """{"gate": [weight, bias or None], "experts": one [fc1_w, fc1_b, fc2_w, fc2_b] per expert (GPU-resident
+        first, then offloaded), "grad": the same per expert, then the gate's gradients; empty unless grad}: all
+        CPU tensors, the layout MOLEModule.get_layer_state returns in the reference."""
+        core.synchronize_tran()           # host arrays may still be the target of a write-back
+        lin = self.gate[0].linear
+        state = {"gate": [lin.weight.detach().cpu(), lin.bias.detach().cpu() if lin.bias is not None else None]}
+        experts, grads = [], []
+        for which, count in ((0, self.s_experts), (1, self.d_experts)):
+            for i in range(count):
+                experts.append([st[which].fetch_single(i).detach().cpu().clone() for st in self._expert_stores()])
+        if grad:
+            for which, count in ((0, self.s_experts), (1, self.d_experts)):
+                for i in range(count):
+                    grads.append([st[which].fetch_single_grad(i).detach().cpu().clone() for st in self._expert_stores()])
+            grads.append(lin.weight.grad.cpu() if lin.weight.grad is not None else None)
+            grads.append(lin.bias.grad.cpu() if lin.bias is not None and lin.bias.grad is not None else None)
+        state["experts"], state["grad"] = experts, grads
+        return state
+
+    @torch.no_grad()
+    def set_layer_state(self, states, grad):
+        """Inverse of get_layer_state (layer.py:350-395)."""
+        core.synchronize_tran()           # no prefetch may be reading the host arrays while they change
+        torch.cuda.synchronize()
+        lin = self.gate[0].linear
+        lin.weight.copy_(states["gate"][0])
+        if lin.bias is not None:
+            lin.bias.copy_(states["gate"][1])
+        j = 0
+        for which, count in ((0, self.s_experts), (1, self.d_experts)):
+            for i in range(count):
+                for st, t in zip(self._expert_stores(), states["experts"][j]):
+                    st[which].fetch_single(i).copy_(t)
+                j += 1
+        if grad:
+            gs = states["grad"]
+            j = 0
+            for which, count in ((0, self.s_experts), (1, self.d_experts)):
+                for i in range(count):
+                    for st, t in zip(self._expert_stores(), gs[j]):
+                        st[which].fetch_single_grad(i).copy_(t)
+                    j += 1
+            lin.weight.grad = None if gs[j] is None else gs[j].to(lin.weight.device)
+            if lin.bias is not None and gs[j + 1] is not None:
+                lin.bias.grad = gs[j + 1].to(lin.bias.device)
+
     # ---- parameter access (layer.py:478-500) ---------------------------------------------------
     def d_experts_param(self):
         if self.d_experts > 0:

@@ -196,3 +196,33 @@ def test_layer_degenerate_inputs():
         m, x, ref = _build(50, 64, 4, 2, 128, dtype, seed=7)
         res = _run_and_compare(m, x, ref, 2, 0.001, dtype)
         assert res.crit.capacity == 0 and float(res.y.abs().max()) == 0.0
+
+
+def test_layer_state_round_trip():
+    """get_layer_state / set_layer_state (the reference's checkpoint payload, layer.py:350-427): a second layer
+    loaded from the first one's state computes the same output and holds the same gradients."""
+    S, M, E, k, Fd, dtype = 300, 64, 6, 2, 128, torch.float32
+    m1, x, _ = _build(S, M, E, k, Fd, dtype, d_experts=4, pool=4, ebatch=2, seed=1)
+    xin = x.clone().requires_grad_(True)
+    y1 = m1(xin, capacity_factor=1.0)
+    y1.backward(torch.ones_like(y1) * 1e-2)
+    torch.cuda.synchronize()
+    state = m1.get_layer_state(True)
+    assert len(state["experts"]) == E and len(state["grad"]) == E + 2
+    assert all(t.device.type == "cpu" for ex in state["experts"] for t in ex)
+    y1 = y1.detach().clone()
+    # MOLEModule keeps one slot pool per process: the first layer goes away before the second is built
+    m2, _, _ = _build(S, M, E, k, Fd, dtype, d_experts=4, pool=4, ebatch=2, seed=2)
+    y_other = m2(x, capacity_factor=1.0).detach()
+    assert not torch.allclose(y_other, y1)
+    m2.set_layer_state(state, True)
+    y2 = m2(x, capacity_factor=1.0).detach()
+    assert torch.equal(y2, y1)
+    back = m2.get_layer_state(True)
+    for a, b in zip(state["experts"] + state["grad"][:E], back["experts"] + back["grad"][:E]):
+        assert all(torch.equal(u, v) for u, v in zip(a, b))
+    assert torch.equal(state["grad"][E], back["grad"][E]) and back["grad"][E + 1] is None
+    m2.unset_lazy_zero()
+    assert m2.FC1_W_CPU.all_tensors.grad_.lazy_zero is False
+    m2.set_hybrid_adam_count(3)
+    assert m2.MOLECore.hybrid_adam_count == 3
