@@ -211,6 +211,137 @@ __global__ __launch_bounds__(256) void dispatch_bwd_gate_kernel(const T *__restr
     }
 }
 
+// The same for bf16 tokens with the gate product on the matrix cores.  dlogits . Wg is a [tokens x E] by
+// [E x M] product with E <= 32: one v_mfma_f32_16x16x32_bf16 per 16 tokens x 16 columns, both operands rounded
+// to bf16 (the sum is rounded to bf16 on the way out anyway).  The fp32 kernel above spends 2 E VALU
+// instructions per pair of output elements on it, which is what bounds it; here the VALU work is the
+// unpack / add / pack of a copy.
+// A block of eight waves covers 1024 columns, a wave 128 columns of 16 tokens at a time: its 8 product tiles go
+// through an 8 KB LDS buffer of its own (the MFMA result has a lane hold one column of four tokens; the
+// row-major side wants 16 bytes of one token per lane), then every lane gathers 8 columns of one token's k
+// source rows, adds and stores 16 bytes.  The first-choice gathers of a group of tokens are issued one group ahead.
+constexpr int DM_TOKENS = 32;                 // tokens per block: two groups of 16
+constexpr int DM_COLS = 128;                  // columns per wave
+constexpr int DM_ROW = DM_COLS + 4;           // floats per token row of the LDS buffer: 4 rows apart = 16 banks apart
+typedef __bf16 perm_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float perm_f32x4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(512) void dispatch_bwd_gate_mfma_kernel(const bf16_t *__restrict__ dxd,
+                                                                     const int32_t *__restrict__ row, int S, int M, int k,
+                                                                     const float *__restrict__ dlogits,
+                                                                     const float *__restrict__ wg, int E,
+                                                                     bf16_t *__restrict__ dx) {
+    __shared__ __align__(16) float s_t[8][16 * DM_ROW];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r16 = lane & 15, kq = lane >> 4;
+    const int col0 = (blockIdx.y * 8 + wave) * DM_COLS;      // this wave's first column
+    if (col0 >= M) return;                                   // M is a multiple of 128: whole waves drop out
+    float *buf = s_t[wave];
+    const int tsel = lane >> 4, c8 = (lane & 15) * 8;        // row-major side: token within a quartet, first of 8 columns
+    // the first-choice source rows of the 4 tokens this lane finishes in a group (tokens tok0 + 4 u + tsel)
+    auto gather = [&](uint4 (&v)[4], int tok0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int t = tok0 + 4 * u + tsel;
+            const int r = t < S ? row[t] : -1;
+            v[u] = r >= 0 ? *reinterpret_cast<const uint4 *>(dxd + (size_t)r * M + col0 + c8) : make_uint4(0, 0, 0, 0);
+        }
+    };
+    uint4 src[4];
+    gather(src, blockIdx.x * DM_TOKENS);
+    // B fragments: Wg[8 kq + i][col0 + 16 cb + r16], i = 0..7, for the wave's 8 column blocks.  Fetched row by row
+    // with 16-byte loads (a lane takes 4 columns of the 8 experts of one group) and turned by way of the LDS
+    // buffer, [expert group][column] with a group's 8 experts as one bf16x8 entry: picking them out of global
+    // memory one float at a time took longer than the rest of the kernel.  Two expert groups per pass.
+    perm_bf16x8 bfrag[8];
+    {
+        perm_bf16x8 *wt = reinterpret_cast<perm_bf16x8 *>(buf);      // [2][DM_COLS]
+        const int c4 = (lane & 31) * 4, half = lane >> 5;
+#pragma unroll
+        for (int pass = 0; pass < 2; ++pass) {
+            if (pass * 16 >= E) break;
+            const int eg = 2 * pass + half;
+            float4 w[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int e = 8 * eg + i;
+                w[i] = e < E ? *reinterpret_cast<const float4 *>(wg + (size_t)e * M + col0 + c4) : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+            perm_bf16x8 *dst = wt + half * DM_COLS + c4;
+            dst[0] = perm_bf16x8{(bf16_t)w[0].x, (bf16_t)w[1].x, (bf16_t)w[2].x, (bf16_t)w[3].x,
+                                 (bf16_t)w[4].x, (bf16_t)w[5].x, (bf16_t)w[6].x, (bf16_t)w[7].x};
+            dst[1] = perm_bf16x8{(bf16_t)w[0].y, (bf16_t)w[1].y, (bf16_t)w[2].y, (bf16_t)w[3].y,
+                                 (bf16_t)w[4].y, (bf16_t)w[5].y, (bf16_t)w[6].y, (bf16_t)w[7].y};
+            dst[2] = perm_bf16x8{(bf16_t)w[0].z, (bf16_t)w[1].z, (bf16_t)w[2].z, (bf16_t)w[3].z,
+                                 (bf16_t)w[4].z, (bf16_t)w[5].z, (bf16_t)w[6].z, (bf16_t)w[7].z};
+            dst[3] = perm_bf16x8{(bf16_t)w[0].w, (bf16_t)w[1].w, (bf16_t)w[2].w, (bf16_t)w[3].w,
+                                 (bf16_t)w[4].w, (bf16_t)w[5].w, (bf16_t)w[6].w, (bf16_t)w[7].w};
+            // the lanes whose expert group (kq) this pass staged pick up their fragments
+            if ((kq >> 1) == pass) {
+#pragma unroll
+                for (int cb = 0; cb < 8; ++cb) bfrag[cb] = wt[(kq & 1) * DM_COLS + 16 * cb + r16];
+            }
+        }
+        if (8 * kq >= E) {        // expert groups past the gate's size contribute nothing
+            const bf16_t z = (bf16_t)0.0f;
+#pragma unroll
+            for (int cb = 0; cb < 8; ++cb) bfrag[cb] = perm_bf16x8{z, z, z, z, z, z, z, z};
+        }
+    }
+#pragma unroll
+    for (int g0 = 0; g0 < DM_TOKENS; g0 += 16) {
+        const int tok0 = blockIdx.x * DM_TOKENS + g0;
+        uint4 nxt[4];
+        if (g0 + 16 < DM_TOKENS) gather(nxt, tok0 + 16);
+        // A fragment: dlogits[tok0 + r16][8 kq .. 8 kq + 7]
+        float d[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int e = 8 * kq + i;
+            d[i] = (tok0 + r16 < S && e < E) ? dlogits[(size_t)(tok0 + r16) * E + e] : 0.f;
+        }
+        const perm_bf16x8 afrag = {(bf16_t)d[0], (bf16_t)d[1], (bf16_t)d[2], (bf16_t)d[3],
+                                   (bf16_t)d[4], (bf16_t)d[5], (bf16_t)d[6], (bf16_t)d[7]};
+        // product tiles into LDS: acc[r] = token 4 kq + r, column 16 cb + r16 (conflict-free: see DM_ROW)
+#pragma unroll
+        for (int cb = 0; cb < 8; ++cb) {
+            const perm_f32x4 acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag, bfrag[cb], perm_f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) buf[(4 * kq + r) * DM_ROW + 16 * cb + r16] = acc[r];
+        }
+        // (a wave's LDS buffer is written and read by that wave only: program order is enough)
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int tl = 4 * u + tsel, t = tok0 + tl;
+            const float4 p0 = *reinterpret_cast<const float4 *>(buf + tl * DM_ROW + c8);
+            const float4 p1 = *reinterpret_cast<const float4 *>(buf + tl * DM_ROW + c8 + 4);
+            float acc[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
+            Vec<bf16_t> v;
+            float f[8];
+            v.raw = src[u];
+            v.unpack(f);
+#pragma unroll
+            for (int q = 0; q < 8; ++q) acc[q] += f[q];
+            for (int j = 1; j < k; ++j) {
+                const int r = t < S ? row[(size_t)j * S + t] : -1;
+                if (r >= 0) {
+                    v.load(dxd + (size_t)r * M + col0 + c8);
+                    v.unpack(f);
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) acc[q] += f[q];
+                }
+            }
+            if (t < S) {
+                v.pack(acc);
+                v.store(dx + (size_t)t * M + col0 + c8);
+            }
+        }
+        if (g0 + 16 < DM_TOKENS) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) src[u] = nxt[u];
+        }
+    }
+}
+
 // Gate weight gradient dWg[e, m] = sum_i dlogits[i, e] * x[i, m] (the Linear backward that
 // autograd runs for MOLETopk, MOLE/utils/Ugate.py:12), in two deterministic passes: blocks of
 // GW_TOKENS tokens write partial [E, M] sums, a second kernel adds the partials in order.
@@ -432,6 +563,13 @@ extern "C" int mole_dispatch_bwd(const void *dxd, int dtype, const int32_t *row,
                  "mole_dispatch_bwd: dlogits given without a valid wg/E");
     ScopedTiming timing(MOLE_K_DISPATCH_BWD, (hipStream_t)stream);
     MOLE_REQUIRE(dx_add == nullptr || aligned16(dx_add), "mole_dispatch_bwd: misaligned dx_add");
+    if (dlogits != nullptr && dx_add == nullptr && E <= 32 && M % DM_COLS == 0 && dtype == MOLE_BF16) {
+        const dim3 grid(ceil_div(S, DM_TOKENS), ceil_div(M, 8 * DM_COLS));
+        hipLaunchKernelGGL(dispatch_bwd_gate_mfma_kernel, grid, dim3(512), 0, (hipStream_t)stream, (const bf16_t *)dxd, row,
+                           S, M, k, dlogits, wg, E, (bf16_t *)dx);
+        MOLE_LAUNCH_CHECK();
+        return 0;
+    }
     if (dlogits != nullptr && dx_add == nullptr && E <= 32 && M % 4 == 0) {
         const dim3 grid(ceil_div(S, DB_TOKENS), ceil_div(M, 1024));
         hipStream_t st = (hipStream_t)stream;

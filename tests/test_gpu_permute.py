@@ -74,3 +74,27 @@ def test_permute_full_size_properties():
     dx = H.dispatch_bwd(d, r.row)
     rhs = (xi.double() * dx.double()).sum()
     assert float(lhs) == float(rhs)
+
+
+@pytest.mark.parametrize("S,E,k,M,cf", [(100, 16, 1, 256, 1.0), (1000, 3, 2, 512, 0.0), (777, 32, 4, 1280, 0.5),
+                                        (16384, 16, 1, 1024, 1.25), (33, 20, 2, 256, 0.0)])
+def test_dispatch_bwd_with_gate_bf16_wide_rows(S, E, k, M, cf):
+    """The fused dispatch backward for bf16 rows of whole 256-column groups (the matrix-core variant): gather-sum
+    of the kept rows plus dlogits @ Wg, against the oracle's gather and an fp32 product of the bf16-rounded
+    operands (the kernel rounds dlogits and Wg to bf16, which the 2e-2 bf16 tolerance covers either way)."""
+    from mole_amd import hip_ops as H
+    print(f"dispatch_bwd+gate S={S} E={E} k={k} M={M} cf={cf}", flush=True)
+    g = torch.Generator().manual_seed(S + M)
+    scores = zipf_scores(S, E, seed=S)
+    c = O.extract_critical(scores.numpy(), k, cf)
+    r = H.route(scores.cuda(), k, cf)
+    total = int(c.offsets[-1])
+    dxd = torch.randn(max(total, 1), M, generator=g).bfloat16()
+    dlog = torch.randn(S, E, generator=g) * 0.1
+    wg = torch.randn(E, M, generator=g)
+    got = H.dispatch_bwd(dxd.cuda(), r.row, dlog.cuda(), wg.cuda())
+    want = O.fast_encode_bwd(dxd[:total].float(), c, True) + dlog @ wg
+    assert got.shape == (S, M)
+    assert rel_err(got, want) < tol(torch.bfloat16)
+    tight = O.fast_encode_bwd(dxd[:total].float(), c, True) + dlog.bfloat16().float() @ wg.bfloat16().float()
+    assert rel_err(got, tight) < 6e-3          # what is left is the output's own rounding to bf16
