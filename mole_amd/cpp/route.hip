@@ -145,11 +145,8 @@ __global__ __launch_bounds__(RT_THREADS) void route_topk_kernel(
 }
 
 // one wave per (choice, expert) pair: exclusive prefix over blocks, total into counts
-__global__ __launch_bounds__(256) void route_scan_kernel(int32_t *__restrict__ hist, int nb, int npairs,
-                                                         int32_t *__restrict__ counts) {
+__device__ __forceinline__ void scan_pair(int32_t *__restrict__ hist, int nb, int pair, int32_t *__restrict__ counts) {
     const int lane = threadIdx.x & 63;
-    const int pair = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (pair >= npairs) return;
     int carry = 0;
     for (int c0 = 0; c0 < nb; c0 += WAVE) {
         const int bi = c0 + lane;
@@ -164,18 +161,30 @@ __global__ __launch_bounds__(256) void route_scan_kernel(int32_t *__restrict__ h
     }
     if (lane == 0) counts[pair] = carry;
 }
+__global__ __launch_bounds__(256) void route_scan_kernel(int32_t *__restrict__ hist, int nb, int npairs,
+                                                         int32_t *__restrict__ counts) {
+    const int pair = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (pair < npairs) scan_pair(hist, nb, pair, counts);
+}
 
 constexpr int FIN_THREADS = 1024;
 
+// scan_hist != NULL: the block first does the work of route_scan_kernel itself (small problems: one launch
+// less), its 16 waves taking the pairs in turn.
 __global__ __launch_bounds__(FIN_THREADS) void route_finish_kernel(
-    const int32_t *__restrict__ counts, const float *__restrict__ colsum, int nb, int S, int E, int k,
+    int32_t *__restrict__ counts, const float *__restrict__ colsum, int nb, int S, int E, int k,
     int cf_sign, int cap_bound, int alignment, int layout, int32_t *__restrict__ basej,
     int32_t *__restrict__ kept_rows, int32_t *__restrict__ offsets, int32_t *__restrict__ capacity,
-    float *__restrict__ l_aux) {
+    float *__restrict__ l_aux, int32_t *__restrict__ scan_hist) {
     __shared__ int s_n[MOLE_MAX_EXPERTS];
     __shared__ int s_red[FIN_THREADS];
     __shared__ float s_fred[FIN_THREADS];
     const int tid = threadIdx.x;
+    if (scan_hist != nullptr) {
+        for (int pair = tid >> 6; pair < k * E; pair += FIN_THREADS / 64) scan_pair(scan_hist, nb, pair, counts);
+        __threadfence_block();
+        __syncthreads();
+    }
     int lmax = 0;
     for (int e = tid; e < E; e += FIN_THREADS) {
         int tot = 0;
@@ -331,8 +340,11 @@ extern "C" int mole_route(const float *scores, int S, int E, int k, double capac
     MOLE_LAUNCH_CHECK();
 
     const int npairs = k * E;
-    hipLaunchKernelGGL(route_scan_kernel, dim3(ceil_div(npairs, 4)), dim3(256), 0, st, hist, nb, npairs, counts);
-    MOLE_LAUNCH_CHECK();
+    const bool scan_in_finish = (long long)npairs * nb <= 16384;   // small enough for one block: saves a launch
+    if (!scan_in_finish) {
+        hipLaunchKernelGGL(route_scan_kernel, dim3(ceil_div(npairs, 4)), dim3(256), 0, st, hist, nb, npairs, counts);
+        MOLE_LAUNCH_CHECK();
+    }
 
     const int spe = (S + E - 1) / E;
     const int cf_sign = capacity_factor > 0. ? 1 : (capacity_factor < 0. ? -1 : 0);
@@ -340,7 +352,8 @@ extern "C" int mole_route(const float *scores, int S, int E, int k, double capac
     const double prod = (capacity_factor < 0. ? -capacity_factor : capacity_factor) * (double)spe;
     const int cap_bound = k * (int)prod;
     hipLaunchKernelGGL(route_finish_kernel, dim3(1), dim3(FIN_THREADS), 0, st, counts, colsum, nb, S, E, k, cf_sign,
-                       cap_bound, alignment, layout, basej, kept_rows, offsets, capacity, l_aux);
+                       cap_bound, alignment, layout, basej, kept_rows, offsets, capacity, l_aux,
+                       scan_in_finish ? hist : (int32_t *)nullptr);
     MOLE_LAUNCH_CHECK();
 
     if (S > 0) {
