@@ -405,6 +405,125 @@ __global__ __launch_bounds__(256) void gate_wgrad_partial_kernel(const float *__
         if (e < E)
             *reinterpret_cast<float2 *>(part + ((size_t)blockIdx.x * E + e) * M + m) = make_float2(acc[e][0], acc[e][1]);
 }
+// The partial sums on the matrix cores, for bf16 tokens and gates of up to 256 experts:
+// part[chunk][e][m] = sum over the chunk's tokens of dlogits[t][e] x[t][m], a [E x tokens] by [tokens x M]
+// product per chunk with v_mfma_f32_16x16x32_bf16 and fp32 accumulation.  dlogits is fp32: it enters as the sum
+// of two bf16 numbers (the rounded value and the rounded remainder, 16 significant bits together), each
+// multiplied separately, so the result stays as close to the exact sum as the fp32 accumulation allows.
+// A block of four waves takes one chunk of tokens, 256 columns (64 per wave) and up to 64 experts (grid z walks
+// the rest).  The contraction runs over tokens, along which neither operand is contiguous in memory, so both
+// are turned in LDS: the chunk's dlogits, 128 tokens at a time, into [expert][token] bf16 rows (an A fragment is
+// then one 16-byte read), x 32 tokens at a time per wave as it lies in memory, read back with the transposing
+// ds_read_b64_tr_b16 (a group of 16 lanes receives a 4-token x 16-column block column by column).  The next
+// 32 tokens' global loads are in flight while the current ones are multiplied.
+constexpr int GM_KSTEP = 32;                  // tokens per MFMA
+constexpr int GM_XROW = 72;                   // bf16 per token row of a wave's x tile: 64 columns + 16 bytes,
+                                              // so that the 4 rows of a transposing read fall into distinct banks
+constexpr int GM_SUB = 128;                   // tokens whose dlogits are staged at a time
+constexpr int GM_DLROW = GM_SUB + 8;          // bf16 per expert row of the staged dlogits (+ 16 bytes: bank spread)
+typedef short perm_s16x4 __attribute__((ext_vector_type(4)));
+template <int EG>   // groups of 16 experts per block
+__global__ __launch_bounds__(256) void gate_wgrad_mfma_kernel(const float *__restrict__ dlogits,
+                                                              const bf16_t *__restrict__ x, int S, int E, int M,
+                                                              int chunk, float *__restrict__ part) {
+    __shared__ __align__(16) bf16_t s_dl[2][16 * EG * GM_DLROW];     // leading and remainder halves of dlogits
+    __shared__ __align__(16) bf16_t s_x[4 * GM_KSTEP * GM_XROW];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r16 = lane & 15, kq = lane >> 4;
+    const int tok0 = blockIdx.x * chunk, ntok = min(chunk, S - tok0);
+    const int e0 = blockIdx.z * 16 * EG;
+    const int col0 = blockIdx.y * 256 + wave * 64;
+    const bool active = col0 < M;             // M is a multiple of 64: a wave is in or out as a whole
+    bf16_t *xt = s_x + wave * (GM_KSTEP * GM_XROW);
+    perm_f32x4 acc[EG][4];
+#pragma unroll
+    for (int g = 0; g < EG; ++g)
+#pragma unroll
+        for (int cb = 0; cb < 4; ++cb) acc[g][cb] = perm_f32x4{0.f, 0.f, 0.f, 0.f};
+    // a wave's x tile of one step: 32 tokens x 64 columns = 4 loads of 16 bytes per lane (token 8 i + lane / 8)
+    const int lt = lane >> 3, lc = (lane & 7) * 8;
+    auto fetch = [&](uint4 (&v)[4], int k0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int t = k0 + 8 * i + lt;
+            v[i] = (active && t < ntok) ? *reinterpret_cast<const uint4 *>(x + (size_t)(tok0 + t) * M + col0 + lc)
+                                        : make_uint4(0, 0, 0, 0);
+        }
+    };
+    uint4 cur[4], nxt[4];
+    fetch(cur, 0);
+    for (int sub0 = 0; sub0 < ntok; sub0 += GM_SUB) {
+        // dlogits of the next GM_SUB tokens -> LDS, transposed and rounded (expert fastest across threads: the
+        // global reads are whole rows of dlogits)
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < 16 * EG * GM_SUB; idx += 256) {
+            const int e = idx % (16 * EG), t = idx / (16 * EG);
+            const float v = (sub0 + t < ntok && e0 + e < E) ? dlogits[(size_t)(tok0 + sub0 + t) * E + e0 + e] : 0.f;
+            const bf16_t hi = (bf16_t)v;
+            s_dl[0][e * GM_DLROW + t] = hi;
+            s_dl[1][e * GM_DLROW + t] = (bf16_t)(v - (float)hi);
+        }
+        __syncthreads();
+        const int sub_end = min(ntok, sub0 + GM_SUB);
+        for (int k0 = sub0; k0 < sub_end; k0 += GM_KSTEP) {
+            fetch(nxt, k0 + GM_KSTEP);        // past the chunk's end: zeros, no loads
+#pragma unroll
+            for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4 *>(xt + (8 * i + lt) * GM_XROW + lc) = cur[i];
+            // (the tile is written and read by this wave only: program order is enough)
+            perm_bf16x8 a[EG], al[EG];
+#pragma unroll
+            for (int g = 0; g < EG; ++g) {
+                a[g] = *reinterpret_cast<const perm_bf16x8 *>(s_dl[0] + (16 * g + r16) * GM_DLROW + (k0 - sub0) + 8 * kq);
+                al[g] = *reinterpret_cast<const perm_bf16x8 *>(s_dl[1] + (16 * g + r16) * GM_DLROW + (k0 - sub0) + 8 * kq);
+            }
+#pragma unroll
+            for (int cb = 0; cb < 4; ++cb) {
+                // tokens 8 kq + (r16 >> 2) (+ 4), columns 16 cb + 4 (r16 & 3) ..: lane r16 receives column 16 cb + r16
+                const bf16_t *p = xt + (8 * kq + (r16 >> 2)) * GM_XROW + 16 * cb + 4 * (r16 & 3);
+                const perm_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((perm_s16x4 __attribute__((address_space(3))) *)(p));
+                const perm_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((perm_s16x4 __attribute__((address_space(3))) *)(p + 4 * GM_XROW));
+                typedef short s16x8 __attribute__((ext_vector_type(8)));
+                const s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                const perm_bf16x8 b = __builtin_bit_cast(perm_bf16x8, v);
+#pragma unroll
+                for (int g = 0; g < EG; ++g) {
+                    acc[g][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al[g], b, acc[g][cb], 0, 0, 0);
+                    acc[g][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[g], b, acc[g][cb], 0, 0, 0);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) cur[i] = nxt[i];
+        }
+    }
+    if (!active) return;
+    // acc[g][cb][r] = expert e0 + 16 g + 4 kq + r, column col0 + 16 cb + r16
+    float *out = part + (size_t)blockIdx.x * E * M;
+#pragma unroll
+    for (int g = 0; g < EG; ++g)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int e = e0 + 16 * g + 4 * kq + r;
+            if (e >= E) continue;
+#pragma unroll
+            for (int cb = 0; cb < 4; ++cb) out[(size_t)e * M + col0 + 16 * cb + r16] = acc[g][cb][r];
+        }
+}
+
+// tokens per chunk of the kernel above: chunks of 128 tokens while the partials stay within 32 MB (or 8
+// chunks), twice as long as often as needed beyond
+static int gate_wgrad_mfma_chunk(int S, int E, int M) {
+    const size_t per_chunk = (size_t)E * M * sizeof(float);
+    size_t max_chunks = (32u << 20) / per_chunk;
+    if (max_chunks < 8) max_chunks = 8;
+    int chunk = 128;
+    while ((size_t)ceil_div(S, chunk) > max_chunks && chunk < (1 << 24)) chunk *= 2;
+    return chunk;
+}
+static bool gate_wgrad_mfma_ok(int dtype, int S, int E, int M) {
+    return dtype == MOLE_BF16 && E <= 256 && M % 64 == 0 && S > 0 &&
+           (size_t)ceil_div(S, gate_wgrad_mfma_chunk(S, E, M)) <= 65535;
+}
+
 // sums the partials in a fixed order: 16 slices of the block list per group of four outputs, then the
 // slices in order
 __global__ __launch_bounds__(256) void gate_wgrad_reduce_kernel(const float *__restrict__ part, int nblocks, int EM,
@@ -596,13 +715,18 @@ extern "C" int mole_dispatch_bwd(const void *dxd, int dtype, const int32_t *row,
 
 extern "C" size_t mole_gate_wgrad_workspace_bytes(int S, int E, int M) {
     if (S <= 0 || E <= 0 || M <= 0) return 0;
-    return (size_t)ceil_div(S, GW_TOKENS) * E * M * sizeof(float);
+    // enough for either kernel: the caller does not say the dtype here (small gates: the VALU kernel's 64-token
+    // partials; large gates only run on the matrix cores, with their own chunking)
+    const size_t mfma = (size_t)ceil_div(S, gate_wgrad_mfma_chunk(S, E, M)) * E * M * sizeof(float);
+    const size_t valu = E <= 32 ? (size_t)ceil_div(S, GW_TOKENS) * E * M * sizeof(float) : 0;
+    return mfma > valu ? mfma : valu;
 }
 
 extern "C" int mole_gate_wgrad(const float *dlogits, const void *x, int dtype, int S, int E, int M, float *dwg,
                                void *workspace, size_t workspace_bytes, mole_stream_t stream) {
     MOLE_REQUIRE(dtype == MOLE_F32 || dtype == MOLE_BF16, "mole_gate_wgrad: bad dtype %d", dtype);
-    MOLE_REQUIRE(S >= 0 && E >= 1 && E <= 32 && M > 0 && M % 4 == 0, "mole_gate_wgrad: need 1 <= E <= 32 and M %% 4 == 0 (S=%d E=%d M=%d)", S, E, M);
+    MOLE_REQUIRE(S >= 0 && E >= 1 && M > 0 && M % 4 == 0 && (E <= 32 || gate_wgrad_mfma_ok(dtype, S, E, M) || S == 0),
+                 "mole_gate_wgrad: need E <= 32, or bf16 tokens with E <= 256 and M %% 64 == 0 (S=%d E=%d M=%d dtype=%d)", S, E, M, dtype);
     MOLE_REQUIRE(dwg != nullptr, "mole_gate_wgrad: null output");
     hipStream_t st = (hipStream_t)stream;
     if (S == 0) {
@@ -618,9 +742,21 @@ extern "C" int mole_gate_wgrad(const float *dlogits, const void *x, int dtype, i
         set_error("mole_gate_wgrad: workspace of %zu bytes, need %zu", workspace_bytes, mole_gate_wgrad_workspace_bytes(S, E, M));
         return MOLE_E_WORKSPACE;
     }
+    float *part = (float *)workspace;
+    if (gate_wgrad_mfma_ok(dtype, S, E, M)) {
+        const int chunk = gate_wgrad_mfma_chunk(S, E, M), nchunks = ceil_div(S, chunk);
+        const int eg = E <= 16 ? 1 : (E <= 32 ? 2 : 4);
+        const dim3 grid(nchunks, ceil_div(M, 256), ceil_div(E, 16 * eg));
+#define MOLE_GM(EG) hipLaunchKernelGGL((gate_wgrad_mfma_kernel<EG>), grid, dim3(256), 0, st, dlogits, (const bf16_t *)x, S, E, M, chunk, part)
+        if (eg == 1) MOLE_GM(1); else if (eg == 2) MOLE_GM(2); else MOLE_GM(4);
+#undef MOLE_GM
+        MOLE_LAUNCH_CHECK();
+        hipLaunchKernelGGL(gate_wgrad_reduce_kernel, dim3(ceil_div(E * M, 64)), dim3(256), 0, st, part, nchunks, E * M, dwg);
+        MOLE_LAUNCH_CHECK();
+        return 0;
+    }
     const int nb = ceil_div(S, GW_TOKENS);
     const dim3 grid(nb, ceil_div(M, 512));
-    float *part = (float *)workspace;
 #define MOLE_GW(T, EB) hipLaunchKernelGGL((gate_wgrad_partial_kernel<T, EB>), grid, dim3(256), 0, st, dlogits, (const T *)x, S, E, M, part)
     if (dtype == MOLE_BF16) {
         if (E <= 8) MOLE_GW(bf16_t, 8); else if (E <= 16) MOLE_GW(bf16_t, 16); else MOLE_GW(bf16_t, 32);

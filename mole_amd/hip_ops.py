@@ -78,12 +78,14 @@ def gate_bwd(dgates: torch.Tensor, scores: torch.Tensor, idx: torch.Tensor, norm
 
 
 def gate_wgrad(dlogits: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
-    """dWg [E,M] fp32 = dlogits[S,E]^T @ x[S,M].  Small gates (E <= 32) run the deterministic HIP kernel;
-    larger ones are a plain library GEMM (plumbing)."""
+    """dWg [E,M] fp32 = dlogits[S,E]^T @ x[S,M], deterministic (partial sums over token chunks, added in a fixed
+    order): on the matrix cores for bf16 tokens (E <= 256, M % 64 == 0), on the VALU for small gates (E <= 32) in
+    either dtype.  What neither kernel covers is a plain library GEMM (plumbing)."""
     _dev(dlogits), _dev(x)
     S, E = dlogits.shape
     M = x.shape[1]
-    if E > 32 or M % 4 != 0:
+    mfma = x.dtype == torch.bfloat16 and E <= 256 and M % 64 == 0 and S > 0
+    if not mfma and (E > 32 or M % 4 != 0):
         return (dlogits.t().to(x.dtype) @ x).float()
     dwg = torch.empty(E, M, dtype=torch.float32, device=x.device)
     nbytes = L.lib().mole_gate_wgrad_workspace_bytes(S, E, M)

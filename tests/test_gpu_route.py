@@ -85,7 +85,8 @@ def test_softmax_and_gate_bwd(S, E):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("S,E,M", [(1, 1, 4), (100, 8, 64), (1000, 16, 1024), (333, 32, 520), (70, 5, 2048)])
+@pytest.mark.parametrize("S,E,M", [(1, 1, 4), (100, 8, 64), (1000, 16, 1024), (333, 32, 520), (70, 5, 2048),
+                                   (16384, 16, 1024), (700, 64, 192), (4100, 256, 2048), (129, 100, 320)])
 def test_gate_wgrad(S, E, M, dtype):
     from mole_amd import hip_ops as H
     print(f"gate_wgrad S={S} E={E} M={M} {dtype}", flush=True)
@@ -94,7 +95,9 @@ def test_gate_wgrad(S, E, M, dtype):
     x = torch.randn(S, M, generator=g).to(dtype)
     got = H.gate_wgrad(dl.cuda(), x.cuda())
     want = dl.double().t() @ x.double()
-    assert rel_err(got, want) < 1e-5       # fp32 sums of exact products in both dtypes
+    # fp32 sums of exact products (VALU kernel) or of products with dlogits split into two bf16 parts (matrix
+    # cores, bf16 tokens); fp32 tokens with a large gate go through a library GEMM in fp32
+    assert rel_err(got, want) < 2e-5
 
 
 @pytest.mark.parametrize("S,E,M,bias", [(100, 16, 128, False), (1000, 8, 256, True), (513, 64, 384, False),
