@@ -475,25 +475,31 @@ __global__ __launch_bounds__(256) void gate_bwd_kernel(const float *__restrict__
 typedef __bf16 gate_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float gate_f32x4 __attribute__((ext_vector_type(4)));
 
-template <int EG, int KSTEPS>
+template <int EG, int KSTEPS, int TG>   // TG groups of 16 tokens per block: Wg is read once for all of them
 __global__ __launch_bounds__(256) void gate_fwd_kernel(const bf16_t *__restrict__ x, const float *__restrict__ wg,
                                                        const float *__restrict__ bias, int S, int E, int M,
                                                        float *__restrict__ scores) {
-    __shared__ float part[4][16][EG * 16 + 1];
+    __shared__ float part[4][16 * TG][EG * 16 + 1];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r16 = lane & 15, kq = lane >> 4;
-    const int tok0 = blockIdx.x * 16;
+    const int tok0 = blockIdx.x * 16 * TG;
     const int kbase = wave * (M >> 2) + 8 * kq;
-    const bf16_t *xp = x + (size_t)min(tok0 + r16, S - 1) * M + kbase;
-    gate_f32x4 acc[EG];
+    const bf16_t *xp[TG];
 #pragma unroll
-    for (int g = 0; g < EG; ++g) acc[g] = gate_f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int tg = 0; tg < TG; ++tg) xp[tg] = x + (size_t)min(tok0 + 16 * tg + r16, S - 1) * M + kbase;
+    gate_f32x4 acc[TG][EG];
+#pragma unroll
+    for (int tg = 0; tg < TG; ++tg)
+#pragma unroll
+        for (int g = 0; g < EG; ++g) acc[tg][g] = gate_f32x4{0.f, 0.f, 0.f, 0.f};
     const int nsteps = M >> 7;                    // 32 of k per step, a quarter of M per wave
     for (int s0 = 0; s0 < nsteps; s0 += KSTEPS) {
-        uint4 a[KSTEPS];
+        uint4 a[TG][KSTEPS];
 #pragma unroll
-        for (int i = 0; i < KSTEPS; ++i)
-            a[i] = s0 + i < nsteps ? *reinterpret_cast<const uint4 *>(xp + (s0 + i) * 32) : make_uint4(0, 0, 0, 0);
+        for (int tg = 0; tg < TG; ++tg)
+#pragma unroll
+            for (int i = 0; i < KSTEPS; ++i)
+                a[tg][i] = s0 + i < nsteps ? *reinterpret_cast<const uint4 *>(xp[tg] + (s0 + i) * 32) : make_uint4(0, 0, 0, 0);
 #pragma unroll
         for (int i = 0; i < KSTEPS; ++i) {
             if (s0 + i >= nsteps) break;
@@ -503,38 +509,46 @@ __global__ __launch_bounds__(256) void gate_fwd_kernel(const bf16_t *__restrict_
                 const float4 w0 = *reinterpret_cast<const float4 *>(wp), w1 = *reinterpret_cast<const float4 *>(wp + 4);
                 const gate_bf16x8 b = {(bf16_t)w0.x, (bf16_t)w0.y, (bf16_t)w0.z, (bf16_t)w0.w,
                                        (bf16_t)w1.x, (bf16_t)w1.y, (bf16_t)w1.z, (bf16_t)w1.w};
-                acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(gate_bf16x8, a[i]), b, acc[g], 0, 0, 0);
+#pragma unroll
+                for (int tg = 0; tg < TG; ++tg)
+                    acc[tg][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(gate_bf16x8, a[tg][i]), b, acc[tg][g], 0, 0, 0);
             }
         }
     }
-    // acc[g][r] = partial logit of token 4 kq + r, expert 16 g + r16
+    // acc[tg][g][r] = partial logit of token 16 tg + 4 kq + r, expert 16 g + r16
 #pragma unroll
-    for (int g = 0; g < EG; ++g)
+    for (int tg = 0; tg < TG; ++tg)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) part[wave][4 * kq + r][g * 16 + r16] = acc[g][r];
+        for (int g = 0; g < EG; ++g)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) part[wave][16 * tg + 4 * kq + r][g * 16 + r16] = acc[tg][g][r];
     __syncthreads();
-    const int t = threadIdx.x >> 4, j = threadIdx.x & 15;      // 16 lanes per token
-    const int token = tok0 + t;
-    float v[EG];
-    float mx = -INFINITY;
+    const int j = threadIdx.x & 15;               // 16 lanes per token
 #pragma unroll
-    for (int g = 0; g < EG; ++g) {
-        const int e = g * 16 + j;
-        v[g] = e < E ? part[0][t][e] + part[1][t][e] + part[2][t][e] + part[3][t][e] + (bias ? bias[e] : 0.f) : -INFINITY;
-        mx = fmaxf(mx, v[g]);
-    }
-    for (int m = 8; m >= 1; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m, WAVE));
-    float sum = 0.f;
+    for (int tg = 0; tg < TG; ++tg) {
+        const int t = 16 * tg + (threadIdx.x >> 4);
+        const int token = tok0 + t;
+        float v[EG];
+        float mx = -INFINITY;
 #pragma unroll
-    for (int g = 0; g < EG; ++g) {
-        v[g] = g * 16 + j < E ? expf(v[g] - mx) : 0.f;
-        sum += v[g];
-    }
-    for (int m = 8; m >= 1; m >>= 1) sum += __shfl_xor(sum, m, WAVE);
+        for (int g = 0; g < EG; ++g) {
+            const int e = g * 16 + j;
+            v[g] = e < E ? part[0][t][e] + part[1][t][e] + part[2][t][e] + part[3][t][e] + (bias ? bias[e] : 0.f) : -INFINITY;
+            mx = fmaxf(mx, v[g]);
+        }
+        for (int m = 8; m >= 1; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m, WAVE));
+        float sum = 0.f;
 #pragma unroll
-    for (int g = 0; g < EG; ++g) {
-        const int e = g * 16 + j;
-        if (token < S && e < E) scores[(size_t)token * E + e] = v[g] / sum;
+        for (int g = 0; g < EG; ++g) {
+            v[g] = g * 16 + j < E ? expf(v[g] - mx) : 0.f;
+            sum += v[g];
+        }
+        for (int m = 8; m >= 1; m >>= 1) sum += __shfl_xor(sum, m, WAVE);
+#pragma unroll
+        for (int g = 0; g < EG; ++g) {
+            const int e = g * 16 + j;
+            if (token < S && e < E) scores[(size_t)token * E + e] = v[g] / sum;
+        }
     }
 }
 
@@ -571,15 +585,16 @@ extern "C" int mole_gate_fwd(const void *x, int dtype, const float *wg, const fl
                  dtype);
     if (S == 0) return 0;
     MOLE_REQUIRE(x && wg && scores, "mole_gate_fwd: null pointer");
-    const dim3 grid(ceil_div(S, 16));
     hipStream_t st = (hipStream_t)stream;
     const bf16_t *xb = (const bf16_t *)x;
     const int eg = ceil_div(E, 16);
-    if (eg == 1) hipLaunchKernelGGL((gate_fwd_kernel<1, 8>), grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores);
-    else if (eg == 2) hipLaunchKernelGGL((gate_fwd_kernel<2, 8>), grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores);
-    else if (eg <= 4) hipLaunchKernelGGL((gate_fwd_kernel<4, 4>), grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores);
-    else if (eg <= 8) hipLaunchKernelGGL((gate_fwd_kernel<8, 4>), grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores);
-    else hipLaunchKernelGGL((gate_fwd_kernel<16, 2>), grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores);
+    // small gates: 32 tokens per block (Wg, which every block reads in full, is then read half as often)
+    const dim3 grid(ceil_div(S, eg <= 2 ? 32 : 16));
+    if (eg == 1) hipLaunchKernelGGL((gate_fwd_kernel<1, 8, 2>), grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores);
+    else if (eg == 2) hipLaunchKernelGGL((gate_fwd_kernel<2, 4, 2>), grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores);
+    else if (eg <= 4) hipLaunchKernelGGL((gate_fwd_kernel<4, 4, 1>), grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores);
+    else if (eg <= 8) hipLaunchKernelGGL((gate_fwd_kernel<8, 4, 1>), grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores);
+    else hipLaunchKernelGGL((gate_fwd_kernel<16, 2, 1>), grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores);
     MOLE_LAUNCH_CHECK();
     return 0;
 }
