@@ -148,16 +148,25 @@ __global__ __launch_bounds__(RT_THREADS) void route_topk_kernel(
 __device__ __forceinline__ void scan_pair(int32_t *__restrict__ hist, int nb, int pair, int32_t *__restrict__ counts) {
     const int lane = threadIdx.x & 63;
     int carry = 0;
-    for (int c0 = 0; c0 < nb; c0 += WAVE) {
-        const int bi = c0 + lane;
-        const int v = bi < nb ? hist[(size_t)pair * nb + bi] : 0;
-        int x = v;
-        for (int d = 1; d < WAVE; d <<= 1) {
-            const int y = __shfl_up(x, d, WAVE);
-            if (lane >= d) x += y;
+    // four chunks of 64 blocks at a time: their loads are in flight together
+    for (int c0 = 0; c0 < nb; c0 += 4 * WAVE) {
+        int v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int bi = c0 + u * WAVE + lane;
+            v[u] = bi < nb ? hist[(size_t)pair * nb + bi] : 0;
         }
-        if (bi < nb) hist[(size_t)pair * nb + bi] = carry + x - v;
-        carry += __shfl(x, WAVE - 1, WAVE);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int bi = c0 + u * WAVE + lane;
+            int x = v[u];
+            for (int d = 1; d < WAVE; d <<= 1) {
+                const int y = __shfl_up(x, d, WAVE);
+                if (lane >= d) x += y;
+            }
+            if (bi < nb) hist[(size_t)pair * nb + bi] = carry + x - v[u];
+            carry += __shfl(x, WAVE - 1, WAVE);
+        }
     }
     if (lane == 0) counts[pair] = carry;
 }
@@ -185,6 +194,10 @@ __global__ __launch_bounds__(FIN_THREADS) void route_finish_kernel(
         __threadfence_block();
         __syncthreads();
     }
+    // only the first min(E, FIN_THREADS) threads hold data: the block-wide reductions and the scan below run over
+    // the next power of two, not over all 1024 threads (fewer barrier rounds for small gates)
+    int P = 1;
+    while (P < E && P < FIN_THREADS) P <<= 1;
     int lmax = 0;
     for (int e = tid; e < E; e += FIN_THREADS) {
         int tot = 0;
@@ -197,7 +210,7 @@ __global__ __launch_bounds__(FIN_THREADS) void route_finish_kernel(
     }
     s_red[tid] = lmax;
     __syncthreads();
-    for (int d = FIN_THREADS / 2; d >= 1; d >>= 1) {
+    for (int d = P / 2; d >= 1; d >>= 1) {
         if (tid < d) s_red[tid] = max(s_red[tid], s_red[tid + d]);
         __syncthreads();
     }
@@ -219,7 +232,7 @@ __global__ __launch_bounds__(FIN_THREADS) void route_finish_kernel(
     }
     s_red[tid] = csum;
     __syncthreads();
-    for (int d = 1; d < FIN_THREADS; d <<= 1) {
+    for (int d = 1; d < P; d <<= 1) {
         const int y = tid >= d ? s_red[tid - d] : 0;
         __syncthreads();
         s_red[tid] += y;
@@ -231,7 +244,7 @@ __global__ __launch_bounds__(FIN_THREADS) void route_finish_kernel(
             offsets[e] = run;
             run += s_n[e];
         }
-        if (tid == FIN_THREADS - 1) offsets[E] = s_red[tid];
+        if (tid == P - 1) offsets[E] = s_red[tid];
     } else {
         for (int e = lo; e < hi; ++e) offsets[e] = e * cap;
         if (tid == 0) offsets[E] = E * cap;
@@ -259,7 +272,7 @@ __global__ __launch_bounds__(FIN_THREADS) void route_finish_kernel(
         __syncthreads();
         s_fred[tid] = acc;
         __syncthreads();
-        for (int d = FIN_THREADS / 2; d >= 1; d >>= 1) {
+        for (int d = P / 2; d >= 1; d >>= 1) {
             if (tid < d) s_fred[tid] += s_fred[tid + d];
             __syncthreads();
         }
