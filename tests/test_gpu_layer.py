@@ -226,3 +226,54 @@ def test_layer_state_round_trip():
     assert m2.FC1_W_CPU.all_tensors.grad_.lazy_zero is False
     m2.set_hybrid_adam_count(3)
     assert m2.MOLECore.hybrid_adam_count == 3
+
+
+def _stack(n_layers, S, M, E, k, Fd, dtype, pool, ebatch, seed):
+    from mole_amd.moe.layer import MOLEModule
+    MOLEModule.reset_instances()
+    torch.manual_seed(seed)
+    dist = {"local_rank": 0, "world_size": 1, "rank": 0}
+    return [MOLEModule(E, 0, M, Fd, pool, k, ebatch, dist, "gelu", 1, False, True, dtype=dtype) for _ in range(n_layers)]
+
+
+def _run_stack(layers, x, prefetch):
+    from mole_amd.utils.Uscheduler import UniScheduler
+    xin = x.clone().requires_grad_(True)
+    if prefetch:
+        UniScheduler.prefetch_fwd()
+    h = xin
+    for m in layers:
+        h = m(h, capacity_factor=0.0, prefetch=prefetch)
+    h.backward(torch.ones_like(h) * 1e-2)
+    torch.cuda.synchronize()
+    from mole_amd import core
+    core.synchronize_tran()
+    grads = [t.grad_.clone() for m in layers for t in m.d_experts_param()]
+    return h.detach().clone(), xin.grad.clone(), grads
+
+
+@pytest.mark.parametrize("global_prefetch", [False, True])
+def test_stack_with_planned_prefetch_matches_plain_run(global_prefetch):
+    """Four offloaded layers share a pool smaller than two layers; the scheduler plans local and cross-layer
+    prefetches from (made-up) layer times.  Prefetching moves copies, never results: output, input gradient and
+    expert gradients equal the run without any prefetch bit for bit, and the prefetch stack ends empty."""
+    from mole_amd import core
+    from mole_amd.utils.Uscheduler import UniScheduler
+    S, M, E, k, Fd, dtype = 200, 64, 4, 2, 128, torch.float32
+    x = torch.randn(S, M, generator=torch.Generator().manual_seed(3)).cuda()
+    layers = _stack(4, S, M, E, k, Fd, dtype, pool=6, ebatch=2, seed=11)
+    want = _run_stack(layers, x, prefetch=False)
+    layers = _stack(4, S, M, E, k, Fd, dtype, pool=6, ebatch=2, seed=11)
+    plan = UniScheduler.set_prefetch_scheme(fwd_stat=[3.0, 1.0, 6.0, 2.0], bwd_stat=[2.0, 5.0, 0.0, 4.0], ftime=1.0,
+                                            global_prefetch=global_prefetch)
+    print("plan", plan, flush=True)
+    assert any(p["local_fwd"] or p["global_fwd"] for p in plan)
+    if global_prefetch:
+        assert any(p["global_fwd"] or p["global_bwd"] for p in plan)
+    for rep in range(2):                      # a second step starts from the state the first one left
+        got = _run_stack(layers, x, prefetch=True)
+        um = core.get_UniMem()
+        assert um.virtual_offset() == 0 and um.view_pool_size() == 6
+        assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+        for a, b in zip(got[2], want[2]):
+            assert torch.equal(a, b)
