@@ -590,22 +590,45 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
         // dependent loads (the scan itself re-reads rows_of through the cache)
         const int rows_lane = lane < nE ? rows_of(lane) : 0;
         const int off_lane = (!single && lane < nE) ? g.offsets[lane] : 0;
-        int n_mt = 0;
-        for (int ee = lane; ee < nE; ee += WAVE) n_mt += ((ee < WAVE ? rows_lane : rows_of(ee)) + Q_BM - 1) / Q_BM;
-        for (int d = WAVE / 2; d >= 1; d >>= 1) n_mt += __shfl_xor(n_mt, d, WAVE);
-        const int total = n_mt * n_tiles;
-        const int per_xcd = (total + 7) >> 3;
-        const int slot = blockIdx.x >> 3;
-        const int t = (blockIdx.x & 7) * per_xcd + slot;
-        if (slot >= per_xcd || t >= total) return;
-        const int target = t / n_tiles;        // index among all m-tiles
+        // An expert's m-tiles are heavy (more than half a tile of rows) or light: the full tiles and, of the
+        // remainder scheme, a remainder above half a tile; with the even split all tiles of an expert alike.
+        // Heavy tiles are numbered before light ones, each class in expert order and each XCD taking a contiguous
+        // range of either: an XCD hands out its blocks in order, so the long tiles start first and the short
+        // ones fill in behind them (skewed loads: otherwise a long tile that starts late ends the launch late).
+        // That order runs an expert's light tile long after its heavy ones, whose weight panels have left the L2 by
+        // then; with many rounds of tiles the order matters little and the re-read does, so beyond 16 rounds
+        // all tiles count as one class, in expert order.
+        bool split = true;
+        auto heavy_of = [&](int r) {
+            const int cnt = (r + Q_BM - 1) / Q_BM;
+            if (cnt == 0 || !split) return cnt;
+            if (TMB == 10) return ((((r + cnt - 1) / cnt) + 31) & ~31) > Q_BM / 2 ? cnt : 0;
+            return cnt - 1 + ((r - (cnt - 1) * Q_BM) > Q_BM / 2 ? 1 : 0);
+        };
+        int n_h = 0, n_l = 0;
+        for (int ee = lane; ee < nE; ee += WAVE) {
+            const int r = ee < WAVE ? rows_lane : rows_of(ee);
+            const int hv = heavy_of(r);
+            n_h += hv;
+            n_l += (r + Q_BM - 1) / Q_BM - hv;
+        }
+        for (int d = WAVE / 2; d >= 1; d >>= 1) { n_h += __shfl_xor(n_h, d, WAVE); n_l += __shfl_xor(n_l, d, WAVE); }
+        if ((n_h + n_l) * n_tiles > 16 * 256) { split = false; n_h += n_l; n_l = 0; }
+        const int total_h = n_h * n_tiles, total_l = n_l * n_tiles;
+        const int per_h = (total_h + 7) >> 3, per_l = (total_l + 7) >> 3;
+        const int slot = blockIdx.x >> 3, xcd = blockIdx.x & 7;
+        const bool heavy = slot < per_h;
+        const int t = heavy ? xcd * per_h + slot : xcd * per_l + (slot - per_h);
+        if (heavy ? t >= total_h : (slot - per_h >= per_l || t >= total_l)) return;
+        const int target = t / n_tiles;        // index among the m-tiles of the class
         nt = t % n_tiles;
-        // the expert whose running count passes `target`
+        // the expert whose running count (of the class) passes `target`
         int run = 0, found = -1, before = 0;
         for (int base = 0; base < nE && found < 0; base += WAVE) {
             const int ee = base + lane;
             const int r = base == 0 ? rows_lane : (ee < nE ? rows_of(ee) : 0);
-            const int cnt = (r + Q_BM - 1) / Q_BM;
+            const int hv = heavy_of(r);
+            const int cnt = heavy ? hv : (r + Q_BM - 1) / Q_BM - hv;
             int incl = cnt;
             for (int d = 1; d < WAVE; d <<= 1) {
                 const int y = __shfl_up(incl, d, WAVE);
@@ -622,7 +645,7 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
         if (found < 0) return;
         e = found;
         m_ext = found < WAVE ? __shfl(rows_lane, found, WAVE) : rows_of(e);
-        mt = target - before;
+        mt = target - before + (heavy ? 0 : heavy_of(m_ext));   // an expert's light tiles follow its heavy ones
         const int t_e = (m_ext + Q_BM - 1) / Q_BM;
         tile_h = TMB == 10 ? ((((m_ext + t_e - 1) / t_e) + 31) & ~31) : Q_BM;
         row0 = single ? 0 : (found < WAVE ? __shfl(off_lane, found, WAVE) : g.offsets[e]);
@@ -751,7 +774,8 @@ static int dispatch256(const GemmArgs &g, bool b_ks, bool wg, int epi, int max_r
     // block slots: the worst-case number of m-tiles (an expert with r rows has ceil(r / BM) of them)
     const int rows_bound = g.offsets ? max_rows : g.single_rows;
     GemmArgs gg = g;
-    const int tiles = ((rows_bound / BM + (g.offsets ? g.E : 1)) * n_tiles + 7) & ~7;
+    // (+ 16: the heavy and the light tiles of an XCD are rounded up to whole slots separately)
+    const int tiles = (((rows_bound / BM + (g.offsets ? g.E : 1)) * n_tiles + 7) & ~7) + 16;
     if (wg) return -100;
     if (!b_ks) {
         if (epi == EPI_DGELU) return launch256<TMB, WM, false, false, EPI_DGELU>(gg, tiles, st, kid);

@@ -52,6 +52,8 @@ CASES = [
     (150, 64, 256, [(7 * e) % 23 if e % 3 else 0 for e in range(149)] + [700], 0),
     # an expert with more rows than four 320-row tiles, and column counts that are not whole tiles
     (3, 264, 520, [1500, 3, 321], 5),
+    # more than 16 rounds of tiles (the grouped kernel then numbers them in plain expert order)
+    (150, 64, 4096, [257 + (11 * e) % 90 for e in range(150)], 0),
 ]
 
 
