@@ -52,7 +52,6 @@ struct GemmArgs {
     int accumulate;         // EPI_WGRAD: add into C
     int gelu_bwd;           // EPI_DGELU: MOLE_GELU_BWD_*
     int n_blocks;           // real number of tiles in the launch (grid is rounded up to 8)
-    int full_blocks;        // 256-wide kernel, row-ragged: block slots reserved for full m-tiles
     void *colsum;           // weight gradients, 256-wide kernel: [E][M] (side 1) or [E][N] (side 2) sums of an operand
     int colsum_side;        //   over the expert's rows: 1 = the m-side operand (A), 2 = the n-side operand (B)
 };

@@ -594,7 +594,7 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
         // remainder scheme, a remainder above half a tile; with the even split all tiles of an expert alike.
         // Heavy tiles are numbered before light ones, each class in expert order and each XCD taking a contiguous
         // range of either: an XCD hands out its blocks in order, so the long tiles start first and the short
-        // ones fill in behind them (skewed loads: otherwise a long tile that starts late ends the launch late).
+        // ones fill in behind them (otherwise a long tile that starts late ends the launch late).
         // That order runs an expert's light tile long after its heavy ones, whose weight panels have left the L2 by
         // then; with many rounds of tiles the order matters little and the re-read does, so beyond 16 rounds
         // all tiles count as one class, in expert order.
@@ -778,8 +778,8 @@ static int dispatch256(const GemmArgs &g, bool b_ks, bool wg, int epi, int max_r
     const int tiles = (((rows_bound / BM + (g.offsets ? g.E : 1)) * n_tiles + 7) & ~7) + 16;
     if (wg) return -100;
     if (!b_ks) {
-        if (epi == EPI_DGELU) return launch256<TMB, WM, false, false, EPI_DGELU>(gg, tiles, st, kid);
         if constexpr (TMB != 10) {
+            if (epi == EPI_DGELU) return launch256<TMB, WM, false, false, EPI_DGELU>(gg, tiles, st, kid);
             if (epi == EPI_BIAS_GELU) return launch256<TMB, WM, false, false, EPI_BIAS_GELU>(gg, tiles, st, kid);
             if (epi == EPI_F32) return launch256<TMB, WM, false, false, EPI_F32>(gg, tiles, st, kid);
         }
@@ -791,19 +791,21 @@ static int dispatch256(const GemmArgs &g, bool b_ks, bool wg, int epi, int max_r
 }
 
 // Tile configuration.  Eight waves (two per SIMD hide each other's waits; one fetch of the n-side tile
-// serves all rows of the tile) for every product.  256-row tiles by default; tiles of up to 320 rows for
-// the three products whose register budget allows 160 accumulators a wave (out = a.w2 + b2, gx = t.w1 and
-// t = (go.w2^T) gelu'(h)): with a capacity factor of 1.25 an expert then never needs more m-tiles than
-// the average one, and the launch stays one round of tiles.  h = xd.w1^T + b1 with the GELU epilogue
-// spills at 160 accumulators and stays at 256 rows.  MOLE_TMB=4|8 in the environment selects the
-// four-wave variants with 128 or 256 rows, 16 the 256-row eight-wave tile for everything (tuning aid).
+// serves all rows of the tile) for every product.  256-row tiles by default; tiles of up to 320 rows, an
+// expert's rows split evenly over them, for the two K = F products (out = a.w2 + b2 and gx = t.w1): one tile
+// is a whole round there, and with a capacity factor of 1.25 no expert then needs more m-tiles than the
+// average one, so the launch stays one round.  The K = M products run four rounds anyway; their short
+// remainder tiles, numbered last, fill the final round, which measured better than the even split
+// (t = (go.w2^T) gelu'(h): 213 against 219 us) - and h = xd.w1^T + b1 with the GELU epilogue would spill at
+// the 160 accumulators of the larger tile.  MOLE_TMB=4|8 in the environment selects the four-wave variants
+// with 128 or 256 rows, 16 the 256-row eight-wave tile for everything (tuning aid).
 static int tile_blocks_for(int kid) {
     static const int forced = [] {
         const char *v = getenv("MOLE_TMB");
         return v ? atoi(v) : 0;
     }();
     if (forced == 4 || forced == 8 || forced == 16) return forced;
-    return (kid == MOLE_K_FFN_FWD2 || kid == MOLE_K_FFN_GX || kid == MOLE_K_FFN_DA) ? 20 : 16;
+    return (kid == MOLE_K_FFN_FWD2 || kid == MOLE_K_FFN_GX) ? 20 : 16;
 }
 
 // Whether the weight-gradient launch for g will also produce the operand sums asked for in g.colsum
@@ -824,7 +826,7 @@ int launch_gemm256(const GemmArgs &g, bool a_ks, bool b_ks, bool wg, int epi, in
     const int tmb = tile_blocks_for(kid);
     if (tmb == 4) return dispatch256<4, 1>(g, b_ks, wg, epi, max_rows, st, kid);
     if (tmb == 16) return dispatch256<8, 2>(g, b_ks, wg, epi, max_rows, st, kid);   // 256 rows, eight waves
-    if (tmb == 20 && !wg && (b_ks || epi == EPI_DGELU)) return dispatch256<10, 2>(g, b_ks, wg, epi, max_rows, st, kid);   // up to 320 rows, eight waves
+    if (tmb == 20 && !wg && b_ks) return dispatch256<10, 2>(g, b_ks, wg, epi, max_rows, st, kid);   // up to 320 rows, eight waves
     if (tmb == 20) return dispatch256<8, 2>(g, b_ks, wg, epi, max_rows, st, kid);
     return dispatch256<8, 1>(g, b_ks, wg, epi, max_rows, st, kid);
 }
