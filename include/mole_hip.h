@@ -95,8 +95,11 @@ int mole_gate_fwd(const void *x, int dtype, const float *wg, const float *logit_
 int mole_gate_bwd(const float *dgates, const float *scores, const int32_t *idx, int S, int E,
                   int k, int normalize_gate, int through_softmax, float *dout, mole_stream_t stream);
 /* Gradient of the gate's Linear (MOLE/utils/Ugate.py:12, run by autograd in the reference):
- * dwg[E,M] = dlogits[S,E]^T . x[S,M], fp32, summed in a fixed order.  1 <= E <= 32; larger gates use
- * a library GEMM.  workspace of mole_gate_wgrad_workspace_bytes(S, E, M) bytes. */
+ * dwg[E,M] = dlogits[S,E]^T . x[S,M], fp32, summed in a fixed order (partial sums per chunk of tokens in the
+ * workspace, then a reduction).  bf16 tokens: E <= 256 and M a multiple of 64 on the matrix cores (dlogits
+ * enters as the sum of two bf16 numbers, so the result keeps fp32-level accuracy); either dtype: E <= 32 and
+ * M a multiple of 4 on the VALU.  Other shapes are rejected (a library GEMM serves them on the host side).
+ * workspace of mole_gate_wgrad_workspace_bytes(S, E, M) bytes. */
 size_t mole_gate_wgrad_workspace_bytes(int S, int E, int M);
 int mole_gate_wgrad(const float *dlogits, const void *x, int dtype, int S, int E, int M, float *dwg,
                     void *workspace, size_t workspace_bytes, mole_stream_t stream);

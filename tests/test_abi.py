@@ -56,3 +56,49 @@ def test_product_package_does_not_import_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".cpp")):
                 src = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in src.replace("the oracle", ""), f"{f} mentions the oracle package"
+
+
+def test_every_entry_point_rejects_bad_arguments_on_the_host():
+    """Shape, dtype, alignment and null checks come before any launch: each call below returns a negative library
+    code and leaves a message that names the entry point, on a machine without a GPU."""
+    import ctypes
+    from mole_amd import _lib as L
+    lib = L.lib()
+    P = ctypes.c_void_p
+    bad16 = P(8)        # a non-null, misaligned "pointer" that is never dereferenced
+    ok = P(4096)
+    cases = [
+        ("mole_softmax_fwd", lambda: lib.mole_softmax_fwd(None, None, 10, 0, None, None)),
+        ("mole_gate_fwd", lambda: lib.mole_gate_fwd(ok, L.MOLE_F32, ok, None, 10, 8, 128, ok, None)),
+        ("mole_gate_fwd", lambda: lib.mole_gate_fwd(ok, L.MOLE_BF16, ok, None, 10, 8, 100, ok, None)),
+        ("mole_gate_bwd", lambda: lib.mole_gate_bwd(ok, ok, ok, 10, 4, 5, 1, 1, ok, None)),
+        ("mole_gate_wgrad", lambda: lib.mole_gate_wgrad(ok, ok, L.MOLE_F32, 10, 64, 128, ok, ok, 1 << 30, None)),
+        ("mole_gate_wgrad", lambda: lib.mole_gate_wgrad(ok, ok, L.MOLE_BF16, 10, 8, 128, ok, ok, 16, None)),
+        ("mole_route", lambda: lib.mole_route(ok, 10, 4, 5, 1.0, 1, 1, 1, ok, ok, ok, ok, ok, ok, ok, ok, ok, ok, 1 << 20, None)),
+        ("mole_route", lambda: lib.mole_route(ok, 10, 4, 2, 1.0, 1, 1, 1, ok, ok, ok, ok, ok, ok, ok, ok, ok, ok, 8, None)),
+        ("mole_dispatch_fwd", lambda: lib.mole_dispatch_fwd(bad16, L.MOLE_F32, ok, 8, 16, 2, ok, None)),
+        ("mole_dispatch_bwd", lambda: lib.mole_dispatch_bwd(ok, L.MOLE_F32, ok, 8, 16, 2, ok, None, 4, None, ok, None)),
+        ("mole_combine_fwd", lambda: lib.mole_combine_fwd(ok, L.MOLE_BF16, ok, ok, 8, 12, 2, ok, None)),
+        ("mole_combine_bwd", lambda: lib.mole_combine_bwd(None, ok, L.MOLE_F32, ok, ok, 8, 16, 2, ok, ok, None)),
+        ("mole_zero_pad_rows", lambda: lib.mole_zero_pad_rows(ok, 9, ok, ok, 4, 16, None)),
+        ("mole_ffn_fwd", lambda: lib.mole_ffn_fwd(ok, L.MOLE_BF16, ok, ok, 2, 16, 12, 16, ok, ok, ok, ok, ok, ok, ok, None)),
+        ("mole_ffn_fwd", lambda: lib.mole_ffn_fwd(bad16, L.MOLE_F32, ok, ok, 2, 16, 16, 16, ok, ok, ok, ok, ok, ok, ok, None)),
+        ("mole_ffn_bwd", lambda: lib.mole_ffn_bwd(ok, ok, ok, ok, 5, ok, ok, 2, 16, 16, 16, ok, ok, ok, ok, ok, ok, ok, ok, 0, 0, None)),
+        ("mole_gemm_nt", lambda: lib.mole_gemm_nt(ok, ok, 4, 16, 16, 16, ok, None)),
+        ("mole_gemm_nn", lambda: lib.mole_gemm_nn(ok, ok, 4, 16, 16, 16, ok, None)),
+        ("mole_adam_step", lambda: lib.mole_adam_step(ok, ok, ok, ok, ok, 64, L.MOLE_F32, 0.9, 0.999, 0, 1e-3, 0.0, 1e-8, 0, None)),
+        ("mole_adam_step", lambda: lib.mole_adam_step(ok, bad16, ok, ok, ok, 64, L.MOLE_BF16, 0.9, 0.999, 1, 1e-3, 0.0, 1e-8, 0, None)),
+        ("mole_adam_step", lambda: lib.mole_adam_step(ok, ok, ok, ok, ok, 64, L.MOLE_F32, 1.0, 0.999, 1, 1e-3, 0.0, 1e-8, 0, None)),
+        ("mole_unimem_prefetch", lambda: lib.mole_unimem_prefetch(None, 0, None, 0, 1)),
+        ("mole_unimem_fetch", lambda: lib.mole_unimem_fetch(None, None, 0, 0, 1, 0, None)),
+        ("mole_unimem_store_grads", lambda: lib.mole_unimem_store_grads(None, None, None, 0, 1, None)),
+        ("mole_unimem_load_state", lambda: lib.mole_unimem_load_state(None, None, None, None, 1, 0, None)),
+        ("mole_unimem_store_state", lambda: lib.mole_unimem_store_state(None, None, None, None, 1, None)),
+        ("mole_unimem_sync_tran", lambda: lib.mole_unimem_sync_tran(None)),
+        ("mole_fast_assign_prefetch", lambda: lib.mole_fast_assign_prefetch(4, None, None, 3, None, None, 0, None)),
+    ]
+    for name, call in cases:
+        rc = call()
+        assert rc < 0, f"{name}: expected a library error code, got {rc}"
+        msg = L.last_error()
+        assert name in msg, f"{name}: message does not name the entry point: {msg!r}"
