@@ -139,3 +139,47 @@ def test_ffn_random_shapes_bf16(seed):
     else:   # no rows at all: every gradient is exactly zero
         for gt in (g_w1, g_b1, g_w2, g_b2):
             assert float(gt.float().abs().max()) == 0.0
+
+
+def test_ffn_benchmark_size_against_fp32_products():
+    """The benchmark's own shape (16 experts of 1024 -> 4096 -> 1024 in bf16, 16384 rows at uneven loads up to the
+    capacity of 1280): forward and backward of three experts against fp32 torch products of the same rounded
+    operands on the GPU (the CPU oracle would take minutes at this size), plus bias gradients of all experts."""
+    from mole_amd import hip_ops as H, _lib as L
+    E, M, Fd = 16, 1024, 4096
+    g = torch.Generator().manual_seed(5)
+    loads = torch.clamp((torch.randn(E, generator=g) * 120 + 1024).int(), min=1, max=1280)
+    off = torch.zeros(E + 1, dtype=torch.int32)
+    off[1:] = torch.cumsum(loads, 0)
+    R = int(off[-1])
+    print(f"ffn benchmark size: loads {loads.tolist()} R={R}", flush=True)
+    dev, dt = "cuda", torch.bfloat16
+    gd = torch.Generator(device=dev).manual_seed(6)
+    rnd = lambda *s, sc=1.0: (torch.randn(*s, generator=gd, device=dev) * sc).to(dt)
+    xd, go = rnd(R, M), rnd(R, M, sc=0.02)
+    w1, b1, w2, b2 = rnd(E, Fd, M, sc=0.03), rnd(E, Fd, sc=0.03), rnd(E, Fd, M, sc=0.03), rnd(E, M, sc=0.03)
+    offd, nd = off.cuda(), loads.int().cuda()
+    out, h, a = H.ffn_fwd(xd, offd, nd, w1, b1, w2, b2)
+    g_w1, g_b1, g_w2, g_b2 = torch.empty_like(w1), torch.empty_like(b1), torch.empty_like(w2), torch.empty_like(b2)
+    gx = H.ffn_bwd(go, xd, h, a, offd, nd, w1, w2, g_w1, g_b1, g_w2, g_b2, True, False, L.GELU_BWD_EXACT)
+    torch.cuda.synchronize()
+    t = tol(dt)
+    for e in (0, 7, 15):
+        lo, hi = int(off[e]), int(off[e + 1])
+        x32, go32 = xd[lo:hi].float(), go[lo:hi].float()
+        h32 = x32 @ w1[e].float().t() + b1[e].float()
+        a32 = torch.nn.functional.gelu(h32)
+        o32 = a32 @ w2[e].float() + b2[e].float()
+        assert rel_err(h[lo:hi], h32) < t and rel_err(a[lo:hi], a32) < t and rel_err(out[lo:hi], o32) < t
+        # backward from the kernel's own (bf16) h, as the kernel sees it
+        hs = h[lo:hi].float()
+        hs.requires_grad_(True)
+        torch.nn.functional.gelu(hs).backward(go32 @ w2[e].float().t())
+        t32 = hs.grad
+        assert rel_err(g_w2[e], a[lo:hi].float().t() @ go32) < t
+        assert rel_err(g_w1[e], t32.t() @ x32) < t
+        assert rel_err(gx[lo:hi], t32 @ w1[e].float()) < t
+        assert rel_err(g_b1[e], t32.sum(0)) < t
+    # bias gradient of the second linear for every expert: plain column sums of go
+    want_b2 = torch.stack([go[int(off[e]):int(off[e + 1])].float().sum(0) for e in range(E)])
+    assert rel_err(g_b2, want_b2) < t
