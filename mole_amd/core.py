@@ -158,8 +158,8 @@ class UniMem:
         L.check(L.lib().mole_unimem_copy_stats(self._h, ctypes.byref(b), ctypes.byref(ms)), "mole_unimem_copy_stats")
         return b.value, ms.value
 
-    def slot_tensor(self, p_id: int, slot: int, n: int) -> torch.Tensor:
-        """Device pointer of `slot` for parameter kind p_id (debug / tests)."""
+    def slot_tensor(self, p_id: int, slot: int, n: int) -> int:
+        """Device address of `slot` for parameter kind p_id (debug / tests)."""
         out = c_void_p()
         L.check(L.lib().mole_unimem_slot_ptr(self._h, p_id, slot, ctypes.byref(out)), "mole_unimem_slot_ptr")
         return int(out.value)
@@ -412,12 +412,22 @@ class MOLECore:
         """Gradients of offloaded experts go back to their pinned host buffers (core.cpp:77-103,
         uparameter.cpp:68-83): overwrite, or add when accumulating and the buffer is not lazily zero."""
         if self.acc_step > 1 and not getattr(host_grads[0], "lazy_zero", True):
-            get_UniMem().sync_tran()      # an earlier step's overwrite may still be in flight
-            for hg, gg in zip(host_grads, g):
-                hg[base:base + size] += gg.to("cpu")
+            self._add_to_host([hg[base:base + size] for hg in host_grads], g)
         else:
             get_UniMem().store_grads(host_grads, g, base, size)
 
+    @staticmethod
+    def _add_to_host(host_slices, g):
+        """host_slices += g without stopping the host: the sums of the earlier micro-steps come up on the copy
+        stream (after any write-back into them still in flight), are added on the GPU and go back on the
+        write-back stream.  The reference adds on the CPU after a blocking copy (data_transfer.cpp:9-12); the
+        sum is the same single rounding of the same two operands."""
+        um = get_UniMem()
+        prev = [torch.empty_like(gg) for gg in g]
+        um.load_state(prev, host_slices, after_writeback=True)
+        for gg, pp in zip(g, prev):
+            gg += pp
+        um.store_state(host_slices, g)
 
     def _instant_adam(self, p_slots, g, base, size):
         """Adam on the GPU for experts [base, base+size) of the offloaded set, inside the backward pipeline
@@ -436,9 +446,7 @@ class MOLECore:
         if n < size:          # experts beyond the GPU-updated prefix: gradients only
             rest = [gg[n:] for gg in g]
             if self.acc_step > 1 and not getattr(host_grads[0], "lazy_zero", True):
-                um.sync_tran()
-                for hg, gg in zip(host_grads, rest):
-                    hg[base + n:base + size] += gg.to("cpu")
+                self._add_to_host([hg[base + n:base + size] for hg in host_grads], rest)
             else:
                 um.store_state([hg[base + n:base + size] for hg in host_grads], rest)
         if n == 0:

@@ -198,6 +198,44 @@ def test_layer_degenerate_inputs():
         assert res.crit.capacity == 0 and float(res.y.abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gradient_accumulation_over_micro_steps(dtype):
+    """acc_step = 3 with two GPU-resident and four offloaded experts: after three backward passes of the same
+    batch the gradient buffers hold g + g + g, summed in the parameter dtype in that order (static experts
+    accumulate in the weight-gradient epilogue, core.cpp:457-514; offloaded ones into their pinned host arrays,
+    core.cpp:77-103) - the first pass overwrites whatever the buffers held (lazy zero)."""
+    from mole_amd import core
+    S, M, E, k, Fd, d = 300, 64, 6, 2, 128, 4
+    print(f"gradient accumulation {dtype}", flush=True)
+
+    def step(m, x):
+        xin = x.clone().requires_grad_(True)
+        y = m(xin, capacity_factor=0.0)
+        y.backward((2.0 * y.detach().float() / y.numel()).to(dtype) * 50.0)
+        torch.cuda.synchronize()
+
+    m0, x, _ = _build(S, M, E, k, Fd, dtype, d_experts=d, pool=4, ebatch=2, seed=3)
+    step(m0, x)
+    core.synchronize_tran()
+    single = [g.clone() for g in _grads(m0, E)]
+    assert all(float(g.abs().max()) > 0 for g in single)
+
+    m1, x1, _ = _build(S, M, E, k, Fd, dtype, d_experts=d, pool=4, ebatch=2, seed=3, acc_step=3)
+    for cp in (m1.FC1_W_CPU, m1.FC1_B_CPU, m1.FC2_W_CPU, m1.FC2_B_CPU):
+        cp.all_tensors.grad_.fill_(7.0)          # stale contents that the first micro-step must overwrite
+    for _ in range(3):
+        step(m1, x1)
+    core.synchronize_tran()
+    s = E - d
+    for name, g1, g3 in zip(("g_w1", "g_b1", "g_w2", "g_b2"), single, _grads(m1, E)):
+        g = g1.to(dtype)
+        want = ((g + g) + g).float()
+        # offloaded experts: one rounding per addition, exactly reproducible
+        assert torch.equal(g3[s:], want[s:]), f"{name} of the offloaded experts"
+        # GPU-resident experts accumulate inside the product's epilogue (fp32 sum, rounded once per pass)
+        assert rel_err(g3[:s], 3.0 * g1[:s]) < (1e-6 if dtype == torch.float32 else 1e-2), f"{name} of the resident experts"
+
+
 def test_layer_state_round_trip():
     """get_layer_state / set_layer_state (the reference's checkpoint payload, layer.py:350-427): a second layer
     loaded from the first one's state computes the same output and holds the same gradients."""
