@@ -71,7 +71,10 @@ enum {
     MOLE_K_ROUTE = 11,    /* the four routing kernels together */
     MOLE_K_GEMM_NT = 12,
     MOLE_K_ADAM = 13,
-    MOLE_K_COUNT = 14
+    MOLE_K_GATE_FWD = 14,   /* gate logits + softmax in one kernel, or the softmax kernel alone */
+    MOLE_K_GATE_BWD = 15,   /* dgates -> dlogits */
+    MOLE_K_GATE_WGRAD = 16, /* dWg: partial sums + their reduction */
+    MOLE_K_COUNT = 17
 };
 int mole_kernel_timing_enable(int on);
 int mole_kernel_timing_read(int n_ids, int *counts, float *ms_total);

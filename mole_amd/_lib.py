@@ -19,7 +19,7 @@ LAYOUT_PADDED, LAYOUT_RAGGED = 0, 1
 GELU_BWD_TANH, GELU_BWD_EXACT = 0, 1
 MAX_TOPK, MAX_EXPERTS = 16, 1024
 KERNEL_IDS = ("ffn_fwd1", "ffn_fwd2", "ffn_gw2", "ffn_da", "ffn_gw1", "ffn_gx", "ffn_gb", "dispatch_fwd", "dispatch_bwd",
-              "combine_fwd", "combine_bwd", "route", "gemm_nt", "adam")
+              "combine_fwd", "combine_bwd", "route", "gemm_nt", "adam", "gate_fwd", "gate_bwd", "gate_wgrad")
 
 _P = c_void_p
 _SIGNATURES = {

@@ -412,27 +412,36 @@ __global__ __launch_bounds__(256) void gate_wgrad_partial_kernel(const float *__
 // multiplied separately, so the result stays as close to the exact sum as the fp32 accumulation allows.
 // A block of four waves takes one chunk of tokens, 256 columns (64 per wave) and up to 64 experts (grid z walks
 // the rest).  The contraction runs over tokens, along which neither operand is contiguous in memory, so both
-// are turned in LDS: the chunk's dlogits, 128 tokens at a time, into [expert][token] bf16 rows (an A fragment is
-// then one 16-byte read), x 32 tokens at a time per wave as it lies in memory, read back with the transposing
-// ds_read_b64_tr_b16 (a group of 16 lanes receives a 4-token x 16-column block column by column).  The next
-// 32 tokens' global loads are in flight while the current ones are multiplied.
+// are turned in LDS: they are staged as they lie in memory, [token][expert] for the chunk's dlogits (128 tokens
+// at a time, shared by the block) and [token][column] for x (32 tokens at a time per wave), and read back with
+// the transposing ds_read_b64_tr_b16 (a group of 16 lanes receives a 4-token x 16-column block column by column).  The next
+// 128 tokens' rows of x and dlogits are in flight while the current ones are multiplied.
 constexpr int GM_KSTEP = 32;                  // tokens per MFMA
 constexpr int GM_XROW = 72;                   // bf16 per token row of a wave's x tile: 64 columns + 16 bytes,
                                               // so that the 4 rows of a transposing read fall into distinct banks
 constexpr int GM_SUB = 128;                   // tokens whose dlogits are staged at a time
-constexpr int GM_DLROW = GM_SUB + 8;          // bf16 per expert row of the staged dlogits (+ 16 bytes: bank spread)
 typedef short perm_s16x4 __attribute__((ext_vector_type(4)));
 template <int EG>   // groups of 16 experts per block
-__global__ __launch_bounds__(256) void gate_wgrad_mfma_kernel(const float *__restrict__ dlogits,
+__global__ __launch_bounds__(256, 2) void gate_wgrad_mfma_kernel(const float *__restrict__ dlogits,
                                                               const bf16_t *__restrict__ x, int S, int E, int M,
-                                                              int chunk, float *__restrict__ part) {
-    __shared__ __align__(16) bf16_t s_dl[2][16 * EG * GM_DLROW];     // leading and remainder halves of dlogits
+                                                              int chunk, int nchunks, int nz, float *__restrict__ part) {
+    // staged dlogits, [token][expert] like x: rounded values and rounded remainders.  Row length: the group's
+    // experts + padding that puts the 4 token rows of a transposing read into distinct banks
+    constexpr int DLROW = 16 * EG + (EG == 2 ? 16 : 8);
+    __shared__ __align__(16) bf16_t s_dl[2][GM_SUB * DLROW];
     __shared__ __align__(16) bf16_t s_x[4 * GM_KSTEP * GM_XROW];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r16 = lane & 15, kq = lane >> 4;
-    const int tok0 = blockIdx.x * chunk, ntok = min(chunk, S - tok0);
-    const int e0 = blockIdx.z * 16 * EG;
-    const int col0 = blockIdx.y * 256 + wave * 64;
+    // block -> (chunk, column block, expert group).  Blocks go round-robin to the 8 XCDs; the nz expert groups of
+    // one (chunk, column block) unit take consecutive slots of one XCD, so the unit's x tile comes out of that
+    // XCD's L2 for all but the first of them.
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int unit = (slot / nz) * 8 + xcd, zi = slot % nz;
+    if (unit >= nchunks * ((M + 255) / 256)) return;     // padding blocks of the last round of units
+    const int ci = unit % nchunks, yi = unit / nchunks;
+    const int tok0 = ci * chunk, ntok = min(chunk, S - tok0);
+    const int e0 = zi * 16 * EG;
+    const int col0 = yi * 256 + wave * 64;
     const bool active = col0 < M;             // M is a multiple of 64: a wave is in or out as a whole
     bf16_t *xt = s_x + wave * (GM_KSTEP * GM_XROW);
     perm_f32x4 acc[EG][4];
@@ -441,63 +450,92 @@ __global__ __launch_bounds__(256) void gate_wgrad_mfma_kernel(const float *__res
 #pragma unroll
         for (int cb = 0; cb < 4; ++cb) acc[g][cb] = perm_f32x4{0.f, 0.f, 0.f, 0.f};
     // a wave's x tile of one step: 32 tokens x 64 columns = 4 loads of 16 bytes per lane (token 8 i + lane / 8)
+    // Every load is issued unconditionally from a clamped, valid address, and what lies past the chunk is
+    // replaced by zero only where the value is used, a sub-chunk later: a load under a branch, or one whose
+    // value is touched right away, makes the compiler wait for all outstanding loads, which undoes the prefetch.
     const int lt = lane >> 3, lc = (lane & 7) * 8;
+    const bf16_t *xcol = x + (active ? col0 : 0) + lc;
     auto fetch = [&](uint4 (&v)[4], int k0) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int t = k0 + 8 * i + lt;
-            v[i] = (active && t < ntok) ? *reinterpret_cast<const uint4 *>(x + (size_t)(tok0 + t) * M + col0 + lc)
-                                        : make_uint4(0, 0, 0, 0);
+            v[i] = *reinterpret_cast<const uint4 *>(xcol + (size_t)(tok0 + min(t, ntok - 1)) * M);
         }
     };
-    uint4 cur[4], nxt[4];
-    fetch(cur, 0);
+    // a thread's share of the dlogits of GM_SUB tokens: expert de of the block's group (expert fastest across
+    // threads: the global reads are whole rows of dlogits), tokens dt0, dt0 + DL_TSTEP, ...; fetched into
+    // registers one sub-chunk ahead, so the loads are in flight while the current sub-chunk is multiplied
+    constexpr int DL_W = 16 * EG, DL_N = GM_SUB * DL_W / 256, DL_TSTEP = 256 / DL_W;
+    const int de = threadIdx.x % DL_W, dt0 = threadIdx.x / DL_W;
+    float dl[DL_N];
+    const bool dl_in = e0 + de < E;
+    const float *dl_col = dlogits + min(e0 + de, E - 1);
+    auto fetch_dl = [&](int sub0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < DL_N; ++i) {
+            const int t = sub0 + dt0 + DL_TSTEP * i;
+            dl[i] = dl_col[(size_t)(tok0 + min(t, ntok - 1)) * E];
+        }
+    };
+    // the x tiles of a whole sub-chunk (GM_SUB / GM_KSTEP = 4 steps) are in flight at any time: a step's
+    // registers are refilled with the same step of the next sub-chunk as soon as its tile is in LDS
+    constexpr int NQ = GM_SUB / GM_KSTEP;
+    uint4 q[NQ][4];
+#pragma unroll
+    for (int i = 0; i < NQ; ++i) fetch(q[i], GM_KSTEP * i);
+    fetch_dl(0);
     for (int sub0 = 0; sub0 < ntok; sub0 += GM_SUB) {
-        // dlogits of the next GM_SUB tokens -> LDS, transposed and rounded (expert fastest across threads: the
-        // global reads are whole rows of dlogits)
+        // this sub-chunk's dlogits -> LDS, transposed and split into rounded value and rounded remainder
         __syncthreads();
-        for (int idx = threadIdx.x; idx < 16 * EG * GM_SUB; idx += 256) {
-            const int e = idx % (16 * EG), t = idx / (16 * EG);
-            const float v = (sub0 + t < ntok && e0 + e < E) ? dlogits[(size_t)(tok0 + sub0 + t) * E + e0 + e] : 0.f;
+#pragma unroll
+        for (int i = 0; i < DL_N; ++i) {
+            const int t = dt0 + DL_TSTEP * i;
+            const float v = (sub0 + t < ntok && dl_in) ? dl[i] : 0.f;
             const bf16_t hi = (bf16_t)v;
-            s_dl[0][e * GM_DLROW + t] = hi;
-            s_dl[1][e * GM_DLROW + t] = (bf16_t)(v - (float)hi);
+            s_dl[0][t * DLROW + de] = hi;
+            s_dl[1][t * DLROW + de] = (bf16_t)(v - (float)hi);
         }
         __syncthreads();
-        const int sub_end = min(ntok, sub0 + GM_SUB);
-        for (int k0 = sub0; k0 < sub_end; k0 += GM_KSTEP) {
-            fetch(nxt, k0 + GM_KSTEP);        // past the chunk's end: zeros, no loads
+        fetch_dl(sub0 + GM_SUB);              // past the chunk's end: zeros
 #pragma unroll
-            for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4 *>(xt + (8 * i + lt) * GM_XROW + lc) = cur[i];
+        for (int qi = 0; qi < NQ; ++qi) {       // steps past the chunk's end multiply zeros
+            const int k0 = sub0 + GM_KSTEP * qi;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                *reinterpret_cast<uint4 *>(xt + (8 * i + lt) * GM_XROW + lc) =
+                    k0 + 8 * i + lt < ntok ? q[qi][i] : make_uint4(0, 0, 0, 0);
             // (the tile is written and read by this wave only: program order is enough)
+            fetch(q[qi], k0 + GM_SUB);        // past the chunk's end: zeros
+            // a fragment by two transposing reads: 4 + 4 tokens from 8 kq + (r16 >> 2) on, 16 columns from col on,
+            // 4 (r16 & 3) .. per lane; lane r16 receives column col + r16 of the 8 tokens 8 kq ..
+            auto frag = [&](const bf16_t *tile, int row_len, int col) __attribute__((always_inline)) {
+                const bf16_t *p = tile + (8 * kq + (r16 >> 2)) * row_len + col + 4 * (r16 & 3);
+                const perm_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((perm_s16x4 __attribute__((address_space(3))) *)(p));
+                const perm_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((perm_s16x4 __attribute__((address_space(3))) *)(p + 4 * row_len));
+                typedef short s16x8 __attribute__((ext_vector_type(8)));
+                const s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                return __builtin_bit_cast(perm_bf16x8, v);
+            };
             perm_bf16x8 a[EG], al[EG];
 #pragma unroll
             for (int g = 0; g < EG; ++g) {
-                a[g] = *reinterpret_cast<const perm_bf16x8 *>(s_dl[0] + (16 * g + r16) * GM_DLROW + (k0 - sub0) + 8 * kq);
-                al[g] = *reinterpret_cast<const perm_bf16x8 *>(s_dl[1] + (16 * g + r16) * GM_DLROW + (k0 - sub0) + 8 * kq);
+                a[g] = frag(s_dl[0] + (k0 - sub0) * DLROW, DLROW, 16 * g);
+                al[g] = frag(s_dl[1] + (k0 - sub0) * DLROW, DLROW, 16 * g);
             }
 #pragma unroll
             for (int cb = 0; cb < 4; ++cb) {
-                // tokens 8 kq + (r16 >> 2) (+ 4), columns 16 cb + 4 (r16 & 3) ..: lane r16 receives column 16 cb + r16
-                const bf16_t *p = xt + (8 * kq + (r16 >> 2)) * GM_XROW + 16 * cb + 4 * (r16 & 3);
-                const perm_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((perm_s16x4 __attribute__((address_space(3))) *)(p));
-                const perm_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((perm_s16x4 __attribute__((address_space(3))) *)(p + 4 * GM_XROW));
-                typedef short s16x8 __attribute__((ext_vector_type(8)));
-                const s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                const perm_bf16x8 b = __builtin_bit_cast(perm_bf16x8, v);
+                const perm_bf16x8 b = frag(xt, GM_XROW, 16 * cb);
 #pragma unroll
                 for (int g = 0; g < EG; ++g) {
                     acc[g][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(al[g], b, acc[g][cb], 0, 0, 0);
                     acc[g][cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[g], b, acc[g][cb], 0, 0, 0);
                 }
             }
-#pragma unroll
-            for (int i = 0; i < 4; ++i) cur[i] = nxt[i];
         }
     }
     if (!active) return;
     // acc[g][cb][r] = expert e0 + 16 g + 4 kq + r, column col0 + 16 cb + r16
-    float *out = part + (size_t)blockIdx.x * E * M;
+    float *out = part + (size_t)ci * E * M;
 #pragma unroll
     for (int g = 0; g < EG; ++g)
 #pragma unroll
@@ -729,6 +767,7 @@ extern "C" int mole_gate_wgrad(const float *dlogits, const void *x, int dtype, i
                  "mole_gate_wgrad: need E <= 32, or bf16 tokens with E <= 256 and M %% 64 == 0 (S=%d E=%d M=%d dtype=%d)", S, E, M, dtype);
     MOLE_REQUIRE(dwg != nullptr, "mole_gate_wgrad: null output");
     hipStream_t st = (hipStream_t)stream;
+    ScopedTiming timing(MOLE_K_GATE_WGRAD, st);
     if (S == 0) {
         // no tokens: the reduction over zero partials writes the zeros (a kernel, not a memset, so that a
         // caller may capture the call in a graph)
@@ -746,8 +785,9 @@ extern "C" int mole_gate_wgrad(const float *dlogits, const void *x, int dtype, i
     if (gate_wgrad_mfma_ok(dtype, S, E, M)) {
         const int chunk = gate_wgrad_mfma_chunk(S, E, M), nchunks = ceil_div(S, chunk);
         const int eg = E <= 16 ? 1 : (E <= 32 ? 2 : 4);
-        const dim3 grid(nchunks, ceil_div(M, 256), ceil_div(E, 16 * eg));
-#define MOLE_GM(EG) hipLaunchKernelGGL((gate_wgrad_mfma_kernel<EG>), grid, dim3(256), 0, st, dlogits, (const bf16_t *)x, S, E, M, chunk, part)
+        const int nz = ceil_div(E, 16 * eg), nunits = nchunks * ceil_div(M, 256);
+        const dim3 grid((unsigned)(ceil_div(nunits, 8) * 8 * nz));
+#define MOLE_GM(EG) hipLaunchKernelGGL((gate_wgrad_mfma_kernel<EG>), grid, dim3(256), 0, st, dlogits, (const bf16_t *)x, S, E, M, chunk, nchunks, nz, part)
         if (eg == 1) MOLE_GM(1); else if (eg == 2) MOLE_GM(2); else MOLE_GM(4);
 #undef MOLE_GM
         MOLE_LAUNCH_CHECK();

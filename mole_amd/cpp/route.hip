@@ -21,18 +21,45 @@
 namespace mole {
 
 constexpr int RT_THREADS = 256;
-constexpr int RT_TOKENS = 64;   // tokens per block: 16 per wave in the top-k phase, one wave ranks all 64
+constexpr int RT_TOKENS = 64;   // tokens per block: 16 per wave in the top-k phase; a choice is ranked by one wave over all 64
 constexpr int RT_WTOK = RT_TOKENS / 4;
 constexpr float FP32_EPS = 1.1920928955078125e-07f;
 
-// strict "a ranks above b" of torch.topk: NaN above everything, NaNs equal among themselves
-__device__ __forceinline__ bool topk_gt(float a, float b) {
-    bool an = a != a, bn = b != b;
-    if (an | bn) return an & !bn;
-    return a > b;
+// torch.topk's order of scores as an unsigned key: NaN ranks above everything and NaNs are equal among
+// themselves, then +inf .. -inf with -0 == +0.  Every key of a real score is above 0, which stands for "not
+// available" (outside the gate, or already chosen).  Equal keys are ranked by expert index, lowest first.
+__device__ __forceinline__ uint32_t topk_key(float v) {
+    uint32_t u = __float_as_uint(v);
+    if (v != v) return 0xffffffffu;
+    if (u == 0x80000000u) u = 0u;
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
-__device__ __forceinline__ bool topk_better(float va, int ia, float vb, int ib) {
-    return topk_gt(va, vb) || (!topk_gt(vb, va) && ia < ib);
+__device__ __forceinline__ float topk_unkey(uint32_t key) {
+    return __uint_as_float((key & 0x80000000u) ? (key ^ 0x80000000u) : ~key);
+}
+
+// max / min over aligned groups of 2^logG lanes, result in every lane of the group.  Within a row of 16 lanes the
+// exchange is a DPP lane pattern (no LDS, no index registers): neighbours, pairs, then the mirrored half row and
+// the mirrored row, each of which pairs a lane with one from the other already-reduced half.  32-lane groups add
+// one crossbar swizzle, the whole wave reads the four row results into scalars.
+template <int CTRL> __device__ __forceinline__ int dpp_lane(int x) {
+    return __builtin_amdgcn_update_dpp(x, x, CTRL, 0xf, 0xf, false);
+}
+template <typename T, typename Op> __device__ __forceinline__ T group_reduce(T x, int logG, Op op) {
+    static_assert(sizeof(T) == 4, "32-bit lanes");
+    auto bits = [](T v) { return __builtin_bit_cast(int, v); };
+    auto val = [](int v) { return __builtin_bit_cast(T, v); };
+    if (logG >= 1) x = op(x, val(dpp_lane<0xb1>(bits(x))));      // quad_perm [1,0,3,2]
+    if (logG >= 2) x = op(x, val(dpp_lane<0x4e>(bits(x))));      // quad_perm [2,3,0,1]
+    if (logG >= 3) x = op(x, val(dpp_lane<0x141>(bits(x))));     // row_half_mirror
+    if (logG >= 4) x = op(x, val(dpp_lane<0x140>(bits(x))));     // row_mirror
+    if (logG == 5) x = op(x, val(__builtin_amdgcn_ds_swizzle(bits(x), 0x401f)));   // lane ^ 16 within 32 lanes
+    if (logG >= 6) {
+        const int xi = bits(x);
+        x = op(op(val(__builtin_amdgcn_readlane(xi, 0)), val(__builtin_amdgcn_readlane(xi, 16))),
+               op(val(__builtin_amdgcn_readlane(xi, 32)), val(__builtin_amdgcn_readlane(xi, 48))));
+    }
+    return x;
 }
 
 template <int VPL>
@@ -43,8 +70,8 @@ __global__ __launch_bounds__(RT_THREADS) void route_topk_kernel(
     extern __shared__ char smem[];
     int *s_idx = (int *)smem;                          // [k][64]
     float *s_graw = (float *)(s_idx + k * RT_TOKENS);  // [k][64]
-    int *s_hist = (int *)(s_graw + k * RT_TOKENS);     // [E]
-    float *s_col = (float *)(s_hist + E);              // [4][E]
+    int *s_hist = (int *)(s_graw + k * RT_TOKENS);     // [4][E]: one histogram per wave
+    float *s_col = (float *)(s_hist + 4 * E);          // [4][E]
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int b = blockIdx.x, tok0 = b * RT_TOKENS;
@@ -62,33 +89,34 @@ __global__ __launch_bounds__(RT_THREADS) void route_topk_kernel(
         const int tl = w * RT_WTOK + tw;
         const int token = tok0 + tl;
         const bool tv = tw < RT_WTOK && token < S;
-        float v[VPL];
-        uint64_t taken = 0;
+        uint32_t key[VPL];
 #pragma unroll
         for (int r = 0; r < VPL; ++r) {
             const int e = g + (r << logG);
             const bool ok = tv && e < E;
-            v[r] = ok ? scores[(size_t)token * E + e] : -INFINITY;
-            if (ok) colacc[r] += v[r];
-            else taken |= 1ull << r;
+            const float sv = ok ? scores[(size_t)token * E + e] : 0.f;
+            if (ok) colacc[r] += sv;
+            key[r] = ok ? topk_key(sv) : 0u;
         }
         for (int j = 0; j < k; ++j) {
-            float bv = -INFINITY;
-            int bi = INT_MAX;
+            // the best score of the token, then the lowest expert index among those that hold it
+            uint32_t best = key[0];
 #pragma unroll
-            for (int r = 0; r < VPL; ++r) {
-                const int e = g + (r << logG);
-                if (!((taken >> r) & 1) && topk_better(v[r], e, bv, bi)) { bv = v[r]; bi = e; }
-            }
-            for (int m = G >> 1; m >= 1; m >>= 1) {
-                const float ov = __shfl_xor(bv, m, WAVE);
-                const int oi = __shfl_xor(bi, m, WAVE);
-                if (topk_better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
-            }
-            if (bi != INT_MAX && (bi & (G - 1)) == g) taken |= 1ull << (bi >> logG);
+            for (int r = 1; r < VPL; ++r) best = max(best, key[r]);
+            const uint32_t top = group_reduce(best, logG, [](uint32_t a, uint32_t c) { return max(a, c); });
+            int cand = INT_MAX;
+#pragma unroll
+            for (int r = VPL - 1; r >= 0; --r)
+                if (key[r] == top) cand = g + (r << logG);             // ends on the lane's lowest such expert
+            if (top == 0u) cand = INT_MAX;                             // nothing available (a token past the end)
+            const int bi = group_reduce(cand, logG, [](int a, int c) { return min(a, c); });
+            const bool mine = bi != INT_MAX && (bi & (G - 1)) == g;
+#pragma unroll
+            for (int r = 0; r < VPL; ++r)
+                if (mine && (bi >> logG) == r) key[r] = 0u;
             if (g == 0 && tv) {
                 s_idx[j * RT_TOKENS + tl] = bi;
-                s_graw[j * RT_TOKENS + tl] = bv;
+                s_graw[j * RT_TOKENS + tl] = topk_unkey(top);
             }
         }
     }
@@ -119,28 +147,30 @@ __global__ __launch_bounds__(RT_THREADS) void route_topk_kernel(
         }
     }
 
-    // ---- phase C: in-block ranks per choice (wave 0: lane = token) -------------------------------
+    // ---- phase C: in-block ranks per choice (lane = token; wave w takes choices w, w + 4, ...) ------
+    // Each wave works on a histogram of its own, so the choices proceed side by side without block barriers
+    // (the loop over distinct experts is a serial chain of ballots: with one wave doing all k choices it was the
+    // longest part of the kernel at top-8).
     const uint64_t lt_mask = (1ull << lane) - 1ull;
-    for (int j = 0; j < k; ++j) {
-        for (int e = tid; e < E; e += RT_THREADS) s_hist[e] = 0;
-        __syncthreads();
-        if (w == 0) {
-            const int e = tv ? s_idx[j * RT_TOKENS + tid] : -1;
-            int rank = 0;
-            uint64_t remaining = __ballot(tv);
-            while (remaining) {
-                const int leader = __ffsll((unsigned long long)remaining) - 1;
-                const int e0 = __shfl(e, leader, WAVE);
-                const uint64_t m = __ballot(tv && e == e0);
-                if (tv && e == e0) rank = __popcll(m & lt_mask);
-                if (lane == leader) s_hist[e0] = __popcll(m);
-                remaining &= ~m;
-            }
-            if (tv) lrank[(size_t)j * S + token] = rank;
+    int *my_hist = s_hist + w * E;
+    const int ctoken = tok0 + lane;
+    const bool cv = ctoken < S;
+    for (int j = w; j < k; j += RT_THREADS / WAVE) {
+        for (int e = lane; e < E; e += WAVE) my_hist[e] = 0;
+        const int e = cv ? s_idx[j * RT_TOKENS + lane] : -1;
+        int rank = 0;
+        uint64_t remaining = __ballot(cv);
+        while (remaining) {
+            const int leader = __ffsll((unsigned long long)remaining) - 1;
+            const int e0 = __shfl(e, leader, WAVE);
+            const uint64_t m = __ballot(cv && e == e0);
+            if (cv && e == e0) rank = __popcll(m & lt_mask);
+            if (lane == leader) my_hist[e0] = __popcll(m);
+            remaining &= ~m;
         }
-        __syncthreads();
-        for (int e2 = tid; e2 < E; e2 += RT_THREADS) hist[((size_t)j * E + e2) * nb + b] = s_hist[e2];
-        __syncthreads();
+        if (cv) lrank[(size_t)j * S + ctoken] = rank;
+        // (the histogram is written and read by this wave only: program order is enough)
+        for (int e2 = lane; e2 < E; e2 += WAVE) hist[((size_t)j * E + e2) * nb + b] = my_hist[e2];
     }
 }
 
@@ -170,10 +200,35 @@ __device__ __forceinline__ void scan_pair(int32_t *__restrict__ hist, int nb, in
     }
     if (lane == 0) counts[pair] = carry;
 }
+// Blocks past the scan's own fold the per-block column sums of the scores (for l_aux) into COLSUM_SLICES rows:
+// slice s adds blocks s, s + COLSUM_SLICES, ... in that order, so the single block that finishes the routing
+// reads COLSUM_SLICES rows instead of one per 64 tokens (at 32768 tokens and 256 experts that loop was 40 us).
+constexpr int COLSUM_SLICES = 16;
 __global__ __launch_bounds__(256) void route_scan_kernel(int32_t *__restrict__ hist, int nb, int npairs,
-                                                         int32_t *__restrict__ counts) {
-    const int pair = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (pair < npairs) scan_pair(hist, nb, pair, counts);
+                                                         int32_t *__restrict__ counts, int scan_blocks,
+                                                         const float *__restrict__ colsum, int E,
+                                                         float *__restrict__ colpart) {
+    if ((int)blockIdx.x < scan_blocks) {
+        const int pair = blockIdx.x * 4 + (threadIdx.x >> 6);
+        if (pair < npairs) scan_pair(hist, nb, pair, counts);
+        return;
+    }
+    const int cb = blockIdx.x - scan_blocks;
+    const int slice = cb % COLSUM_SLICES, e = (cb / COLSUM_SLICES) * 256 + threadIdx.x;
+    if (e >= E) return;
+    float me = 0.f;
+    for (int b0 = slice; b0 < nb; b0 += 8 * COLSUM_SLICES) {        // 8 loads in flight, added in block order
+        float t[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int b = b0 + u * COLSUM_SLICES;
+            t[u] = b < nb ? colsum[(size_t)b * E + e] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (b0 + u * COLSUM_SLICES < nb) me += t[u];
+    }
+    colpart[slice * E + e] = me;
 }
 
 constexpr int FIN_THREADS = 1024;
@@ -304,13 +359,13 @@ extern "C" size_t mole_route_workspace_bytes(int S, int E, int k) {
     if (S < 0 || E <= 0 || k <= 0) return 0;
     const size_t nb = (size_t)ceil_div(S > 0 ? S : 1, RT_TOKENS);
     return align256(nb * k * E * sizeof(int32_t)) + align256((size_t)k * E * sizeof(int32_t)) +
-           align256(nb * E * sizeof(float));
+           align256(nb * E * sizeof(float)) + align256((size_t)COLSUM_SLICES * E * sizeof(float));
 }
 
 template <int VPL>
 static void launch_topk(const float *scores, int S, int E, int k, int logG, int normalize, int32_t *idx,
                         int32_t *loc, float *gates, int32_t *hist, float *colsum, int nb, hipStream_t st) {
-    const size_t lds = (size_t)k * RT_TOKENS * 8 + (size_t)E * 4 + (size_t)E * 4 * 4;
+    const size_t lds = (size_t)k * RT_TOKENS * 8 + (size_t)E * 4 * 4 + (size_t)E * 4 * 4;
     hipLaunchKernelGGL(route_topk_kernel<VPL>, dim3(nb), dim3(RT_THREADS), lds, st, scores, S, E, k, logG,
                        normalize, idx, loc, gates, hist, colsum, nb);
 }
@@ -341,6 +396,8 @@ extern "C" int mole_route(const float *scores, int S, int E, int k, double capac
     int32_t *basej = (int32_t *)ws;
     ws += align256((size_t)k * E * sizeof(int32_t));
     float *colsum = (float *)ws;
+    ws += align256((size_t)nb * E * sizeof(float));
+    float *colpart = (float *)ws;
 
     int logG = 0;
     while ((1 << logG) < E && logG < 6) ++logG;
@@ -355,7 +412,9 @@ extern "C" int mole_route(const float *scores, int S, int E, int k, double capac
     const int npairs = k * E;
     const bool scan_in_finish = (long long)npairs * nb <= 16384;   // small enough for one block: saves a launch
     if (!scan_in_finish) {
-        hipLaunchKernelGGL(route_scan_kernel, dim3(ceil_div(npairs, 4)), dim3(256), 0, st, hist, nb, npairs, counts);
+        const int scan_blocks = ceil_div(npairs, 4);
+        hipLaunchKernelGGL(route_scan_kernel, dim3(scan_blocks + COLSUM_SLICES * ceil_div(E, 256)), dim3(256), 0, st, hist,
+                           nb, npairs, counts, scan_blocks, colsum, E, colpart);
         MOLE_LAUNCH_CHECK();
     }
 
@@ -364,7 +423,9 @@ extern "C" int mole_route(const float *scores, int S, int E, int k, double capac
     // int(cf * spe) of the Python reference: the product is taken in double precision
     const double prod = (capacity_factor < 0. ? -capacity_factor : capacity_factor) * (double)spe;
     const int cap_bound = k * (int)prod;
-    hipLaunchKernelGGL(route_finish_kernel, dim3(1), dim3(FIN_THREADS), 0, st, counts, colsum, nb, S, E, k, cf_sign,
+    // (when the scan kernel ran, it also folded the column sums: the finish then adds its COLSUM_SLICES rows)
+    hipLaunchKernelGGL(route_finish_kernel, dim3(1), dim3(FIN_THREADS), 0, st, counts,
+                       scan_in_finish ? colsum : colpart, scan_in_finish ? nb : min(nb, COLSUM_SLICES), S, E, k, cf_sign,
                        cap_bound, alignment, layout, basej, kept_rows, offsets, capacity, l_aux,
                        scan_in_finish ? hist : (int32_t *)nullptr);
     MOLE_LAUNCH_CHECK();
@@ -586,6 +647,7 @@ extern "C" int mole_softmax_fwd(const float *logits, const float *logit_bias, in
     const int vpl = ceil_div(E, 1 << logG);
     const int tpw = 64 >> logG;
     const dim3 grid(ceil_div(S, 4 * tpw));
+    ScopedTiming timing(MOLE_K_GATE_FWD, (hipStream_t)stream);
     MOLE_VPL_DISPATCH(vpl, softmax_fwd_kernel, grid, (hipStream_t)stream, logits, logit_bias, S, E, logG, scores);
     MOLE_LAUNCH_CHECK();
     return 0;
@@ -603,6 +665,7 @@ extern "C" int mole_gate_fwd(const void *x, int dtype, const float *wg, const fl
     const int eg = ceil_div(E, 16);
     // small gates: 32 tokens per block (Wg, which every block reads in full, is then read half as often)
     const dim3 grid(ceil_div(S, eg <= 2 ? 32 : 16));
+    ScopedTiming timing(MOLE_K_GATE_FWD, st);
     if (eg == 1) hipLaunchKernelGGL((gate_fwd_kernel<1, 8, 2>), grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores);
     else if (eg == 2) hipLaunchKernelGGL((gate_fwd_kernel<2, 4, 2>), grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores);
     else if (eg <= 4) hipLaunchKernelGGL((gate_fwd_kernel<4, 4, 1>), grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores);
@@ -623,6 +686,7 @@ extern "C" int mole_gate_bwd(const float *dgates, const float *scores, const int
     const int vpl = ceil_div(E, 1 << logG);
     const int tpw = 64 >> logG;
     const dim3 grid(ceil_div(S, 4 * tpw));
+    ScopedTiming timing(MOLE_K_GATE_BWD, (hipStream_t)stream);
     MOLE_VPL_DISPATCH(vpl, gate_bwd_kernel, grid, (hipStream_t)stream, dgates, scores, idx, S, E, k, logG,
                       normalize_gate, through_softmax, dlogits);
     MOLE_LAUNCH_CHECK();
