@@ -465,7 +465,7 @@ __global__ __launch_bounds__(256) void softmax_fwd_kernel(const float *__restric
         v[r] = ok ? logits[(size_t)token * E + e] + (bias ? bias[e] : 0.f) : -INFINITY;
         mx = fmaxf(mx, v[r]);
     }
-    for (int m = G >> 1; m >= 1; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m, WAVE));
+    mx = group_reduce(mx, logG, [](float a, float c) { return fmaxf(a, c); });
     float sum = 0.f;
 #pragma unroll
     for (int r = 0; r < VPL; ++r) {
@@ -473,7 +473,7 @@ __global__ __launch_bounds__(256) void softmax_fwd_kernel(const float *__restric
         v[r] = (tv && e < E) ? expf(v[r] - mx) : 0.f;
         sum += v[r];
     }
-    for (int m = G >> 1; m >= 1; m >>= 1) sum += __shfl_xor(sum, m, WAVE);
+    sum = group_reduce(sum, logG, [](float a, float c) { return a + c; });
 #pragma unroll
     for (int r = 0; r < VPL; ++r) {
         const int e = g + (r << logG);
@@ -531,7 +531,7 @@ __global__ __launch_bounds__(256) void gate_bwd_kernel(const float *__restrict__
     float dot = 0.f;
 #pragma unroll
     for (int r = 0; r < VPL; ++r) dot += ds[r] * s[r];
-    for (int m = G >> 1; m >= 1; m >>= 1) dot += __shfl_xor(dot, m, WAVE);
+    dot = group_reduce(dot, logG, [](float a, float c) { return a + c; });
 #pragma unroll
     for (int r = 0; r < VPL; ++r) {
         const int e = g + (r << logG);
