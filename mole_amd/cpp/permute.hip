@@ -20,6 +20,13 @@ template <> struct Vec<float> {
     __device__ __forceinline__ void unpack(float *f) const { f[0] = raw.x; f[1] = raw.y; f[2] = raw.z; f[3] = raw.w; }
     __device__ __forceinline__ void pack(const float *f) { raw = make_float4(f[0], f[1], f[2], f[3]); }
     __device__ __forceinline__ void zero() { raw = make_float4(0.f, 0.f, 0.f, 0.f); }
+    // makes the loaded value opaque to the compiler at this point: without it a load whose only uses sit under
+    // branches is repeated inside every one of them, each time followed by a full wait
+    __device__ __forceinline__ void pin() { asm volatile("" : "+v"(raw.x), "+v"(raw.y), "+v"(raw.z), "+v"(raw.w)); }
+    __device__ __forceinline__ void mask(uint32_t m) {        // m = all ones (keep) or 0 (becomes +0)
+        raw = make_float4(__uint_as_float(__float_as_uint(raw.x) & m), __uint_as_float(__float_as_uint(raw.y) & m),
+                          __uint_as_float(__float_as_uint(raw.z) & m), __uint_as_float(__float_as_uint(raw.w) & m));
+    }
 };
 template <> struct Vec<bf16_t> {
     static constexpr int N = 8;
@@ -44,33 +51,69 @@ template <> struct Vec<bf16_t> {
         raw = make_uint4(w[0], w[1], w[2], w[3]);
     }
     __device__ __forceinline__ void zero() { raw = make_uint4(0, 0, 0, 0); }
+    __device__ __forceinline__ void pin() { asm volatile("" : "+v"(raw.x), "+v"(raw.y), "+v"(raw.z), "+v"(raw.w)); }
+    __device__ __forceinline__ void mask(uint32_t m) { raw = make_uint4(raw.x & m, raw.y & m, raw.z & m, raw.w & m); }
 };
 
 constexpr int PM_THREADS = 256;  // 4 waves = 4 tokens per block
 
-template <typename T>
+// How these kernels keep memory busy.  A wave's loads are issued unconditionally, from addresses clamped to
+// something valid, and a value that must not count (a dropped pair, a choice past k, a chunk past the row's end)
+// is cleared with a bit mask where it is used.  A load written under a condition ("r >= 0 ? load : 0") compiles
+// to a branch around the load, and the compiler then waits for every outstanding load at each such branch: the k
+// row fetches of a token ran one after the other.  With K (the template's bound on k) x PM_U chunk loads in
+// flight per wave the gathers reach the rate of a plain copy.
+constexpr int PM_U = 2;          // 1 KiB chunks of a row in flight per wave and source row
+
+// destination/source rows of token i for the K choice slots: row index (0 when the slot does not count) and
+// keep mask (all ones when it does: a choice below k whose pair was kept)
+template <int K>
+__device__ __forceinline__ void load_rows(const int32_t *__restrict__ row, int S, int k, int i, int (&r)[K],
+                                          uint32_t (&keep)[K]) {
+#pragma unroll
+    for (int j = 0; j < K; ++j) r[j] = row[(size_t)min(j, k - 1) * S + i];      // all K loads first
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+        keep[j] = (j < k && r[j] >= 0) ? 0xffffffffu : 0u;
+        r[j] &= (int)keep[j];
+    }
+}
+
+template <typename T, int K>
 __global__ __launch_bounds__(PM_THREADS) void dispatch_fwd_kernel(const T *__restrict__ x,
                                                                   const int32_t *__restrict__ row, int S, int M,
                                                                   int k, T *__restrict__ xd) {
     const int i = blockIdx.x * (PM_THREADS / WAVE) + (threadIdx.x >> 6);
     if (i >= S) return;
     const int lane = lane_id();
-    int r[MOLE_MAX_TOPK];
-#pragma unroll
-    for (int j = 0; j < MOLE_MAX_TOPK; ++j) r[j] = j < k ? row[(size_t)j * S + i] : -1;
+    int r[K];
+    uint32_t keep[K];
+    load_rows<K>(row, S, k, i, r, keep);
     constexpr int N = Vec<T>::N;
+    constexpr int U = 2 * PM_U;                  // one source row: more of its chunks in flight
     const int chunks = M / N;
     const T *src = x + (size_t)i * M;
-    for (int c = lane; c < chunks; c += WAVE) {
-        Vec<T> v;
-        v.load(src + (size_t)c * N);
+    for (int c0 = lane; c0 < chunks; c0 += U * WAVE) {
+        Vec<T> v[U];
 #pragma unroll
-        for (int j = 0; j < MOLE_MAX_TOPK; ++j)
-            if (r[j] >= 0) v.store(xd + (size_t)r[j] * M + (size_t)c * N);
+        for (int u = 0; u < U; ++u) {
+            const int c = c0 + u * WAVE;
+            v[u].load(src + (size_t)(c < chunks ? c : c0) * N);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int c = c0 + u * WAVE;
+            v[u].pin();
+            if (c < chunks) {
+#pragma unroll
+                for (int j = 0; j < K; ++j)
+                    if (keep[j]) v[u].store(xd + (size_t)r[j] * M + (size_t)c * N);
+            }
+        }
     }
 }
 
-template <typename T>
+template <typename T, int K>
 __global__ __launch_bounds__(PM_THREADS) void dispatch_bwd_kernel(const T *__restrict__ dxd,
                                                                   const int32_t *__restrict__ row, int S, int M,
                                                                   int k, const float *__restrict__ dlogits,
@@ -79,51 +122,61 @@ __global__ __launch_bounds__(PM_THREADS) void dispatch_bwd_kernel(const T *__res
     const int i = blockIdx.x * (PM_THREADS / WAVE) + (threadIdx.x >> 6);
     if (i >= S) return;
     const int lane = lane_id();
-    int r[MOLE_MAX_TOPK];
-#pragma unroll
-    for (int j = 0; j < MOLE_MAX_TOPK; ++j) r[j] = j < k ? row[(size_t)j * S + i] : -1;
+    int r[K];
+    uint32_t keep[K];
+    load_rows<K>(row, S, k, i, r, keep);
     constexpr int N = Vec<T>::N;
+    constexpr int U = K >= 16 ? 1 : PM_U;
     const int chunks = M / N;
-    for (int c = lane; c < chunks; c += WAVE) {
-        float acc[N];
+    // the optional addend goes through the same path as one more source row (row i of dx_add, or masked out)
+    const T *add_row = dx_add != nullptr ? dx_add + (size_t)i * M : dxd;
+    const uint32_t add_keep = dx_add != nullptr ? 0xffffffffu : 0u;
+    for (int c0 = lane; c0 < chunks; c0 += U * WAVE) {
+        Vec<T> v[U][K], va[U];
 #pragma unroll
-        for (int q = 0; q < N; ++q) acc[q] = 0.f;
+        for (int u = 0; u < U; ++u) {
+            const int c = c0 + u * WAVE;
+            const size_t off = (size_t)(c < chunks ? c : c0) * N;
 #pragma unroll
-        for (int j = 0; j < MOLE_MAX_TOPK; ++j) {
-            if (r[j] >= 0) {
-                Vec<T> v;
-                float f[N];
-                v.load(dxd + (size_t)r[j] * M + (size_t)c * N);
-                v.unpack(f);
+            for (int j = 0; j < K; ++j) v[u][j].load(dxd + (size_t)r[j] * M + off);
+            va[u].load(add_row + off);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int c = c0 + u * WAVE;
+            if (c >= chunks) continue;
+            float acc[N], f[N];
+#pragma unroll
+            for (int q = 0; q < N; ++q) acc[q] = 0.f;
+#pragma unroll
+            for (int j = 0; j < K; ++j) {
+                v[u][j].mask(keep[j]);
+                v[u][j].unpack(f);
 #pragma unroll
                 for (int q = 0; q < N; ++q) acc[q] += f[q];
             }
-        }
-        if (dx_add != nullptr) {
-            Vec<T> v;
-            float f[N];
-            v.load(dx_add + (size_t)i * M + (size_t)c * N);
-            v.unpack(f);
+            va[u].mask(add_keep);
+            va[u].unpack(f);
 #pragma unroll
             for (int q = 0; q < N; ++q) acc[q] += f[q];
-        }
-        if (dlogits != nullptr) {
-            for (int e = 0; e < E; ++e) {
-                const float dl = dlogits[(size_t)i * E + e];
-                const float *wrow = wg + (size_t)e * M + (size_t)c * N;
+            if (dlogits != nullptr) {
+                for (int e = 0; e < E; ++e) {
+                    const float dl = dlogits[(size_t)i * E + e];
+                    const float *wrow = wg + (size_t)e * M + (size_t)c * N;
 #pragma unroll
-                for (int q = 0; q < N; q += 4) {
-                    const float4 wv = *reinterpret_cast<const float4 *>(wrow + q);
-                    acc[q] += dl * wv.x;
-                    acc[q + 1] += dl * wv.y;
-                    acc[q + 2] += dl * wv.z;
-                    acc[q + 3] += dl * wv.w;
+                    for (int q = 0; q < N; q += 4) {
+                        const float4 wv = *reinterpret_cast<const float4 *>(wrow + q);
+                        acc[q] += dl * wv.x;
+                        acc[q + 1] += dl * wv.y;
+                        acc[q + 2] += dl * wv.z;
+                        acc[q + 3] += dl * wv.w;
+                    }
                 }
             }
+            Vec<T> o;
+            o.pack(acc);
+            o.store(dx + (size_t)i * M + (size_t)c * N);
         }
-        Vec<T> o;
-        o.pack(acc);
-        o.store(dx + (size_t)i * M + (size_t)c * N);
     }
 }
 
@@ -150,34 +203,43 @@ __global__ __launch_bounds__(256) void dispatch_bwd_gate_kernel(const T *__restr
     // current batch is finished: one token at a time, or one batch at a time, runs at the memory latency.
     constexpr int U = 8;
     typedef typename std::conditional<sizeof(T) == 2, uint2, float4>::type Raw;
-    auto gather = [&](Raw (&v)[U], int ib, int j) __attribute__((always_inline)) {
+    // (every load is issued unconditionally from a clamped address; what must not count - a token past the
+    // block's end, a dropped pair - is masked when it is added: loads under a condition are waited for one by one)
+    auto gather = [&](Raw (&v)[U], uint32_t (&ok)[U], int ib, int j) __attribute__((always_inline)) {
+        int r[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) r[u] = row[(size_t)j * S + min(ib + u, i1 - 1)];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int r = ib + u < i1 ? row[(size_t)j * S + ib + u] : -1;
-            if constexpr (sizeof(T) == 2) v[u] = r >= 0 ? *reinterpret_cast<const uint2 *>(dxd + (size_t)r * M + m) : make_uint2(0, 0);
-            else v[u] = r >= 0 ? *reinterpret_cast<const float4 *>(dxd + (size_t)r * M + m) : make_float4(0.f, 0.f, 0.f, 0.f);
+            ok[u] = (ib + u < i1 && r[u] >= 0) ? 0xffffffffu : 0u;
+            v[u] = *reinterpret_cast<const Raw *>(dxd + (size_t)(r[u] & (int)ok[u]) * M + m);
         }
     };
-    auto add = [&](float (&acc)[U][4], const Raw (&v)[U]) __attribute__((always_inline)) {
+    auto add = [&](float (&acc)[U][4], const Raw (&v)[U], const uint32_t (&ok)[U]) __attribute__((always_inline)) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             if constexpr (sizeof(T) == 2) {
-                acc[u][0] += __uint_as_float(v[u].x << 16); acc[u][1] += __uint_as_float(v[u].x & 0xffff0000u);
-                acc[u][2] += __uint_as_float(v[u].y << 16); acc[u][3] += __uint_as_float(v[u].y & 0xffff0000u);
+                const uint32_t x = v[u].x & ok[u], y = v[u].y & ok[u];
+                acc[u][0] += __uint_as_float(x << 16); acc[u][1] += __uint_as_float(x & 0xffff0000u);
+                acc[u][2] += __uint_as_float(y << 16); acc[u][3] += __uint_as_float(y & 0xffff0000u);
             } else {
-                acc[u][0] += v[u].x; acc[u][1] += v[u].y; acc[u][2] += v[u].z; acc[u][3] += v[u].w;
+                acc[u][0] += __uint_as_float(__float_as_uint(v[u].x) & ok[u]);
+                acc[u][1] += __uint_as_float(__float_as_uint(v[u].y) & ok[u]);
+                acc[u][2] += __uint_as_float(__float_as_uint(v[u].z) & ok[u]);
+                acc[u][3] += __uint_as_float(__float_as_uint(v[u].w) & ok[u]);
             }
         }
     };
-    auto finish = [&](const Raw (&first)[U], int ib) __attribute__((always_inline)) {
+    auto finish = [&](const Raw (&first)[U], const uint32_t (&first_ok)[U], int ib) __attribute__((always_inline)) {
         float acc[U][4];
 #pragma unroll
         for (int u = 0; u < U; ++u) acc[u][0] = acc[u][1] = acc[u][2] = acc[u][3] = 0.f;
-        add(acc, first);
+        add(acc, first, first_ok);
         for (int j = 1; j < k; ++j) {
             Raw v[U];
-            gather(v, ib, j);
-            add(acc, v);
+            uint32_t ok[U];
+            gather(v, ok, ib, j);
+            add(acc, v, ok);
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
@@ -202,12 +264,13 @@ __global__ __launch_bounds__(256) void dispatch_bwd_gate_kernel(const T *__restr
         }
     };
     Raw va[U], vb[U];
-    gather(va, i0, 0);
+    uint32_t oka[U], okb[U];
+    gather(va, oka, i0, 0);
     for (int ib = i0; ib < i1; ib += 2 * U) {
-        gather(vb, ib + U, 0);
-        finish(va, ib);
-        gather(va, ib + 2 * U, 0);
-        if (ib + U < i1) finish(vb, ib + U);
+        gather(vb, okb, ib + U, 0);
+        finish(va, oka, ib);
+        gather(va, oka, ib + 2 * U, 0);
+        if (ib + U < i1) finish(vb, okb, ib + U);
     }
 }
 
@@ -238,16 +301,21 @@ __global__ __launch_bounds__(512) void dispatch_bwd_gate_mfma_kernel(const bf16_
     float *buf = s_t[wave];
     const int tsel = lane >> 4, c8 = (lane & 15) * 8;        // row-major side: token within a quartet, first of 8 columns
     // the first-choice source rows of the 4 tokens this lane finishes in a group (tokens tok0 + 4 u + tsel)
-    auto gather = [&](uint4 (&v)[4], int tok0) __attribute__((always_inline)) {
+    // (loads are unconditional, from clamped addresses, and what must not count is masked where it is used: a
+    // load under a condition would make the compiler wait for all loads in flight at every such place)
+    auto gather = [&](uint4 (&v)[4], uint32_t (&ok)[4], int tok0) __attribute__((always_inline)) {
+        int r[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) r[u] = row[min(tok0 + 4 * u + tsel, S - 1)];
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            const int t = tok0 + 4 * u + tsel;
-            const int r = t < S ? row[t] : -1;
-            v[u] = r >= 0 ? *reinterpret_cast<const uint4 *>(dxd + (size_t)r * M + col0 + c8) : make_uint4(0, 0, 0, 0);
+            ok[u] = (tok0 + 4 * u + tsel < S && r[u] >= 0) ? 0xffffffffu : 0u;
+            v[u] = *reinterpret_cast<const uint4 *>(dxd + (size_t)(r[u] & (int)ok[u]) * M + col0 + c8);
         }
     };
     uint4 src[4];
-    gather(src, blockIdx.x * DM_TOKENS);
+    uint32_t src_ok[4];
+    gather(src, src_ok, blockIdx.x * DM_TOKENS);
     // B fragments: Wg[8 kq + i][col0 + 16 cb + r16], i = 0..7, for the wave's 8 column blocks.  Fetched row by row
     // with 16-byte loads (a lane takes 4 columns of the 8 experts of one group) and turned by way of the LDS
     // buffer, [expert group][column] with a group's 8 experts as one bf16x8 entry: picking them out of global
@@ -262,10 +330,10 @@ __global__ __launch_bounds__(512) void dispatch_bwd_gate_mfma_kernel(const bf16_
             const int eg = 2 * pass + half;
             float4 w[8];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const int e = 8 * eg + i;
-                w[i] = e < E ? *reinterpret_cast<const float4 *>(wg + (size_t)e * M + col0 + c4) : make_float4(0.f, 0.f, 0.f, 0.f);
-            }
+            for (int i = 0; i < 8; ++i) w[i] = *reinterpret_cast<const float4 *>(wg + (size_t)min(8 * eg + i, E - 1) * M + col0 + c4);
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (8 * eg + i >= E) w[i] = make_float4(0.f, 0.f, 0.f, 0.f);
             perm_bf16x8 *dst = wt + half * DM_COLS + c4;
             dst[0] = perm_bf16x8{(bf16_t)w[0].x, (bf16_t)w[1].x, (bf16_t)w[2].x, (bf16_t)w[3].x,
                                  (bf16_t)w[4].x, (bf16_t)w[5].x, (bf16_t)w[6].x, (bf16_t)w[7].x};
@@ -291,14 +359,15 @@ __global__ __launch_bounds__(512) void dispatch_bwd_gate_mfma_kernel(const bf16_
     for (int g0 = 0; g0 < DM_TOKENS; g0 += 16) {
         const int tok0 = blockIdx.x * DM_TOKENS + g0;
         uint4 nxt[4];
-        if (g0 + 16 < DM_TOKENS) gather(nxt, tok0 + 16);
+        uint32_t nxt_ok[4];
+        if (g0 + 16 < DM_TOKENS) gather(nxt, nxt_ok, tok0 + 16);
         // A fragment: dlogits[tok0 + r16][8 kq .. 8 kq + 7]
         float d[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int e = 8 * kq + i;
-            d[i] = (tok0 + r16 < S && e < E) ? dlogits[(size_t)(tok0 + r16) * E + e] : 0.f;
-        }
+        for (int i = 0; i < 8; ++i) d[i] = dlogits[(size_t)min(tok0 + r16, S - 1) * E + min(8 * kq + i, E - 1)];
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (tok0 + r16 >= S || 8 * kq + i >= E) d[i] = 0.f;
         const perm_bf16x8 afrag = {(bf16_t)d[0], (bf16_t)d[1], (bf16_t)d[2], (bf16_t)d[3],
                                    (bf16_t)d[4], (bf16_t)d[5], (bf16_t)d[6], (bf16_t)d[7]};
         // product tiles into LDS: acc[r] = token 4 kq + r, column 16 cb + r16 (conflict-free: see DM_ROW)
@@ -318,17 +387,18 @@ __global__ __launch_bounds__(512) void dispatch_bwd_gate_mfma_kernel(const bf16_
             Vec<bf16_t> v;
             float f[8];
             v.raw = src[u];
+            v.mask(src_ok[u]);
             v.unpack(f);
 #pragma unroll
             for (int q = 0; q < 8; ++q) acc[q] += f[q];
             for (int j = 1; j < k; ++j) {
-                const int r = t < S ? row[(size_t)j * S + t] : -1;
-                if (r >= 0) {
-                    v.load(dxd + (size_t)r * M + col0 + c8);
-                    v.unpack(f);
+                const int r = row[(size_t)j * S + min(t, S - 1)];
+                const uint32_t ok = (t < S && r >= 0) ? 0xffffffffu : 0u;
+                v.load(dxd + (size_t)(r & (int)ok) * M + col0 + c8);
+                v.mask(ok);
+                v.unpack(f);
 #pragma unroll
-                    for (int q = 0; q < 8; ++q) acc[q] += f[q];
-                }
+                for (int q = 0; q < 8; ++q) acc[q] += f[q];
             }
             if (t < S) {
                 v.pack(acc);
@@ -337,7 +407,7 @@ __global__ __launch_bounds__(512) void dispatch_bwd_gate_mfma_kernel(const bf16_
         }
         if (g0 + 16 < DM_TOKENS) {
 #pragma unroll
-            for (int u = 0; u < 4; ++u) src[u] = nxt[u];
+            for (int u = 0; u < 4; ++u) { src[u] = nxt[u]; src_ok[u] = nxt_ok[u]; }
         }
     }
 }
@@ -588,7 +658,7 @@ __global__ __launch_bounds__(256) void gate_wgrad_reduce_kernel(const float *__r
     }
 }
 
-template <typename T>
+template <typename T, int K>
 __global__ __launch_bounds__(PM_THREADS) void combine_fwd_kernel(const T *__restrict__ o,
                                                                  const int32_t *__restrict__ row,
                                                                  const float *__restrict__ gates, int S, int M,
@@ -596,37 +666,47 @@ __global__ __launch_bounds__(PM_THREADS) void combine_fwd_kernel(const T *__rest
     const int i = blockIdx.x * (PM_THREADS / WAVE) + (threadIdx.x >> 6);
     if (i >= S) return;
     const int lane = lane_id();
-    int r[MOLE_MAX_TOPK];
-    float g[MOLE_MAX_TOPK];
+    int r[K];
+    uint32_t keep[K];
+    float g[K];
+    load_rows<K>(row, S, k, i, r, keep);
 #pragma unroll
-    for (int j = 0; j < MOLE_MAX_TOPK; ++j) {
-        r[j] = j < k ? row[(size_t)j * S + i] : -1;
-        g[j] = j < k ? gates[(size_t)j * S + i] : 0.f;
-    }
+    for (int j = 0; j < K; ++j) g[j] = gates[(size_t)min(j, k - 1) * S + i];
     constexpr int N = Vec<T>::N;
+    constexpr int U = K >= 16 ? 1 : PM_U;
     const int chunks = M / N;
-    for (int c = lane; c < chunks; c += WAVE) {
-        float acc[N];
+    for (int c0 = lane; c0 < chunks; c0 += U * WAVE) {
+        Vec<T> v[U][K];
 #pragma unroll
-        for (int q = 0; q < N; ++q) acc[q] = 0.f;
+        for (int u = 0; u < U; ++u) {
+            const int c = c0 + u * WAVE;
+            const size_t off = (size_t)(c < chunks ? c : c0) * N;
 #pragma unroll
-        for (int j = 0; j < MOLE_MAX_TOPK; ++j) {
-            if (r[j] >= 0) {
-                Vec<T> v;
-                float f[N];
-                v.load(o + (size_t)r[j] * M + (size_t)c * N);
-                v.unpack(f);
-#pragma unroll
-                for (int q = 0; q < N; ++q) acc[q] += g[j] * f[q];
-            }
+            for (int j = 0; j < K; ++j) v[u][j].load(o + (size_t)r[j] * M + off);
         }
-        Vec<T> out;
-        out.pack(acc);
-        out.store(y + (size_t)i * M + (size_t)c * N);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int c = c0 + u * WAVE;
+            if (c >= chunks) continue;
+            float acc[N], f[N];
+#pragma unroll
+            for (int q = 0; q < N; ++q) acc[q] = 0.f;
+#pragma unroll
+            for (int j = 0; j < K; ++j) {
+                v[u][j].mask(keep[j]);         // a slot that does not count contributes g * (+0)
+                v[u][j].unpack(f);
+                const float gj = __uint_as_float(__float_as_uint(g[j]) & keep[j]);
+#pragma unroll
+                for (int q = 0; q < N; ++q) acc[q] += gj * f[q];
+            }
+            Vec<T> out;
+            out.pack(acc);
+            out.store(y + (size_t)i * M + (size_t)c * N);
+        }
     }
 }
 
-template <typename T>
+template <typename T, int K>
 __global__ __launch_bounds__(PM_THREADS) void combine_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ o,
                                                                  const int32_t *__restrict__ row,
                                                                  const float *__restrict__ gates, int S, int M,
@@ -635,31 +715,56 @@ __global__ __launch_bounds__(PM_THREADS) void combine_bwd_kernel(const T *__rest
     const int i = blockIdx.x * (PM_THREADS / WAVE) + (threadIdx.x >> 6);
     if (i >= S) return;
     const int lane = lane_id();
+    int r[K];
+    uint32_t keep[K];
+    float g[K], dot[K];
+    load_rows<K>(row, S, k, i, r, keep);
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+        g[j] = gates[(size_t)min(j, k - 1) * S + i];
+        dot[j] = 0.f;
+    }
     constexpr int N = Vec<T>::N;
+    constexpr int U = K >= 8 ? 1 : PM_U;
     const int chunks = M / N;
-    for (int j = 0; j < k; ++j) {
-        const int r = row[(size_t)j * S + i];
-        float dot = 0.f;
-        if (r >= 0) {
-            const float g = gates[(size_t)j * S + i];
-            for (int c = lane; c < chunks; c += WAVE) {
-                Vec<T> a, b, w;
-                float fa[N], fb[N], fo[N];
-                a.load(dy + (size_t)i * M + (size_t)c * N);
-                b.load(o + (size_t)r * M + (size_t)c * N);
-                a.unpack(fa);
-                b.unpack(fb);
+    for (int c0 = lane; c0 < chunks; c0 += U * WAVE) {
+        Vec<T> a[U], b[U][K];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int c = c0 + u * WAVE;
+            const size_t off = (size_t)(c < chunks ? c : c0) * N;
+            a[u].load(dy + (size_t)i * M + off);
+#pragma unroll
+            for (int j = 0; j < K; ++j) b[u][j].load(o + (size_t)r[j] * M + off);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int c = c0 + u * WAVE;
+            if (c >= chunks) continue;
+            float fa[N];
+            a[u].unpack(fa);
+#pragma unroll
+            for (int j = 0; j < K; ++j) {
+                float fb[N], fo[N];
+                b[u][j].mask(keep[j]);         // a slot that does not count: dot stays 0, nothing is stored
+                b[u][j].unpack(fb);
 #pragma unroll
                 for (int q = 0; q < N; ++q) {
-                    dot += fa[q] * fb[q];
-                    fo[q] = g * fa[q];
+                    dot[j] += fa[q] * fb[q];
+                    fo[q] = g[j] * fa[q];
                 }
-                w.pack(fo);
-                w.store(d_o + (size_t)r * M + (size_t)c * N);
+                if (keep[j]) {
+                    Vec<T> w;
+                    w.pack(fo);
+                    w.store(d_o + (size_t)r[j] * M + (size_t)c * N);
+                }
             }
-            dot = wave_sum(dot);
         }
-        if (lane == 0) dgates[(size_t)j * S + i] = dot;
+    }
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+        const float d = wave_sum(dot[j]);
+        if (lane == 0 && j < k) dgates[(size_t)j * S + i] = d;
     }
 }
 
@@ -689,6 +794,16 @@ static int check_perm(const char *fn, int dtype, int S, int M, int k) {
 }
 static bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
+// the kernels above for the smallest K in {1, 2, 4, 8, 16} that holds k
+#define PM_LAUNCH_K(KERNEL, T, ...)                                                                                   \
+    do {                                                                                                              \
+        if (k <= 1) hipLaunchKernelGGL((KERNEL<T, 1>), grid, dim3(PM_THREADS), 0, (hipStream_t)stream, __VA_ARGS__);       \
+        else if (k <= 2) hipLaunchKernelGGL((KERNEL<T, 2>), grid, dim3(PM_THREADS), 0, (hipStream_t)stream, __VA_ARGS__);  \
+        else if (k <= 4) hipLaunchKernelGGL((KERNEL<T, 4>), grid, dim3(PM_THREADS), 0, (hipStream_t)stream, __VA_ARGS__);  \
+        else if (k <= 8) hipLaunchKernelGGL((KERNEL<T, 8>), grid, dim3(PM_THREADS), 0, (hipStream_t)stream, __VA_ARGS__);  \
+        else hipLaunchKernelGGL((KERNEL<T, 16>), grid, dim3(PM_THREADS), 0, (hipStream_t)stream, __VA_ARGS__);             \
+    } while (0)
+
 }  // namespace mole
 
 using namespace mole;
@@ -701,11 +816,9 @@ extern "C" int mole_dispatch_fwd(const void *x, int dtype, const int32_t *row, i
     const dim3 grid(ceil_div(S, PM_THREADS / WAVE));
     ScopedTiming timing(MOLE_K_DISPATCH_FWD, (hipStream_t)stream);
     if (dtype == MOLE_BF16)
-        hipLaunchKernelGGL(dispatch_fwd_kernel<bf16_t>, grid, dim3(PM_THREADS), 0, (hipStream_t)stream,
-                           (const bf16_t *)x, row, S, M, k, (bf16_t *)xd);
+        PM_LAUNCH_K(dispatch_fwd_kernel, bf16_t, (const bf16_t *)x, row, S, M, k, (bf16_t *)xd);
     else
-        hipLaunchKernelGGL(dispatch_fwd_kernel<float>, grid, dim3(PM_THREADS), 0, (hipStream_t)stream,
-                           (const float *)x, row, S, M, k, (float *)xd);
+        PM_LAUNCH_K(dispatch_fwd_kernel, float, (const float *)x, row, S, M, k, (float *)xd);
     MOLE_LAUNCH_CHECK();
     return 0;
 }
@@ -742,11 +855,9 @@ extern "C" int mole_dispatch_bwd(const void *dxd, int dtype, const int32_t *row,
     }
     const dim3 grid(ceil_div(S, PM_THREADS / WAVE));
     if (dtype == MOLE_BF16)
-        hipLaunchKernelGGL(dispatch_bwd_kernel<bf16_t>, grid, dim3(PM_THREADS), 0, (hipStream_t)stream,
-                           (const bf16_t *)dxd, row, S, M, k, dlogits, wg, E, (const bf16_t *)dx_add, (bf16_t *)dx);
+        PM_LAUNCH_K(dispatch_bwd_kernel, bf16_t, (const bf16_t *)dxd, row, S, M, k, dlogits, wg, E, (const bf16_t *)dx_add, (bf16_t *)dx);
     else
-        hipLaunchKernelGGL(dispatch_bwd_kernel<float>, grid, dim3(PM_THREADS), 0, (hipStream_t)stream,
-                           (const float *)dxd, row, S, M, k, dlogits, wg, E, (const float *)dx_add, (float *)dx);
+        PM_LAUNCH_K(dispatch_bwd_kernel, float, (const float *)dxd, row, S, M, k, dlogits, wg, E, (const float *)dx_add, (float *)dx);
     MOLE_LAUNCH_CHECK();
     return 0;
 }
@@ -818,11 +929,9 @@ extern "C" int mole_combine_fwd(const void *o, int dtype, const int32_t *row, co
     const dim3 grid(ceil_div(S, PM_THREADS / WAVE));
     ScopedTiming timing(MOLE_K_COMBINE_FWD, (hipStream_t)stream);
     if (dtype == MOLE_BF16)
-        hipLaunchKernelGGL(combine_fwd_kernel<bf16_t>, grid, dim3(PM_THREADS), 0, (hipStream_t)stream,
-                           (const bf16_t *)o, row, gates, S, M, k, (bf16_t *)y);
+        PM_LAUNCH_K(combine_fwd_kernel, bf16_t, (const bf16_t *)o, row, gates, S, M, k, (bf16_t *)y);
     else
-        hipLaunchKernelGGL(combine_fwd_kernel<float>, grid, dim3(PM_THREADS), 0, (hipStream_t)stream,
-                           (const float *)o, row, gates, S, M, k, (float *)y);
+        PM_LAUNCH_K(combine_fwd_kernel, float, (const float *)o, row, gates, S, M, k, (float *)y);
     MOLE_LAUNCH_CHECK();
     return 0;
 }
@@ -836,11 +945,9 @@ extern "C" int mole_combine_bwd(const void *dy, const void *o, int dtype, const 
     const dim3 grid(ceil_div(S, PM_THREADS / WAVE));
     ScopedTiming timing(MOLE_K_COMBINE_BWD, (hipStream_t)stream);
     if (dtype == MOLE_BF16)
-        hipLaunchKernelGGL(combine_bwd_kernel<bf16_t>, grid, dim3(PM_THREADS), 0, (hipStream_t)stream,
-                           (const bf16_t *)dy, (const bf16_t *)o, row, gates, S, M, k, (bf16_t *)d_o, dgates);
+        PM_LAUNCH_K(combine_bwd_kernel, bf16_t, (const bf16_t *)dy, (const bf16_t *)o, row, gates, S, M, k, (bf16_t *)d_o, dgates);
     else
-        hipLaunchKernelGGL(combine_bwd_kernel<float>, grid, dim3(PM_THREADS), 0, (hipStream_t)stream,
-                           (const float *)dy, (const float *)o, row, gates, S, M, k, (float *)d_o, dgates);
+        PM_LAUNCH_K(combine_bwd_kernel, float, (const float *)dy, (const float *)o, row, gates, S, M, k, (float *)d_o, dgates);
     MOLE_LAUNCH_CHECK();
     return 0;
 }
