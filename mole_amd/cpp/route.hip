@@ -25,6 +25,14 @@ constexpr int RT_TOKENS = 64;   // tokens per block: 16 per wave in the top-k ph
 constexpr int RT_WTOK = RT_TOKENS / 4;
 constexpr float FP32_EPS = 1.1920928955078125e-07f;
 
+// A load that is always issued (the caller clamps the address to something valid) and gives +0 where the value
+// must not count.  Written as "ok ? p[i] : 0" the load sits under a branch, and the compiler then waits for every
+// load in flight at each such branch: a batch of loads meant to overlap runs one after the other.
+__device__ __forceinline__ float load_or_zero(const float *p, bool ok) {
+    return __uint_as_float(__float_as_uint(*p) & (ok ? 0xffffffffu : 0u));
+}
+__device__ __forceinline__ int load_or_zero(const int *p, bool ok) { return *p & (ok ? -1 : 0); }
+
 // torch.topk's order of scores as an unsigned key: NaN ranks above everything and NaNs are equal among
 // themselves, then +inf .. -inf with -0 == +0.  Every key of a real score is above 0, which stands for "not
 // available" (outside the gate, or already chosen).  Equal keys are ranked by expert index, lowest first.
@@ -84,6 +92,16 @@ __global__ __launch_bounds__(RT_THREADS) void route_topk_kernel(
 #pragma unroll
     for (int r = 0; r < VPL; ++r) colacc[r] = 0.f;
 
+    // the scores of the wave's next token(s) are fetched while the current ones go through their k rounds
+    float nxt[VPL];
+#pragma unroll
+    for (int r = 0; r < VPL; ++r) nxt[r] = 0.f;
+    auto fetch = [&](int it) __attribute__((always_inline)) {
+        const int tok = min(tok0 + w * RT_WTOK + it * tpw + tg, S - 1);
+#pragma unroll
+        for (int r = 0; r < VPL; ++r) nxt[r] = scores[(size_t)tok * E + min(g + (r << logG), E - 1)];
+    };
+    if (S > 0) fetch(0);
     for (int it = 0; it * tpw < RT_WTOK; ++it) {
         const int tw = it * tpw + tg;                  // token within the wave's 16
         const int tl = w * RT_WTOK + tw;
@@ -92,12 +110,12 @@ __global__ __launch_bounds__(RT_THREADS) void route_topk_kernel(
         uint32_t key[VPL];
 #pragma unroll
         for (int r = 0; r < VPL; ++r) {
-            const int e = g + (r << logG);
-            const bool ok = tv && e < E;
-            const float sv = ok ? scores[(size_t)token * E + e] : 0.f;
-            if (ok) colacc[r] += sv;
+            const bool ok = tv && g + (r << logG) < E;
+            const float sv = __uint_as_float(__float_as_uint(nxt[r]) & (ok ? 0xffffffffu : 0u));
+            colacc[r] += sv;
             key[r] = ok ? topk_key(sv) : 0u;
         }
+        if (S > 0 && (it + 1) * tpw < RT_WTOK) fetch(it + 1);
         for (int j = 0; j < k; ++j) {
             // the best score of the token, then the lowest expert index among those that hold it
             uint32_t best = key[0];
@@ -184,7 +202,7 @@ __device__ __forceinline__ void scan_pair(int32_t *__restrict__ hist, int nb, in
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int bi = c0 + u * WAVE + lane;
-            v[u] = bi < nb ? hist[(size_t)pair * nb + bi] : 0;
+            v[u] = load_or_zero(hist + (size_t)pair * nb + min(bi, nb - 1), bi < nb);
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
@@ -222,7 +240,7 @@ __global__ __launch_bounds__(256) void route_scan_kernel(int32_t *__restrict__ h
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             const int b = b0 + u * COLSUM_SLICES;
-            t[u] = b < nb ? colsum[(size_t)b * E + e] : 0.f;
+            t[u] = load_or_zero(colsum + (size_t)min(b, nb - 1) * E + e, b < nb);
         }
 #pragma unroll
         for (int u = 0; u < 8; ++u)
@@ -462,7 +480,9 @@ __global__ __launch_bounds__(256) void softmax_fwd_kernel(const float *__restric
     for (int r = 0; r < VPL; ++r) {
         const int e = g + (r << logG);
         const bool ok = tv && e < E;
-        v[r] = ok ? logits[(size_t)token * E + e] + (bias ? bias[e] : 0.f) : -INFINITY;
+        // (an unconditional load from a clamped address; entries that do not exist become -inf)
+        const float lg = load_or_zero(logits + (size_t)min(token, S - 1) * E + min(e, E - 1), ok);
+        v[r] = lg + (ok ? (bias ? bias[e] : 0.f) : -INFINITY);
         mx = fmaxf(mx, v[r]);
     }
     mx = group_reduce(mx, logG, [](float a, float c) { return fmaxf(a, c); });
@@ -482,8 +502,8 @@ __global__ __launch_bounds__(256) void softmax_fwd_kernel(const float *__restric
 }
 
 // dlogits[i,e] = s[i,e] * (dscore[i,e] - sum_e' dscore[i,e'] s[i,e']), dscore scattered from dgates
-// through gate_j = graw_j / max(sum graw, eps).  One thread per token for the k-sized part, then the
-// group of lanes writes the row.
+// through gate_j = graw_j / max(sum graw, eps).  The token's group of lanes shares the k-sized part, then
+// writes the row.
 template <int VPL>
 __global__ __launch_bounds__(256) void gate_bwd_kernel(const float *__restrict__ dgates,
                                                        const float *__restrict__ scores,
@@ -501,31 +521,40 @@ __global__ __launch_bounds__(256) void gate_bwd_kernel(const float *__restrict__
 #pragma unroll
     for (int r = 0; r < VPL; ++r) {
         const int e = g + (r << logG);
-        s[r] = (tv && e < E) ? scores[(size_t)token * E + e] : 0.f;
+        s[r] = load_or_zero(scores + (size_t)min(token, S - 1) * E + min(e, E - 1), tv && e < E);
         ds[r] = 0.f;
     }
-    if (tv) {
-        float denom = 0.f, dotg = 0.f;
-        for (int j = 0; j < k; ++j) {
-            const int e = idx[(size_t)j * S + token];
-            const float gr = scores[(size_t)token * E + e];
-            denom += gr;
-            dotg += dgates[(size_t)j * S + token] * gr;
+    // Lane j < k of the token's group fetches choice j (index, incoming gradient, raw gate value), the sums over
+    // the k choices are lane reductions, and each choice is then handed round the group.  (With every lane walking
+    // the k choices itself the token paid 2 k dependent memory latencies.)
+    const bool has = tv && g < k;
+    const int tokc = min(token, S - 1), jc = min(g, k - 1);
+    const int my_e = idx[(size_t)jc * S + tokc];
+    const float my_dg = load_or_zero(dgates + (size_t)jc * S + tokc, has);
+    const float my_gr = load_or_zero(scores + (size_t)tokc * E + min(max(my_e, 0), E - 1), has);
+    const float denom = group_reduce(my_gr, logG, [](float a, float c) { return a + c; });
+    const float dotg = group_reduce(my_dg * my_gr, logG, [](float a, float c) { return a + c; });
+    const bool norm = k > 1 && normalize;
+    const bool clamped = denom < FP32_EPS;
+    const float den = clamped ? FP32_EPS : denom;
+    const float sub = (norm && !clamped) ? dotg / (den * den) : 0.f;
+    const float my_dgraw = norm ? my_dg / den - sub : my_dg;
+    const int group_base = lane & ~(G - 1);
+    for (int j = 0; j < k; ++j) {
+        int e;
+        float dgraw;
+        if (logG >= 6) {       // the group is the wave: lane j is a scalar read
+            e = __builtin_amdgcn_readlane(my_e, j);
+            dgraw = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_dgraw), j));
+        } else {
+            e = __shfl(my_e, group_base + j, WAVE);
+            dgraw = __shfl(my_dgraw, group_base + j, WAVE);
         }
-        const bool norm = k > 1 && normalize;
-        const bool clamped = denom < FP32_EPS;
-        const float den = clamped ? FP32_EPS : denom;
-        const float sub = (norm && !clamped) ? dotg / (den * den) : 0.f;
-        for (int j = 0; j < k; ++j) {
-            const int e = idx[(size_t)j * S + token];
-            const float dg = dgates[(size_t)j * S + token];
-            const float dgraw = norm ? dg / den - sub : dg;
-            if ((e & (G - 1)) == g) {
-                const int rr = e >> logG;
+        if ((e & (G - 1)) == g) {
+            const int rr = e >> logG;
 #pragma unroll
-                for (int r = 0; r < VPL; ++r)
-                    if (r == rr) ds[r] += dgraw;
-            }
+            for (int r = 0; r < VPL; ++r)
+                if (r == rr) ds[r] += dgraw;
         }
     }
     float dot = 0.f;
