@@ -432,17 +432,21 @@ __device__ __forceinline__ void epilogue(const GemmArgs &g, f32x16 (&acc)[Tile<T
                 *reinterpret_cast<uint4 *>(dst + (crow0 + m0 + row) * g.ldc + nw0 + jc * 8) = v;
         }
     };
-    // global -> slab, eight rows' loads in flight at a time
+    // global -> slab, eight rows' loads in flight at a time.  Every load is issued, from an address clamped
+    // into the operand (rows past the end read its last row, columns past the end its first column): what lands
+    // in cells outside the live part is never written back, and a load under a condition would make the
+    // compiler wait for all loads in flight at each one, so the eight would run one after the other.
+    const long row_last = crow0 + m_ext - 1;
+    const int col_c = col_ok ? nw0 + jc * 8 : 0;
     auto fill = [&](const bf16_t *src) __attribute__((always_inline)) {
 #pragma unroll
         for (int it0 = 0; it0 < TMC * 4; it0 += 8) {
             uint4 v[8];
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const int row = (it0 + i) * 8 + jr;
-                v[i] = make_uint4(0, 0, 0, 0);
-                if (it0 + i < TMC * 4 && row < live && col_ok)
-                    v[i] = *reinterpret_cast<const uint4 *>(src + (crow0 + m0 + row) * g.ldc + nw0 + jc * 8);
+                if (it0 + i >= TMC * 4) continue;
+                const long row = crow0 + m0 + (it0 + i) * 8 + jr;
+                v[i] = *reinterpret_cast<const uint4 *>(src + (row < row_last ? row : row_last) * g.ldc + col_c);
             }
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
