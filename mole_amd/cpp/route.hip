@@ -596,20 +596,47 @@ __global__ __launch_bounds__(256) void gate_fwd_kernel(const bf16_t *__restrict_
 #pragma unroll
         for (int g = 0; g < EG; ++g) acc[tg][g] = gate_f32x4{0.f, 0.f, 0.f, 0.f};
     const int nsteps = M >> 7;                    // 32 of k per step, a quarter of M per wave
+    // All loads of a round of KSTEPS steps go out first, unconditionally (a step past the end repeats the last
+    // one and is masked below): under a condition each load would be waited for before the next is issued.  For
+    // small gates the weights of the round are fetched ahead as well.
+    constexpr bool W_AHEAD = EG * KSTEPS <= 16;
     for (int s0 = 0; s0 < nsteps; s0 += KSTEPS) {
         uint4 a[TG][KSTEPS];
-#pragma unroll
-        for (int tg = 0; tg < TG; ++tg)
-#pragma unroll
-            for (int i = 0; i < KSTEPS; ++i)
-                a[tg][i] = s0 + i < nsteps ? *reinterpret_cast<const uint4 *>(xp[tg] + (s0 + i) * 32) : make_uint4(0, 0, 0, 0);
+        float4 wa[W_AHEAD ? KSTEPS : 1][W_AHEAD ? EG : 1][2];
 #pragma unroll
         for (int i = 0; i < KSTEPS; ++i) {
-            if (s0 + i >= nsteps) break;
+            const int sc = min(s0 + i, nsteps - 1);
+#pragma unroll
+            for (int tg = 0; tg < TG; ++tg) a[tg][i] = *reinterpret_cast<const uint4 *>(xp[tg] + sc * 32);
+            if constexpr (W_AHEAD) {
+#pragma unroll
+                for (int g = 0; g < EG; ++g) {
+                    const float *wp = wg + (size_t)min(g * 16 + r16, E - 1) * M + kbase + sc * 32;
+                    wa[i][g][0] = *reinterpret_cast<const float4 *>(wp);
+                    wa[i][g][1] = *reinterpret_cast<const float4 *>(wp + 4);
+                }
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);       // or the scheduler moves each load down to its use again
+#pragma unroll
+        for (int i = 0; i < KSTEPS; ++i) {
+            // (no branch here, so that the round stays one block of code and its loads stay ahead of it: a step
+            // past the end multiplies zeros)
+            const uint32_t keep = s0 + i < nsteps ? 0xffffffffu : 0u;
+#pragma unroll
+            for (int tg = 0; tg < TG; ++tg)
+                a[tg][i] = make_uint4(a[tg][i].x & keep, a[tg][i].y & keep, a[tg][i].z & keep, a[tg][i].w & keep);
 #pragma unroll
             for (int g = 0; g < EG; ++g) {
-                const float *wp = wg + (size_t)min(g * 16 + r16, E - 1) * M + kbase + (s0 + i) * 32;
-                const float4 w0 = *reinterpret_cast<const float4 *>(wp), w1 = *reinterpret_cast<const float4 *>(wp + 4);
+                float4 w0, w1;
+                if constexpr (W_AHEAD) {
+                    w0 = wa[i][g][0];
+                    w1 = wa[i][g][1];
+                } else {
+                    const float *wp = wg + (size_t)min(g * 16 + r16, E - 1) * M + kbase + min(s0 + i, nsteps - 1) * 32;
+                    w0 = *reinterpret_cast<const float4 *>(wp);
+                    w1 = *reinterpret_cast<const float4 *>(wp + 4);
+                }
                 const gate_bf16x8 b = {(bf16_t)w0.x, (bf16_t)w0.y, (bf16_t)w0.z, (bf16_t)w0.w,
                                        (bf16_t)w1.x, (bf16_t)w1.y, (bf16_t)w1.z, (bf16_t)w1.w};
 #pragma unroll
