@@ -53,8 +53,9 @@ int mole_version(void);
 const char *mole_last_error_string(void);
 
 /* Optional per-kernel timing for benchmarks (no counterpart in the reference, whose timers wrap
- * whole layers: MOLE/utils/Utimer.py:5-70).  While enabled, each kernel below is bracketed by two
- * events on the stream it runs on; mole_kernel_timing_read() waits for them and returns, for ids
+ * whole layers: MOLE/utils/Utimer.py:5-70).  While enabled, each kernel launch carries a start and a
+ * stop event of its own (entry points that launch several kernels under one id are bracketed by two
+ * events on the stream instead); mole_kernel_timing_read() waits for them and returns, for ids
  * 0..n_ids-1, the number of launches and their summed duration in ms, then forgets them. */
 enum {
     MOLE_K_FFN_FWD1 = 0,  /* h = xd.w1^T + b1, a = gelu(h) */

@@ -115,13 +115,12 @@ extern "C" int mole_adam_step(const void *p, const void *g, float *m, float *v, 
     const size_t blocks = (n + per_block - 1) / per_block;
     MOLE_REQUIRE(blocks <= 0x7fffffffull, "mole_adam_step: n=%zu too large for one launch", n);
     hipStream_t st = (hipStream_t)stream;
-    ScopedTiming timing(MOLE_K_ADAM, st);
     if (dtype == MOLE_BF16)
-        hipLaunchKernelGGL(adam_bf16_kernel, dim3((unsigned)blocks), dim3(ADAM_THREADS), 0, st, (const bf16_t *)p,
-                           (const bf16_t *)g, m, v, (bf16_t *)p_out, n, a);
+        timed_launch(MOLE_K_ADAM, adam_bf16_kernel, dim3((unsigned)blocks), dim3(ADAM_THREADS), 0, st, (const bf16_t *)p,
+                     (const bf16_t *)g, m, v, (bf16_t *)p_out, n, a);
     else
-        hipLaunchKernelGGL(adam_f32_kernel, dim3((unsigned)blocks), dim3(ADAM_THREADS), 0, st, (const float *)p,
-                           (const float *)g, m, v, (float *)p_out, n, a);
+        timed_launch(MOLE_K_ADAM, adam_f32_kernel, dim3((unsigned)blocks), dim3(ADAM_THREADS), 0, st, (const float *)p,
+                     (const float *)g, m, v, (float *)p_out, n, a);
     MOLE_LAUNCH_CHECK();
     return 0;
 }

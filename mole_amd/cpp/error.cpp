@@ -1,8 +1,9 @@
 // Library-wide plumbing of the C ABI: error string, version, and optional per-kernel timing.
 //
-// Timing: when enabled, every instrumented launch is bracketed by two events recorded on the
-// stream the kernel runs on; mole_kernel_timing_read() synchronises those events and returns, per
-// kernel id, the number of launches and their summed duration.  Disabled (the default) it costs
+// Timing: when enabled, every instrumented kernel launch carries a start and a stop event of its own
+// (entry points that launch several kernels under one id are bracketed by two events recorded on the
+// stream instead); mole_kernel_timing_read() synchronises those events and returns, per kernel id, the
+// number of launches and their summed duration.  Disabled (the default) it costs
 // one predictable branch per launch.
 #include "common.h"
 
@@ -41,6 +42,13 @@ void timing_begin(int id, hipStream_t st) {
     std::lock_guard<std::mutex> lk(g_tmu);
     TimedLaunch t{id, get_event(), get_event()};
     (void)hipEventRecord(t.a, st);
+    g_launches.push_back(t);
+}
+void timing_events(int id, hipEvent_t *start, hipEvent_t *stop) {
+    std::lock_guard<std::mutex> lk(g_tmu);
+    TimedLaunch t{id, get_event(), get_event()};
+    *start = t.a;
+    *stop = t.b;
     g_launches.push_back(t);
 }
 void timing_end(hipStream_t st) {

@@ -397,7 +397,6 @@ __global__ __launch_bounds__(BG_WAVES * 64) void bias_grad_kernel(const T *__res
 template <typename T, bool A_KS, bool B_KS, bool WG, int BM, int BN, int EPI>
 static int launch_gemm(GemmArgs g, int tiles, hipStream_t st, int kid) {
     if (tiles <= 0) return 0;
-    ScopedTiming timing(kid, st);
     g.n_blocks = tiles;
     const int grid = (tiles + 7) & ~7;
     const size_t lds = 2 * (size_t)(BM + BN) * 128;
@@ -407,7 +406,7 @@ static int launch_gemm(GemmArgs g, int tiles, hipStream_t st, int kid) {
         MOLE_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         attr_done = true;
     }
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(GEMM_THREADS), lds, st, g);
+    timed_launch(kid, kern, dim3(grid), dim3(GEMM_THREADS), (unsigned)lds, st, g);
     MOLE_LAUNCH_CHECK();
     return 0;
 }

@@ -750,7 +750,6 @@ template <int TMB, int WM, bool N_KS, bool WG, int EPI>
 static int launch256(GemmArgs g, int tiles, hipStream_t st, int kid) {
     typedef Tile<TMB, WM> TL;
     if (tiles <= 0) return 0;
-    ScopedTiming timing(kid, st);
     g.n_blocks = tiles;
     const int grid = (tiles + 7) & ~7;
     auto kern = gemm256_kernel<TMB, WM, N_KS, WG, EPI>;
@@ -759,7 +758,7 @@ static int launch256(GemmArgs g, int tiles, hipStream_t st, int kid) {
         MOLE_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, TL::LDS_BYTES));
         attr_done = true;
     }
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(TL::THREADS), TL::LDS_BYTES, st, g);
+    timed_launch(kid, kern, dim3(grid), dim3(TL::THREADS), TL::LDS_BYTES, st, g);
     MOLE_LAUNCH_CHECK();
     return 0;
 }

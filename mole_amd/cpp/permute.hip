@@ -795,13 +795,14 @@ static int check_perm(const char *fn, int dtype, int S, int M, int k) {
 static bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
 // the kernels above for the smallest K in {1, 2, 4, 8, 16} that holds k
-#define PM_LAUNCH_K(KERNEL, T, ...)                                                                                   \
-    do {                                                                                                              \
-        if (k <= 1) hipLaunchKernelGGL((KERNEL<T, 1>), grid, dim3(PM_THREADS), 0, (hipStream_t)stream, __VA_ARGS__);       \
-        else if (k <= 2) hipLaunchKernelGGL((KERNEL<T, 2>), grid, dim3(PM_THREADS), 0, (hipStream_t)stream, __VA_ARGS__);  \
-        else if (k <= 4) hipLaunchKernelGGL((KERNEL<T, 4>), grid, dim3(PM_THREADS), 0, (hipStream_t)stream, __VA_ARGS__);  \
-        else if (k <= 8) hipLaunchKernelGGL((KERNEL<T, 8>), grid, dim3(PM_THREADS), 0, (hipStream_t)stream, __VA_ARGS__);  \
-        else hipLaunchKernelGGL((KERNEL<T, 16>), grid, dim3(PM_THREADS), 0, (hipStream_t)stream, __VA_ARGS__);             \
+#define PM_LAUNCH_K(KID, KERNEL, T, ...)                                                                         \
+    do {                                                                                                         \
+        const dim3 blk_(PM_THREADS);                                                                             \
+        if (k <= 1) timed_launch(KID, KERNEL<T, 1>, grid, blk_, 0, (hipStream_t)stream, __VA_ARGS__);            \
+        else if (k <= 2) timed_launch(KID, KERNEL<T, 2>, grid, blk_, 0, (hipStream_t)stream, __VA_ARGS__);       \
+        else if (k <= 4) timed_launch(KID, KERNEL<T, 4>, grid, blk_, 0, (hipStream_t)stream, __VA_ARGS__);       \
+        else if (k <= 8) timed_launch(KID, KERNEL<T, 8>, grid, blk_, 0, (hipStream_t)stream, __VA_ARGS__);       \
+        else timed_launch(KID, KERNEL<T, 16>, grid, blk_, 0, (hipStream_t)stream, __VA_ARGS__);                  \
     } while (0)
 
 }  // namespace mole
@@ -814,11 +815,10 @@ extern "C" int mole_dispatch_fwd(const void *x, int dtype, const int32_t *row, i
     if (S == 0) return 0;
     MOLE_REQUIRE(x && row && xd && aligned16(x) && aligned16(xd), "mole_dispatch_fwd: null or misaligned pointer");
     const dim3 grid(ceil_div(S, PM_THREADS / WAVE));
-    ScopedTiming timing(MOLE_K_DISPATCH_FWD, (hipStream_t)stream);
     if (dtype == MOLE_BF16)
-        PM_LAUNCH_K(dispatch_fwd_kernel, bf16_t, (const bf16_t *)x, row, S, M, k, (bf16_t *)xd);
+        PM_LAUNCH_K(MOLE_K_DISPATCH_FWD, dispatch_fwd_kernel, bf16_t, (const bf16_t *)x, row, S, M, k, (bf16_t *)xd);
     else
-        PM_LAUNCH_K(dispatch_fwd_kernel, float, (const float *)x, row, S, M, k, (float *)xd);
+        PM_LAUNCH_K(MOLE_K_DISPATCH_FWD, dispatch_fwd_kernel, float, (const float *)x, row, S, M, k, (float *)xd);
     MOLE_LAUNCH_CHECK();
     return 0;
 }
@@ -831,19 +831,18 @@ extern "C" int mole_dispatch_bwd(const void *dxd, int dtype, const int32_t *row,
     MOLE_REQUIRE(dxd && row && dx && aligned16(dxd) && aligned16(dx), "mole_dispatch_bwd: null or misaligned pointer");
     MOLE_REQUIRE(dlogits == nullptr || (wg != nullptr && E >= 1 && aligned16(wg) && M % 4 == 0),
                  "mole_dispatch_bwd: dlogits given without a valid wg/E");
-    ScopedTiming timing(MOLE_K_DISPATCH_BWD, (hipStream_t)stream);
     MOLE_REQUIRE(dx_add == nullptr || aligned16(dx_add), "mole_dispatch_bwd: misaligned dx_add");
     if (dlogits != nullptr && dx_add == nullptr && E <= 32 && M % DM_COLS == 0 && dtype == MOLE_BF16) {
         const dim3 grid(ceil_div(S, DM_TOKENS), ceil_div(M, 8 * DM_COLS));
-        hipLaunchKernelGGL(dispatch_bwd_gate_mfma_kernel, grid, dim3(512), 0, (hipStream_t)stream, (const bf16_t *)dxd, row,
-                           S, M, k, dlogits, wg, E, (bf16_t *)dx);
+        timed_launch(MOLE_K_DISPATCH_BWD, dispatch_bwd_gate_mfma_kernel, grid, dim3(512), 0, (hipStream_t)stream,
+                     (const bf16_t *)dxd, row, S, M, k, dlogits, wg, E, (bf16_t *)dx);
         MOLE_LAUNCH_CHECK();
         return 0;
     }
     if (dlogits != nullptr && dx_add == nullptr && E <= 32 && M % 4 == 0) {
         const dim3 grid(ceil_div(S, DB_TOKENS), ceil_div(M, 1024));
         hipStream_t st = (hipStream_t)stream;
-#define MOLE_DB(T, EB) hipLaunchKernelGGL((dispatch_bwd_gate_kernel<T, EB>), grid, dim3(256), 0, st, (const T *)dxd, row, S, M, k, dlogits, wg, E, (T *)dx)
+#define MOLE_DB(T, EB) timed_launch(MOLE_K_DISPATCH_BWD, dispatch_bwd_gate_kernel<T, EB>, grid, dim3(256), 0, st, (const T *)dxd, row, S, M, k, dlogits, wg, E, (T *)dx)
         if (dtype == MOLE_BF16) {
             if (E <= 8) MOLE_DB(bf16_t, 8); else if (E <= 16) MOLE_DB(bf16_t, 16); else MOLE_DB(bf16_t, 32);
         } else {
@@ -855,9 +854,9 @@ extern "C" int mole_dispatch_bwd(const void *dxd, int dtype, const int32_t *row,
     }
     const dim3 grid(ceil_div(S, PM_THREADS / WAVE));
     if (dtype == MOLE_BF16)
-        PM_LAUNCH_K(dispatch_bwd_kernel, bf16_t, (const bf16_t *)dxd, row, S, M, k, dlogits, wg, E, (const bf16_t *)dx_add, (bf16_t *)dx);
+        PM_LAUNCH_K(MOLE_K_DISPATCH_BWD, dispatch_bwd_kernel, bf16_t, (const bf16_t *)dxd, row, S, M, k, dlogits, wg, E, (const bf16_t *)dx_add, (bf16_t *)dx);
     else
-        PM_LAUNCH_K(dispatch_bwd_kernel, float, (const float *)dxd, row, S, M, k, dlogits, wg, E, (const float *)dx_add, (float *)dx);
+        PM_LAUNCH_K(MOLE_K_DISPATCH_BWD, dispatch_bwd_kernel, float, (const float *)dxd, row, S, M, k, dlogits, wg, E, (const float *)dx_add, (float *)dx);
     MOLE_LAUNCH_CHECK();
     return 0;
 }
@@ -927,11 +926,10 @@ extern "C" int mole_combine_fwd(const void *o, int dtype, const int32_t *row, co
     if (S == 0) return 0;
     MOLE_REQUIRE(o && row && gates && y && aligned16(o) && aligned16(y), "mole_combine_fwd: null or misaligned pointer");
     const dim3 grid(ceil_div(S, PM_THREADS / WAVE));
-    ScopedTiming timing(MOLE_K_COMBINE_FWD, (hipStream_t)stream);
     if (dtype == MOLE_BF16)
-        PM_LAUNCH_K(combine_fwd_kernel, bf16_t, (const bf16_t *)o, row, gates, S, M, k, (bf16_t *)y);
+        PM_LAUNCH_K(MOLE_K_COMBINE_FWD, combine_fwd_kernel, bf16_t, (const bf16_t *)o, row, gates, S, M, k, (bf16_t *)y);
     else
-        PM_LAUNCH_K(combine_fwd_kernel, float, (const float *)o, row, gates, S, M, k, (float *)y);
+        PM_LAUNCH_K(MOLE_K_COMBINE_FWD, combine_fwd_kernel, float, (const float *)o, row, gates, S, M, k, (float *)y);
     MOLE_LAUNCH_CHECK();
     return 0;
 }
@@ -943,11 +941,10 @@ extern "C" int mole_combine_bwd(const void *dy, const void *o, int dtype, const 
     MOLE_REQUIRE(dy && o && row && gates && d_o && dgates && aligned16(dy) && aligned16(o) && aligned16(d_o),
                  "mole_combine_bwd: null or misaligned pointer");
     const dim3 grid(ceil_div(S, PM_THREADS / WAVE));
-    ScopedTiming timing(MOLE_K_COMBINE_BWD, (hipStream_t)stream);
     if (dtype == MOLE_BF16)
-        PM_LAUNCH_K(combine_bwd_kernel, bf16_t, (const bf16_t *)dy, (const bf16_t *)o, row, gates, S, M, k, (bf16_t *)d_o, dgates);
+        PM_LAUNCH_K(MOLE_K_COMBINE_BWD, combine_bwd_kernel, bf16_t, (const bf16_t *)dy, (const bf16_t *)o, row, gates, S, M, k, (bf16_t *)d_o, dgates);
     else
-        PM_LAUNCH_K(combine_bwd_kernel, float, (const float *)dy, (const float *)o, row, gates, S, M, k, (float *)d_o, dgates);
+        PM_LAUNCH_K(MOLE_K_COMBINE_BWD, combine_bwd_kernel, float, (const float *)dy, (const float *)o, row, gates, S, M, k, (float *)d_o, dgates);
     MOLE_LAUNCH_CHECK();
     return 0;
 }

@@ -721,12 +721,11 @@ extern "C" int mole_gate_fwd(const void *x, int dtype, const float *wg, const fl
     const int eg = ceil_div(E, 16);
     // small gates: 32 tokens per block (Wg, which every block reads in full, is then read half as often)
     const dim3 grid(ceil_div(S, eg <= 2 ? 32 : 16));
-    ScopedTiming timing(MOLE_K_GATE_FWD, st);
-    if (eg == 1) hipLaunchKernelGGL((gate_fwd_kernel<1, 8, 2>), grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores);
-    else if (eg == 2) hipLaunchKernelGGL((gate_fwd_kernel<2, 4, 2>), grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores);
-    else if (eg <= 4) hipLaunchKernelGGL((gate_fwd_kernel<4, 4, 1>), grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores);
-    else if (eg <= 8) hipLaunchKernelGGL((gate_fwd_kernel<8, 4, 1>), grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores);
-    else hipLaunchKernelGGL((gate_fwd_kernel<16, 2, 1>), grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores);
+    if (eg == 1) timed_launch(MOLE_K_GATE_FWD, gate_fwd_kernel<1, 8, 2>, grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores);
+    else if (eg == 2) timed_launch(MOLE_K_GATE_FWD, gate_fwd_kernel<2, 4, 2>, grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores);
+    else if (eg <= 4) timed_launch(MOLE_K_GATE_FWD, gate_fwd_kernel<4, 4, 1>, grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores);
+    else if (eg <= 8) timed_launch(MOLE_K_GATE_FWD, gate_fwd_kernel<8, 4, 1>, grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores);
+    else timed_launch(MOLE_K_GATE_FWD, gate_fwd_kernel<16, 2, 1>, grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores);
     MOLE_LAUNCH_CHECK();
     return 0;
 }
