@@ -12,7 +12,10 @@ pytestmark = pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("ragged", [True, False])
 @pytest.mark.parametrize("S,E,k,cf,M", [(1, 2, 1, 1.0, 8), (300, 8, 2, 1.0, 64), (1000, 16, 1, 0.5, 520),
-                                        (513, 4, 4, 0.0, 1024), (200, 32, 8, 0.0, 2048), (300, 64, 4, 0.0, 256)])
+                                        (513, 4, 4, 0.0, 1024), (200, 32, 8, 0.0, 2048), (300, 64, 4, 0.0, 256),
+                                        # top-k values between the kernels' compiled bounds (1, 2, 4, 8, 16), with drops
+                                        (257, 8, 3, 0.5, 72), (129, 16, 5, 1.0, 264), (65, 32, 16, 0.0, 128),
+                                        (40, 16, 16, 0.5, 1032), (90, 12, 7, 0.3, 2056)])
 def test_permutes_match_oracle(S, E, k, cf, M, ragged, dtype):
     from mole_amd import hip_ops as H, _lib as L
     print(f"permute S={S} E={E} k={k} cf={cf} M={M} ragged={ragged} {dtype}", flush=True)
