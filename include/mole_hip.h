@@ -151,6 +151,9 @@ int mole_route(const float *scores, int S, int E, int k, double capacity_factor,
  *   zero_pad_rows: zero the rows of a [total_rows, M] buffer that no kept pair owns
  *                  (rows offsets[e]+kept_rows[e] .. offsets[e+1]), which the reference's zeroed
  *                  [E,C,M] buffers contain.
+ * The expert-contiguous buffers (xd, dxd, o, d_o) must hold at least one row even when every pair was
+ * dropped: the gathers read row 0 in place of a dropped pair's row and discard what they read.
+ * The kernels are compiled for k <= 1, 2, 4, 8 and 16 and run the smallest that holds k.
  * ------------------------------------------------------------------------------------------ */
 int mole_dispatch_fwd(const void *x, int dtype, const int32_t *row, int S, int M, int k, void *xd,
                       mole_stream_t stream);

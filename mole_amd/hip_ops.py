@@ -160,6 +160,8 @@ def dispatch_bwd(dxd: torch.Tensor, row: torch.Tensor, dlogits: Optional[torch.T
     _dev(dxd), _dev(row)
     k, S = row.shape
     M = dxd.shape[-1]
+    if dxd.numel() == 0:         # every pair was dropped: the kernel still wants one (unused) row to read
+        dxd = torch.zeros(1, M, dtype=dxd.dtype, device=dxd.device)
     dx = torch.empty(S, M, dtype=dxd.dtype, device=dxd.device)
     E = 0
     dx_add = None
