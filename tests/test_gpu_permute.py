@@ -101,3 +101,35 @@ def test_dispatch_bwd_with_gate_bf16_wide_rows(S, E, k, M, cf):
     assert rel_err(got, want) < tol(torch.bfloat16)
     tight = O.fast_encode_bwd(dxd[:total].float(), c, True) + dlog.bfloat16().float() @ wg.bfloat16().float()
     assert rel_err(got, tight) < 6e-3          # what is left is the output's own rounding to bf16
+
+
+def test_kernel_timing_counts_launches_and_leaves_results_alone():
+    """The optional per-kernel timing (events attached to the launches): counts one launch per call and id,
+    reports a positive duration, and the timed launches give the same bits as the untimed ones."""
+    from mole_amd import hip_ops as H, _lib as L
+    S, E, k, M = 700, 8, 2, 256
+    print("kernel timing", flush=True)
+    scores = zipf_scores(S, E, seed=3).cuda()
+    x = torch.randn(S, M, generator=torch.Generator().manual_seed(1)).bfloat16().cuda()
+
+    def run():
+        r = H.route(scores, k, 1.0)
+        xd = H.dispatch_fwd(x, r.row, S * k)
+        total = int(r.offsets[-1])                    # rows past the kept ones are never written
+        return xd[:total], H.combine_fwd(xd, r.row, r.gates), r.row
+
+    plain = [t.clone() for t in run()]
+    L.kernel_timing_read()                                              # forget whatever an earlier test left
+    L.kernel_timing_enable(True)
+    try:
+        timed = [[t.clone() for t in run()] for _ in range(3)]
+        stats = L.kernel_timing_read()
+    finally:
+        L.kernel_timing_enable(False)
+    for name in ("route", "dispatch_fwd", "combine_fwd"):
+        count, ms = stats[name]
+        assert count == 3 and 0.0 < ms < 50.0, (name, count, ms)
+    assert stats["combine_bwd"][0] == 0
+    for rep in timed:
+        assert all(torch.equal(a, b) for a, b in zip(rep, plain))
+    assert all(c == 0 for c, _ in L.kernel_timing_read().values())      # a read forgets what it returned
