@@ -183,3 +183,51 @@ def test_ffn_benchmark_size_against_fp32_products():
     # bias gradient of the second linear for every expert: plain column sums of go
     want_b2 = torch.stack([go[int(off[e]):int(off[e + 1])].float().sum(0) for e in range(E)])
     assert rel_err(g_b2, want_b2) < t
+
+
+def test_ffn_imbalanced_full_size_against_fp32_products():
+    """The imbalanced configuration at its real shape (64 experts of 2048 -> 8192 -> 2048 in bf16, 16384 kept rows,
+    expert loads from a Zipf-biased top-2 routing: a handful of rows up to well over a thousand): the lightest, a
+    middle and the heaviest expert against fp32 torch products of the same rounded operands, forward and backward."""
+    from mole_amd import hip_ops as H, _lib as L
+    from tests.util import zipf_scores
+    S, E, k, M, Fd = 8192, 64, 2, 2048, 8192
+    r = H.route(zipf_scores(S, E, seed=11).cuda(), k, 0.0)
+    loads = r.kept_rows.cpu()
+    off = r.offsets.cpu()
+    R = int(off[-1])
+    assert R == S * k
+    order = torch.argsort(loads)
+    picks = [int(order[0]), int(order[E // 2]), int(order[-1])]
+    print(f"ffn imbalanced full size: loads min {int(loads.min())} median {int(loads.median())} max {int(loads.max())}, "
+          f"experts {picks}", flush=True)
+    dev, dt = "cuda", torch.bfloat16
+    gd = torch.Generator(device=dev).manual_seed(12)
+    rnd = lambda *s, sc=1.0: (torch.randn(*s, generator=gd, device=dev) * sc).to(dt)
+    xd, go = rnd(R, M), rnd(R, M, sc=0.02)
+    w1, b1, w2, b2 = rnd(E, Fd, M, sc=0.02), rnd(E, Fd, sc=0.02), rnd(E, Fd, M, sc=0.02), rnd(E, M, sc=0.02)
+    out, h, a = H.ffn_fwd(xd, r.offsets, r.kept_rows, w1, b1, w2, b2)
+    g_w1, g_b1, g_w2, g_b2 = torch.empty_like(w1), torch.empty_like(b1), torch.empty_like(w2), torch.empty_like(b2)
+    gx = H.ffn_bwd(go, xd, h, a, r.offsets, r.kept_rows, w1, w2, g_w1, g_b1, g_w2, g_b2, True, False, L.GELU_BWD_TANH)
+    torch.cuda.synchronize()
+    t = tol(dt)
+    c = 0.7978845608028654
+    for e in picks:
+        lo, hi = int(off[e]), int(off[e + 1])
+        if hi == lo:
+            assert float(g_w1[e].float().abs().max()) == 0.0 and float(g_w2[e].float().abs().max()) == 0.0
+            continue
+        x32, go32 = xd[lo:hi].float(), go[lo:hi].float()
+        h32 = x32 @ w1[e].float().t() + b1[e].float()
+        assert rel_err(h[lo:hi], h32) < t
+        assert rel_err(a[lo:hi], torch.nn.functional.gelu(h32)) < t
+        assert rel_err(out[lo:hi], torch.nn.functional.gelu(h32) @ w2[e].float() + b2[e].float()) < t
+        hs = h[lo:hi].float()                      # the derivative the reference compiles (MOLE/cpp/gelu.cu:3-14)
+        th = torch.tanh(c * (hs + 0.044715 * hs ** 3))
+        dg = 0.5 * (1 + th) + 0.5 * hs * c * (1 - th * th) * (1 + 3 * 0.044715 * hs * hs)
+        t32 = (go32 @ w2[e].float().t()) * dg
+        assert rel_err(g_w2[e], a[lo:hi].float().t() @ go32) < t
+        assert rel_err(g_w1[e], t32.t() @ x32) < t
+        assert rel_err(gx[lo:hi], t32 @ w1[e].float()) < t
+        assert rel_err(g_b1[e], t32.sum(0)) < t
+        assert rel_err(g_b2[e], go32.sum(0)) < t
