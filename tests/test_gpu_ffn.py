@@ -231,3 +231,42 @@ def test_ffn_imbalanced_full_size_against_fp32_products():
         assert rel_err(gx[lo:hi], t32 @ w1[e].float()) < t
         assert rel_err(g_b1[e], t32.sum(0)) < t
         assert rel_err(g_b2[e], go32.sum(0)) < t
+
+
+def test_ffn_fine_grained_full_size_against_fp32_products():
+    """The fine-grained configuration at its real shape (256 experts of 2048 -> 1024 -> 2048 in bf16, top-8 of
+    32768 tokens: 262144 kept rows, about a thousand per expert, more than 16 rounds of tiles per launch): three
+    experts against fp32 torch products of the same rounded operands, forward and backward (exact GELU')."""
+    from mole_amd import hip_ops as H, _lib as L
+    S, E, k, M, Fd = 32768, 256, 8, 2048, 1024
+    dev, dt = "cuda", torch.bfloat16
+    gd = torch.Generator(device=dev).manual_seed(21)
+    scores = torch.softmax(torch.randn(S, E, generator=gd, device=dev), -1)
+    r = H.route(scores, k, 0.0)
+    off = r.offsets.cpu()
+    R = int(off[-1])
+    assert R == S * k
+    print(f"ffn fine-grained full size: loads {int(r.kept_rows.min())}..{int(r.kept_rows.max())}", flush=True)
+    rnd = lambda *s, sc=1.0: (torch.randn(*s, generator=gd, device=dev) * sc).to(dt)
+    xd, go = rnd(R, M), rnd(R, M, sc=0.02)
+    w1, b1, w2, b2 = rnd(E, Fd, M, sc=0.02), rnd(E, Fd, sc=0.02), rnd(E, Fd, M, sc=0.02), rnd(E, M, sc=0.02)
+    out, h, a = H.ffn_fwd(xd, r.offsets, r.kept_rows, w1, b1, w2, b2)
+    g_w1, g_b1, g_w2, g_b2 = torch.empty_like(w1), torch.empty_like(b1), torch.empty_like(w2), torch.empty_like(b2)
+    gx = H.ffn_bwd(go, xd, h, a, r.offsets, r.kept_rows, w1, w2, g_w1, g_b1, g_w2, g_b2, True, False, L.GELU_BWD_EXACT)
+    torch.cuda.synchronize()
+    t = tol(dt)
+    for e in (0, 131, 255):
+        lo, hi = int(off[e]), int(off[e + 1])
+        x32, go32 = xd[lo:hi].float(), go[lo:hi].float()
+        h32 = x32 @ w1[e].float().t() + b1[e].float()
+        assert rel_err(h[lo:hi], h32) < t
+        assert rel_err(out[lo:hi], torch.nn.functional.gelu(h32) @ w2[e].float() + b2[e].float()) < t
+        hs = h[lo:hi].float()
+        hs.requires_grad_(True)
+        torch.nn.functional.gelu(hs).backward(go32 @ w2[e].float().t())
+        t32 = hs.grad
+        assert rel_err(g_w2[e], a[lo:hi].float().t() @ go32) < t
+        assert rel_err(g_w1[e], t32.t() @ x32) < t
+        assert rel_err(gx[lo:hi], t32 @ w1[e].float()) < t
+        assert rel_err(g_b1[e], t32.sum(0)) < t
+        assert rel_err(g_b2[e], go32.sum(0)) < t
