@@ -423,22 +423,20 @@ __device__ __forceinline__ void epilogue(const GemmArgs &g, f32x16 (&acc)[Tile<T
         return (row & 16) ? make_uint4(v.z, v.w, v.x, v.y) : v;
     };
     // slab -> global: rows [0, live) of the slab, 128 bytes each
-    // stream_out: a non-temporal store, for outputs that nothing reads soon - the pre-activation h, which only
-    // the GELU' product reads, five launches later, and the weight gradients, which wait for the optimizer - so
-    // that they do not push the operands of the next products (a, d_o, t, the weights) out of the L2 and the
-    // last-level cache: measured at 16 experts of 1024 x 4096 over 16384 rows, -6 us on h = xd.w1^T and -3 us on
-    // the product that reads a after it; -6 us on g_w2, -6 us on the GELU' product after it.
-    auto flush = [&](bf16_t *dst, bool stream_out = false) __attribute__((always_inline)) {
+    // Results leave with non-temporal stores.  A launch writes 34-270 MB that no block of the same launch reads,
+    // and ordinary stores let that push the operand panels of the running K loops out of the L2 and the
+    // last-level cache.  Measured at 16 experts of 1024 x 4096 over 16384 rows (same-box A/B): h and a of the
+    // first product -11 us, the weight gradients -6 us and the GELU' product that follows them -6 us, t of the
+    // GELU' product -4 us; the next launch reads what it needs from HBM at no loss (it is MFMA-bound).
+    auto flush = [&](bf16_t *dst) __attribute__((always_inline)) {
         typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 #pragma unroll
         for (int it = 0; it < TMC * 4; ++it) {
             const int row = it * 8 + jr;
             const uint4 v = fix16(*reinterpret_cast<const uint4 *>(slab_at(row, jc, (row >> 4) & 1)), row);
-            if (row < live && col_ok) {
-                uint4 *p = reinterpret_cast<uint4 *>(dst + (crow0 + m0 + row) * g.ldc + nw0 + jc * 8);
-                if (stream_out) __builtin_nontemporal_store(u32x4{v.x, v.y, v.z, v.w}, reinterpret_cast<u32x4 *>(p));
-                else *p = v;
-            }
+            if (row < live && col_ok)
+                __builtin_nontemporal_store(u32x4{v.x, v.y, v.z, v.w},
+                                            reinterpret_cast<u32x4 *>(dst + (crow0 + m0 + row) * g.ldc + nw0 + jc * 8));
         }
     };
     // global -> slab, eight rows' loads in flight at a time.  Every load is issued, from an address clamped
@@ -536,7 +534,7 @@ __device__ __forceinline__ void epilogue(const GemmArgs &g, f32x16 (&acc)[Tile<T
                 }
             }
         }
-        flush(pass == 0 ? Cb : (bf16_t *)g.C2, (EPI == EPI_BIAS_GELU && pass == 0) || EPI == EPI_WGRAD);
+        flush(pass == 0 ? Cb : (bf16_t *)g.C2);
     }
 }
 
