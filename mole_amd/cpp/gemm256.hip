@@ -423,20 +423,25 @@ __device__ __forceinline__ void epilogue(const GemmArgs &g, f32x16 (&acc)[Tile<T
         return (row & 16) ? make_uint4(v.z, v.w, v.x, v.y) : v;
     };
     // slab -> global: rows [0, live) of the slab, 128 bytes each
-    // Results leave with non-temporal stores.  A launch writes 34-270 MB that no block of the same launch reads,
-    // and ordinary stores let that push the operand panels of the running K loops out of the L2 and the
-    // last-level cache.  Measured at 16 experts of 1024 x 4096 over 16384 rows (same-box A/B): h and a of the
-    // first product -11 us, the weight gradients -6 us and the GELU' product that follows them -6 us, t of the
-    // GELU' product -4 us; the next launch reads what it needs from HBM at no loss (it is MFMA-bound).
+    // The large results - h, a, t and the weight gradients, 134-270 MB a launch, which no block of the same
+    // launch reads - leave with non-temporal stores: ordinary stores let them push the operand panels of the
+    // running K loops out of the L2 and the last-level cache.  Measured at 16 experts of 1024 x 4096 over 16384
+    // rows (same-box A/B): h and a of the first product -11 us, the weight gradients -6 us and the GELU' product
+    // that follows them -6 us, t of the GELU' product -4 us; the launches that read them later are MFMA-bound
+    // and take them from HBM at no loss.  The small results (out, gx: 34 MB) stay ordinary: the row permutes
+    // that read them next are memory-bound and lost more than the products gained.
+    constexpr bool STREAM_OUT = EPI == EPI_BIAS_GELU || EPI == EPI_DGELU || EPI == EPI_WGRAD;
     auto flush = [&](bf16_t *dst) __attribute__((always_inline)) {
         typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 #pragma unroll
         for (int it = 0; it < TMC * 4; ++it) {
             const int row = it * 8 + jr;
             const uint4 v = fix16(*reinterpret_cast<const uint4 *>(slab_at(row, jc, (row >> 4) & 1)), row);
-            if (row < live && col_ok)
-                __builtin_nontemporal_store(u32x4{v.x, v.y, v.z, v.w},
-                                            reinterpret_cast<u32x4 *>(dst + (crow0 + m0 + row) * g.ldc + nw0 + jc * 8));
+            if (row < live && col_ok) {
+                uint4 *p = reinterpret_cast<uint4 *>(dst + (crow0 + m0 + row) * g.ldc + nw0 + jc * 8);
+                if constexpr (STREAM_OUT) __builtin_nontemporal_store(u32x4{v.x, v.y, v.z, v.w}, reinterpret_cast<u32x4 *>(p));
+                else *p = v;
+            }
         }
     };
     // global -> slab, eight rows' loads in flight at a time.  Every load is issued, from an address clamped
