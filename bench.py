@@ -32,8 +32,8 @@ PEAK_HBM_GBS = 8000.0
 # WRITE_SIZE runs of this script scaled by the same counters' readings for a copy of known size
 # (profiles/bench_c2_hbm_traffic.txt); other workloads have no counter run and report null
 MEASURED_TRAFFIC_BYTES = {
-    "c2": {"ffn_fwd1": 770.1e6, "ffn_fwd2": 355.9e6, "ffn_gw2": 545.5e6, "ffn_da": 755.4e6, "ffn_gw1": 545.5e6,
-           "ffn_gx": 378.9e6},
+    "c2": {"ffn_fwd1": 751.8e6, "ffn_fwd2": 383.9e6, "ffn_gw2": 546.7e6, "ffn_da": 741.5e6, "ffn_gw1": 546.7e6,
+           "ffn_gx": 385.0e6},
 }
 
 
