@@ -428,7 +428,7 @@ extern "C" int mole_route(const float *scores, int S, int E, int k, double capac
     MOLE_LAUNCH_CHECK();
 
     const int npairs = k * E;
-    const bool scan_in_finish = (long long)npairs * nb <= 16384;   // small enough for one block: saves a launch
+    const bool scan_in_finish = (long long)npairs * nb <= 8192;    // small enough for one block: saves a launch
     if (!scan_in_finish) {
         const int scan_blocks = ceil_div(npairs, 4);
         hipLaunchKernelGGL(route_scan_kernel, dim3(scan_blocks + COLSUM_SLICES * ceil_div(E, 256)), dim3(256), 0, st, hist,
