@@ -332,7 +332,17 @@ __global__ __launch_bounds__(FIN_THREADS) void route_finish_kernel(
         if (tid < groups * E && E <= FIN_THREADS) {
             const int e = tid % E, gq = tid / E;
             float me = 0.f;
-            for (int b = gq; b < nb; b += groups) me += colsum[(size_t)b * E + e];
+            for (int b0 = gq; b0 < nb; b0 += 8 * groups) {       // 8 loads in flight, added in block order
+                float t[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int b = b0 + u * groups;
+                    t[u] = load_or_zero(colsum + (size_t)min(b, nb - 1) * E + e, b < nb);
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u)
+                    if (b0 + u * groups < nb) me += t[u];
+            }
             s_fred[tid] = me;
         }
         __syncthreads();
