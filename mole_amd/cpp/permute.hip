@@ -181,15 +181,16 @@ __global__ __launch_bounds__(PM_THREADS) void dispatch_bwd_kernel(const T *__res
 }
 
 // dispatch backward with the gate's input gradient folded in, for small gates (E <= 32): a thread
-// owns 4 columns and keeps its 4 x E slice of Wg in registers; the block walks DB_TOKENS tokens, whose
+// owns 4 columns and keeps its 4 x E slice of Wg in registers; the block walks db_tokens tokens (8 or 32), whose
 // row indices and dlogits are block-uniform (scalar loads).  Larger gates use the kernel above.
-constexpr int DB_TOKENS = 32;
+constexpr int DB_TOKENS = 32;   // tokens per block when there are enough of them to fill the chip several times over
+constexpr int DB_TOKENS_FEW = 8;   // otherwise: more, shorter blocks (4096 x 512 fp32 tokens: 10.5 against 22 us)
 template <typename T, int EB>
 __global__ __launch_bounds__(256) void dispatch_bwd_gate_kernel(const T *__restrict__ dxd,
                                                                 const int32_t *__restrict__ row, int S, int M, int k,
                                                                 const float *__restrict__ dlogits,
                                                                 const float *__restrict__ wg, int E,
-                                                                T *__restrict__ dx) {
+                                                                T *__restrict__ dx, int db_tokens) {
     const int m = (blockIdx.y * 256 + threadIdx.x) * 4;
     if (m >= M) return;
     float w[EB][4];
@@ -198,7 +199,7 @@ __global__ __launch_bounds__(256) void dispatch_bwd_gate_kernel(const T *__restr
         const float4 v = e < E ? *reinterpret_cast<const float4 *>(wg + (size_t)e * M + m) : make_float4(0.f, 0.f, 0.f, 0.f);
         w[e][0] = v.x; w[e][1] = v.y; w[e][2] = v.z; w[e][3] = v.w;
     }
-    const int i0 = blockIdx.x * DB_TOKENS, i1 = min(i0 + DB_TOKENS, S);
+    const int i0 = blockIdx.x * db_tokens, i1 = min(i0 + db_tokens, S);
     // Eight tokens per batch; the first choice's row gathers of the next batch are in flight while the
     // current batch is finished: one token at a time, or one batch at a time, runs at the memory latency.
     constexpr int U = 8;
@@ -840,9 +841,10 @@ extern "C" int mole_dispatch_bwd(const void *dxd, int dtype, const int32_t *row,
         return 0;
     }
     if (dlogits != nullptr && dx_add == nullptr && E <= 32 && M % 4 == 0) {
-        const dim3 grid(ceil_div(S, DB_TOKENS), ceil_div(M, 1024));
+        const int db_tokens = (long)ceil_div(S, DB_TOKENS) * ceil_div(M, 1024) < 1024 ? DB_TOKENS_FEW : DB_TOKENS;
+        const dim3 grid(ceil_div(S, db_tokens), ceil_div(M, 1024));
         hipStream_t st = (hipStream_t)stream;
-#define MOLE_DB(T, EB) timed_launch(MOLE_K_DISPATCH_BWD, dispatch_bwd_gate_kernel<T, EB>, grid, dim3(256), 0, st, (const T *)dxd, row, S, M, k, dlogits, wg, E, (T *)dx)
+#define MOLE_DB(T, EB) timed_launch(MOLE_K_DISPATCH_BWD, dispatch_bwd_gate_kernel<T, EB>, grid, dim3(256), 0, st, (const T *)dxd, row, S, M, k, dlogits, wg, E, (T *)dx, db_tokens)
         if (dtype == MOLE_BF16) {
             if (E <= 8) MOLE_DB(bf16_t, 8); else if (E <= 16) MOLE_DB(bf16_t, 16); else MOLE_DB(bf16_t, 32);
         } else {
