@@ -89,11 +89,13 @@ int mole_kernel_timing_read(int n_ids, int *counts, float *ms_total);
  * ------------------------------------------------------------------------------------------ */
 int mole_softmax_fwd(const float *logits, const float *logit_bias, int S, int E, float *scores,
                      mole_stream_t stream);
-/* The whole of MOLETopk.forward (MOLE/utils/Ugate.py:11-14) in one kernel for bf16 tokens:
- * scores[S,E] = softmax(x[S,M] . wg[E,M]^T + logit_bias), wg fp32 (rounded to bf16 for the products, fp32
- * accumulation), logit_bias [E] or NULL.  Needs dtype == MOLE_BF16, M a multiple of 128, E <= 256; other
- * cases use mole_gemm_nt + mole_softmax_fwd.  Every block of 16 tokens reads all of wg, so beyond a few dozen
- * experts the two-kernel path is the faster one (the Python host side switches at E = 32). */
+/* The whole of MOLETopk.forward (MOLE/utils/Ugate.py:11-14) in one kernel:
+ * scores[S,E] = softmax(x[S,M] . wg[E,M]^T + logit_bias), wg fp32, logit_bias [E] or NULL.
+ * bf16 tokens: M a multiple of 128, E <= 256; wg is rounded to bf16 for the products, fp32 accumulation.  Every
+ * block of 16 tokens reads all of wg, so beyond a few dozen experts the two-kernel path is the faster one (the
+ * Python host side switches at E = 32).
+ * fp32 tokens: M a multiple of 4, E <= 32, x and wg 16-byte aligned; fp32 FMAs throughout.
+ * Other cases use mole_gemm_nt + mole_softmax_fwd. */
 int mole_gate_fwd(const void *x, int dtype, const float *wg, const float *logit_bias, int S, int E, int M,
                   float *scores, mole_stream_t stream);
 int mole_gate_bwd(const float *dgates, const float *scores, const int32_t *idx, int S, int E,

@@ -48,14 +48,16 @@ def softmax_fwd(logits: torch.Tensor, logit_bias: Optional[torch.Tensor] = None)
 
 def gate_fwd(x: torch.Tensor, wg: torch.Tensor, logit_bias: Optional[torch.Tensor] = None,
              fused: Optional[bool] = None) -> torch.Tensor:
-    """scores [S,E] fp32 = softmax(x @ wg.T + logit_bias): one fused kernel for bf16 tokens and small gates
-    (M % 128 == 0, E <= 32: a block of 16 tokens re-reads all of wg, which only pays while wg is small), the NT
-    GEMM followed by the softmax kernel otherwise.  fused=True asks for the one-kernel path at any E <= 256."""
+    """scores [S,E] fp32 = softmax(x @ wg.T + logit_bias): one fused kernel for small gates (E <= 32; bf16 tokens
+    with M % 128 == 0, where a block of 16 tokens re-reads all of wg, which only pays while wg is small, or fp32
+    tokens with M % 4 == 0), the NT GEMM followed by the softmax kernel otherwise.  fused=True asks for the
+    one-kernel path where the kernel allows it (bf16: any E <= 256)."""
     _dev(x), _dev(wg)
     S, M = x.shape
     E = wg.shape[0]
     if fused is None:
-        fused = x.dtype == torch.bfloat16 and wg.dtype == torch.float32 and M % 128 == 0 and E <= 32
+        fused = wg.dtype == torch.float32 and E <= 32 and (
+            (x.dtype == torch.bfloat16 and M % 128 == 0) or (x.dtype == torch.float32 and M % 4 == 0))
     if fused:
         scores = torch.empty(S, E, dtype=torch.float32, device=x.device)
         L.check(L.lib().mole_gate_fwd(L.ptr(x), L.dtype_code(x.dtype), L.ptr(wg), L.ptr(logit_bias), S, E, M, L.ptr(scores),

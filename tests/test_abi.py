@@ -69,7 +69,8 @@ def test_every_entry_point_rejects_bad_arguments_on_the_host():
     ok = P(4096)
     cases = [
         ("mole_softmax_fwd", lambda: lib.mole_softmax_fwd(None, None, 10, 0, None, None)),
-        ("mole_gate_fwd", lambda: lib.mole_gate_fwd(ok, L.MOLE_F32, ok, None, 10, 8, 128, ok, None)),
+        ("mole_gate_fwd", lambda: lib.mole_gate_fwd(ok, L.MOLE_F32, ok, None, 10, 64, 128, ok, None)),      # fp32: E <= 32
+        ("mole_gate_fwd", lambda: lib.mole_gate_fwd(bad16, L.MOLE_F32, ok, None, 10, 8, 128, ok, None)),    # fp32: alignment
         ("mole_gate_fwd", lambda: lib.mole_gate_fwd(ok, L.MOLE_BF16, ok, None, 10, 8, 100, ok, None)),
         ("mole_gate_bwd", lambda: lib.mole_gate_bwd(ok, ok, ok, 10, 4, 5, 1, 1, ok, None)),
         ("mole_gate_wgrad", lambda: lib.mole_gate_wgrad(ok, ok, L.MOLE_F32, 10, 64, 128, ok, ok, 1 << 30, None)),

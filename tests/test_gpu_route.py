@@ -120,6 +120,25 @@ def test_fused_gate_forward(S, E, M, bias):
     assert rel_err(got, unfused) < 1e-5
 
 
+@pytest.mark.parametrize("S,E,M,bias", [(4096, 8, 512, False), (777, 3, 260, True), (1000, 32, 1024, True),
+                                        (5, 17, 4, False), (300, 16, 2048, False)])
+def test_fused_gate_forward_fp32_tokens(S, E, M, bias):
+    """mole_gate_fwd for fp32 tokens and small gates (one wave per token, fp32 FMAs) against the oracle's gate and
+    against the GEMM + softmax path it replaces."""
+    from mole_amd import hip_ops as H
+    print(f"gate_fwd fp32 S={S} E={E} M={M} bias={bias}", flush=True)
+    g = torch.Generator().manual_seed(S + E)
+    x = torch.randn(S, M, generator=g)
+    wg = torch.randn(E, M, generator=g) * 0.05
+    b = torch.log(torch.arange(1, E + 1, dtype=torch.float32) ** -1.2) if bias else None
+    got = H.gate_fwd(x.cuda(), wg.cuda(), b.cuda() if bias else None).cpu()          # the fused kernel by default
+    assert got.shape == (S, E)
+    assert rel_err(got, O.gate_scores(x, wg, b)) < 1e-5
+    assert float((got.sum(-1) - 1).abs().max()) < 1e-5
+    unfused = H.gate_fwd(x.cuda(), wg.cuda(), b.cuda() if bias else None, fused=False).cpu()
+    assert rel_err(got, unfused) < 1e-5
+
+
 def test_route_random_sweep():
     """Sixty seeded random (S, E, k, capacity factor, alignment) combinations, both layouts, bit for bit."""
     rng = np.random.default_rng(2024)
