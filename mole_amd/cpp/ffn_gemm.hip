@@ -301,6 +301,17 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kernel(const GemmArgs g) {
         if constexpr (EPI == EPI_BIAS || EPI == EPI_BIAS_GELU) bias = to_f32(((const T *)g.bias)[(long)e * g.N + n]);
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) {
+            // GELU': the 16 pre-activations of this cell are fetched first, unconditionally (rows past the end read
+            // the expert's last row and are not used) - a load behind the row test below would be waited for
+            // before the next one is issued
+            float hv16[16];
+            if constexpr (EPI == EPI_DGELU) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int m = m0 + rowA0 + tm * 32 + 8 * (i >> 2) + 4 * h + (i & 3);
+                    hv16[i] = to_f32(((const T *)g.H)[(crow0 + min(m, m_ext - 1)) * g.ldc + n]);
+                }
+            }
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const int m = m0 + rowA0 + tm * 32 + 8 * (i >> 2) + 4 * h + (i & 3);
@@ -318,7 +329,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_kernel(const GemmArgs g) {
                     ((T *)Cb)[off] = from_f32<T>(v);
                     ((T *)g.C2)[off] = from_f32<T>(gelu_erf(v));
                 } else if constexpr (EPI == EPI_DGELU) {
-                    const float hv = to_f32(((const T *)g.H)[off]);
+                    const float hv = hv16[i];
                     const float d = g.gelu_bwd == MOLE_GELU_BWD_TANH ? d_gelu_tanh(hv) : d_gelu_exact(hv);
                     ((T *)Cb)[off] = from_f32<T>(v * d);
                 } else {  // EPI_WGRAD
