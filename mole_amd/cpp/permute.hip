@@ -289,6 +289,7 @@ constexpr int DM_COLS = 128;                  // columns per wave
 constexpr int DM_ROW = DM_COLS + 4;           // floats per token row of the LDS buffer: 4 rows apart = 16 banks apart
 typedef __bf16 perm_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float perm_f32x4 __attribute__((ext_vector_type(4)));
+template <bool E8>   // E8: E is a multiple of 8, a lane's 8 gradients are two 16-byte loads
 __global__ __launch_bounds__(512) void dispatch_bwd_gate_mfma_kernel(const bf16_t *__restrict__ dxd,
                                                                      const int32_t *__restrict__ row, int S, int M, int k,
                                                                      const float *__restrict__ dlogits,
@@ -364,8 +365,15 @@ __global__ __launch_bounds__(512) void dispatch_bwd_gate_mfma_kernel(const bf16_
         if (g0 + 16 < DM_TOKENS) gather(nxt, nxt_ok, tok0 + 16);
         // A fragment: dlogits[tok0 + r16][8 kq .. 8 kq + 7]
         float d[8];
+        if constexpr (E8) {
+            const float4 *dp = reinterpret_cast<const float4 *>(dlogits + (size_t)min(tok0 + r16, S - 1) * E + min(8 * kq, E - 8));
+            const float4 d0 = dp[0], d1 = dp[1];
+            d[0] = d0.x; d[1] = d0.y; d[2] = d0.z; d[3] = d0.w;
+            d[4] = d1.x; d[5] = d1.y; d[6] = d1.z; d[7] = d1.w;
+        } else {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) d[i] = dlogits[(size_t)min(tok0 + r16, S - 1) * E + min(8 * kq + i, E - 1)];
+            for (int i = 0; i < 8; ++i) d[i] = dlogits[(size_t)min(tok0 + r16, S - 1) * E + min(8 * kq + i, E - 1)];
+        }
 #pragma unroll
         for (int i = 0; i < 8; ++i)
             if (tok0 + r16 >= S || 8 * kq + i >= E) d[i] = 0.f;
@@ -835,8 +843,12 @@ extern "C" int mole_dispatch_bwd(const void *dxd, int dtype, const int32_t *row,
     MOLE_REQUIRE(dx_add == nullptr || aligned16(dx_add), "mole_dispatch_bwd: misaligned dx_add");
     if (dlogits != nullptr && dx_add == nullptr && E <= 32 && M % DM_COLS == 0 && dtype == MOLE_BF16) {
         const dim3 grid(ceil_div(S, DM_TOKENS), ceil_div(M, 8 * DM_COLS));
-        timed_launch(MOLE_K_DISPATCH_BWD, dispatch_bwd_gate_mfma_kernel, grid, dim3(512), 0, (hipStream_t)stream,
-                     (const bf16_t *)dxd, row, S, M, k, dlogits, wg, E, (bf16_t *)dx);
+        if (E % 8 == 0 && ((uintptr_t)dlogits & 15) == 0)
+            timed_launch(MOLE_K_DISPATCH_BWD, dispatch_bwd_gate_mfma_kernel<true>, grid, dim3(512), 0, (hipStream_t)stream,
+                         (const bf16_t *)dxd, row, S, M, k, dlogits, wg, E, (bf16_t *)dx);
+        else
+            timed_launch(MOLE_K_DISPATCH_BWD, dispatch_bwd_gate_mfma_kernel<false>, grid, dim3(512), 0, (hipStream_t)stream,
+                         (const bf16_t *)dxd, row, S, M, k, dlogits, wg, E, (bf16_t *)dx);
         MOLE_LAUNCH_CHECK();
         return 0;
     }

@@ -80,7 +80,8 @@ def test_permute_full_size_properties():
 
 
 @pytest.mark.parametrize("S,E,k,M,cf", [(100, 16, 1, 256, 1.0), (1000, 3, 2, 512, 0.0), (777, 32, 4, 1280, 0.5),
-                                        (16384, 16, 1, 1024, 1.25), (33, 20, 2, 256, 0.0)])
+                                        (16384, 16, 1, 1024, 1.25), (33, 20, 2, 256, 0.0),
+                                        (500, 24, 2, 384, 1.0), (64, 8, 1, 128, 1.0)])
 def test_dispatch_bwd_with_gate_bf16_wide_rows(S, E, k, M, cf):
     """The fused dispatch backward for bf16 rows of whole 256-column groups (the matrix-core variant): gather-sum
     of the kept rows plus dlogits @ Wg, against the oracle's gather and an fp32 product of the bf16-rounded
