@@ -305,10 +305,14 @@ __global__ __launch_bounds__(512) void dispatch_bwd_gate_mfma_kernel(const bf16_
     // the first-choice source rows of the 4 tokens this lane finishes in a group (tokens tok0 + 4 u + tsel)
     // (loads are unconditional, from clamped addresses, and what must not count is masked where it is used: a
     // load under a condition would make the compiler wait for all loads in flight at every such place)
+    // (the first-choice rows of the block's 64 tokens come with one load, lane l holding token l's, and are handed
+    // round between lanes: the gathers' addresses then wait for no load of their own)
+    static_assert(DM_TOKENS == WAVE, "one first-choice row per lane");
+    const int my_row = row[min((int)blockIdx.x * DM_TOKENS + lane, S - 1)];
     auto gather = [&](uint4 (&v)[4], uint32_t (&ok)[4], int tok0) __attribute__((always_inline)) {
         int r[4];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) r[u] = row[min(tok0 + 4 * u + tsel, S - 1)];
+        for (int u = 0; u < 4; ++u) r[u] = __shfl(my_row, (tok0 - (int)blockIdx.x * DM_TOKENS + 4 * u + tsel) & (WAVE - 1), WAVE);
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             ok[u] = (tok0 + 4 * u + tsel < S && r[u] >= 0) ? 0xffffffffu : 0u;
