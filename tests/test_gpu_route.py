@@ -101,7 +101,8 @@ def test_gate_wgrad(S, E, M, dtype):
 
 
 @pytest.mark.parametrize("S,E,M,bias", [(100, 16, 128, False), (1000, 8, 256, True), (513, 64, 384, False),
-                                        (300, 256, 1024, True), (64, 100, 128, True), (16384, 16, 1024, False)])
+                                        (300, 256, 1024, True), (64, 100, 128, True), (16384, 16, 1024, False),
+                                        (333, 12, 1280, True), (47, 16, 640, False)])
 def test_fused_gate_forward(S, E, M, bias):
     """mole_gate_fwd (bf16 tokens) against the oracle's gate on the same rounded operands, and against the
     unfused GEMM + softmax path it replaces."""
