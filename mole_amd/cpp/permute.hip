@@ -653,12 +653,24 @@ __global__ __launch_bounds__(256) void gate_wgrad_reduce_kernel(const float *__r
     const int o = threadIdx.x & 15, slice = threadIdx.x >> 4;
     const int idx = (blockIdx.x * 16 + o) * 4;
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (idx < EM) {
+    if (nblocks > 0) {
+        // eight partials per batch, loaded unconditionally from clamped addresses so that they are in flight
+        // together, and added in order; what lies past the slice is cleared by a bit mask
         const int per = (nblocks + 15) / 16;
         const int b1 = min(nblocks, (slice + 1) * per);
-        for (int b = slice * per; b < b1; ++b) {
-            const float4 v = *reinterpret_cast<const float4 *>(part + (size_t)b * EM + idx);
-            acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+        const float *src = part + (idx < EM ? idx : 0);
+        for (int b0 = slice * per; b0 < b1; b0 += 8) {
+            float4 v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const float4 *>(src + (size_t)min(b0 + u, nblocks - 1) * EM);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const uint32_t keep = b0 + u < b1 ? 0xffffffffu : 0u;
+                acc.x += __uint_as_float(__float_as_uint(v[u].x) & keep);
+                acc.y += __uint_as_float(__float_as_uint(v[u].y) & keep);
+                acc.z += __uint_as_float(__float_as_uint(v[u].z) & keep);
+                acc.w += __uint_as_float(__float_as_uint(v[u].w) & keep);
+            }
         }
     }
     s_acc[slice][o] = acc;
