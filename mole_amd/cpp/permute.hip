@@ -504,7 +504,7 @@ constexpr int GM_XROW = 72;                   // bf16 per token row of a wave's 
                                               // so that the 4 rows of a transposing read fall into distinct banks
 constexpr int GM_SUB = 128;                   // tokens whose dlogits are staged at a time
 typedef short perm_s16x4 __attribute__((ext_vector_type(4)));
-template <int EG>   // groups of 16 experts per block
+template <int EG, bool DL4>   // groups of 16 experts per block; DL4: E is a multiple of 4, dlogits come by 16-byte loads
 __global__ __launch_bounds__(256, 2) void gate_wgrad_mfma_kernel(const float *__restrict__ dlogits,
                                                               const bf16_t *__restrict__ x, int S, int E, int M,
                                                               int chunk, int nchunks, int nz, float *__restrict__ part) {
@@ -548,16 +548,24 @@ __global__ __launch_bounds__(256, 2) void gate_wgrad_mfma_kernel(const float *__
     // a thread's share of the dlogits of GM_SUB tokens: expert de of the block's group (expert fastest across
     // threads: the global reads are whole rows of dlogits), tokens dt0, dt0 + DL_TSTEP, ...; fetched into
     // registers one sub-chunk ahead, so the loads are in flight while the current sub-chunk is multiplied
-    constexpr int DL_W = 16 * EG, DL_N = GM_SUB * DL_W / 256, DL_TSTEP = 256 / DL_W;
-    const int de = threadIdx.x % DL_W, dt0 = threadIdx.x / DL_W;
-    float dl[DL_N];
+    // (DL4: four consecutive experts per thread and load, a quarter of the load instructions)
+    constexpr int DL_V = DL4 ? 4 : 1;
+    constexpr int DL_W = 16 * EG / DL_V, DL_N = GM_SUB * DL_W / 256, DL_TSTEP = 256 / DL_W;
+    const int de = (threadIdx.x % DL_W) * DL_V, dt0 = threadIdx.x / DL_W;
+    float dl[DL_N][DL_V];
     const bool dl_in = e0 + de < E;
-    const float *dl_col = dlogits + min(e0 + de, E - 1);
+    const float *dl_col = dlogits + min(e0 + de, E - DL_V);
     auto fetch_dl = [&](int sub0) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < DL_N; ++i) {
             const int t = sub0 + dt0 + DL_TSTEP * i;
-            dl[i] = dl_col[(size_t)(tok0 + min(t, ntok - 1)) * E];
+            const float *p = dl_col + (size_t)(tok0 + min(t, ntok - 1)) * E;
+            if constexpr (DL4) {
+                const float4 v = *reinterpret_cast<const float4 *>(p);
+                dl[i][0] = v.x; dl[i][1] = v.y; dl[i][2] = v.z; dl[i][3] = v.w;
+            } else {
+                dl[i][0] = *p;
+            }
         }
     };
     // the x tiles of a whole sub-chunk (GM_SUB / GM_KSTEP = 4 steps) are in flight at any time: a step's
@@ -573,10 +581,13 @@ __global__ __launch_bounds__(256, 2) void gate_wgrad_mfma_kernel(const float *__
 #pragma unroll
         for (int i = 0; i < DL_N; ++i) {
             const int t = dt0 + DL_TSTEP * i;
-            const float v = (sub0 + t < ntok && dl_in) ? dl[i] : 0.f;
-            const bf16_t hi = (bf16_t)v;
-            s_dl[0][t * DLROW + de] = hi;
-            s_dl[1][t * DLROW + de] = (bf16_t)(v - (float)hi);
+#pragma unroll
+            for (int c = 0; c < DL_V; ++c) {
+                const float v = (sub0 + t < ntok && dl_in) ? dl[i][c] : 0.f;
+                const bf16_t hi = (bf16_t)v;
+                s_dl[0][t * DLROW + de + c] = hi;
+                s_dl[1][t * DLROW + de + c] = (bf16_t)(v - (float)hi);
+            }
         }
         __syncthreads();
         fetch_dl(sub0 + GM_SUB);              // past the chunk's end: zeros
@@ -927,8 +938,12 @@ extern "C" int mole_gate_wgrad(const float *dlogits, const void *x, int dtype, i
         const int eg = E <= 16 ? 1 : (E <= 32 ? 2 : 4);
         const int nz = ceil_div(E, 16 * eg), nunits = nchunks * ceil_div(M, 256);
         const dim3 grid((unsigned)(ceil_div(nunits, 8) * 8 * nz));
-#define MOLE_GM(EG) hipLaunchKernelGGL((gate_wgrad_mfma_kernel<EG>), grid, dim3(256), 0, st, dlogits, (const bf16_t *)x, S, E, M, chunk, nchunks, nz, part)
-        if (eg == 1) MOLE_GM(1); else if (eg == 2) MOLE_GM(2); else MOLE_GM(4);
+#define MOLE_GM(EG, V) hipLaunchKernelGGL((gate_wgrad_mfma_kernel<EG, V>), grid, dim3(256), 0, st, dlogits, (const bf16_t *)x, S, E, M, chunk, nchunks, nz, part)
+        if (E % 4 == 0 && aligned16(dlogits)) {
+            if (eg == 1) MOLE_GM(1, true); else if (eg == 2) MOLE_GM(2, true); else MOLE_GM(4, true);
+        } else {
+            if (eg == 1) MOLE_GM(1, false); else if (eg == 2) MOLE_GM(2, false); else MOLE_GM(4, false);
+        }
 #undef MOLE_GM
         MOLE_LAUNCH_CHECK();
         hipLaunchKernelGGL(gate_wgrad_reduce_kernel, dim3(ceil_div(E * M, 64)), dim3(256), 0, st, part, nchunks, E * M, dwg);
