@@ -1,0 +1,7 @@
+"""Where the reference keeps its native extension.  The C ABI of the MI355X implementation is declared in
+mole_hip.h in this directory and built into mole_amd/cpp/libmole_hip.so; LIB_PATH names the built library."""
+import os
+
+from mole_amd._lib import LIB_PATH  # noqa: F401
+
+HEADER = os.path.join(os.path.dirname(os.path.abspath(__file__)), "mole_hip.h")

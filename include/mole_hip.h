@@ -85,9 +85,16 @@ int mole_kernel_timing_read(int n_ids, int *counts, float *ms_total);
  * logits [S,E] fp32 (x . Wg^T, produced by mole_gemm_nt or any GEMM); logit_bias [E] or NULL.
  * mole_gate_bwd replaces the autograd of the gate normalisation inside tutel's
  * extract_critical and, with through_softmax != 0, of the softmax as well: from dgates [k,S]
- * it produces d(scores) [S,E] (through_softmax == 0) or d(logits) [S,E].
+ * it produces d(scores) [S,E] (through_softmax == 0) or d(logits) [S,E].  counts0 [E] (the first
+ * choice's per-expert counts from mole_route) and d_l_aux [1] (device, the gradient arriving at l_aux) are
+ * given together or both NULL: with them d(scores)[i,e] also carries d_l_aux * E/S^2 * counts0[e], the
+ * gradient of tutel's gshard_loss, which the reference adds to its loss through autograd (MOLE/moe/layer.py:447).
  * ------------------------------------------------------------------------------------------ */
 int mole_softmax_fwd(const float *logits, const float *logit_bias, int S, int E, float *scores,
+                     mole_stream_t stream);
+/* dlogits = scores * (dscores - sum_e dscores scores): the softmax's backward alone, for the gate module used
+ * outside the fused layer (autograd runs it in the reference, MOLE/utils/Ugate.py:13). */
+int mole_softmax_bwd(const float *dscores, const float *scores, int S, int E, float *dlogits,
                      mole_stream_t stream);
 /* The whole of MOLETopk.forward (MOLE/utils/Ugate.py:11-14) in one kernel:
  * scores[S,E] = softmax(x[S,M] . wg[E,M]^T + logit_bias), wg fp32, logit_bias [E] or NULL.
@@ -99,7 +106,8 @@ int mole_softmax_fwd(const float *logits, const float *logit_bias, int S, int E,
 int mole_gate_fwd(const void *x, int dtype, const float *wg, const float *logit_bias, int S, int E, int M,
                   float *scores, mole_stream_t stream);
 int mole_gate_bwd(const float *dgates, const float *scores, const int32_t *idx, int S, int E,
-                  int k, int normalize_gate, int through_softmax, float *dout, mole_stream_t stream);
+                  int k, int normalize_gate, int through_softmax, const int32_t *counts0, const float *d_l_aux,
+                  float *dout, mole_stream_t stream);
 /* Gradient of the gate's Linear (MOLE/utils/Ugate.py:12, run by autograd in the reference):
  * dwg[E,M] = dlogits[S,E]^T . x[S,M], fp32, summed in a fixed order (partial sums per chunk of tokens in the
  * workspace, then a reduction).  bf16 tokens: E <= 256 and M a multiple of 64 on the matrix cores (dlogits
@@ -199,6 +207,10 @@ int mole_gemm_nt(const void *a, const void *b, int dtype, int rows, int N, int K
  * too large for mole_dispatch_bwd to fold in). */
 int mole_gemm_nn(const void *a, const void *b, int dtype, int rows, int N, int K, void *c,
                  mole_stream_t stream);
+/* c[Mo,N] = a[rows,Mo]^T . b[rows,N], result in `dtype`: the gate's weight gradient dlogits^T . x for the shapes
+ * mole_gate_wgrad does not take (one output tile per block, the contraction over all rows inside it). */
+int mole_gemm_tn(const void *a, const void *b, int dtype, int rows, int Mo, int N, void *c,
+                 mole_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
  * Slot pool and pinned-host expert prefetch.  Replaces _UniMem (MOLE/cpp/umemory.cpp,
@@ -223,6 +235,13 @@ int mole_gemm_nn(const void *a, const void *b, int dtype, int rows, int N, int K
  *                                 event.
  *   wait_params(stream)           the compute stream waits for the last fetch/prefetch.
  *   release(view_base, n, stream) records that compute on `stream` has finished with the slots.
+ *
+ * prefetch_ids / fetch_ids are the same two calls for an explicit list of experts instead of a range:
+ * expert expert_ids[i] (an index into the pinned host arrays) lands in the i-th slot of the call, so the
+ * host side can bring in only the experts that routing activated (kept_rows[e] > 0) and hand the grouped
+ * FFN a compacted offsets / kept_rows pair in the same order.  The reference always copies whole index
+ * ranges (MOLE/cpp/core.cpp:41-57, 1025-1047); these two have no counterpart there.  Consecutive ids that
+ * go to consecutive slots still travel as one copy per parameter kind.
  * ------------------------------------------------------------------------------------------ */
 int mole_unimem_create(int device, int pool_size, int dtype, int64_t F, int64_t M, void **handle);
 int mole_unimem_destroy(void *handle);
@@ -231,9 +250,17 @@ int mole_unimem_view_pool_size(void *handle, int *out);
 int mole_unimem_virtual_offset(void *handle, int *out);
 int mole_unimem_slot_ptr(void *handle, int p_id, int slot, void **out);
 int mole_unimem_prefetch(void *handle, int layer, const void *const host_src[4], int base, int n);
+int mole_unimem_prefetch_ids(void *handle, int layer, const void *const host_src[4], const int32_t *expert_ids,
+                             int n);
+/* The bookkeeping half of prefetch alone (_UniMem::prefetch, MOLE/cpp/umemory.cpp:131-154, exported by the
+ * reference as pool_prefetch, MOLE/cpp/core.cpp:1425): reserve n slots for `layer` and return their addresses;
+ * the caller fills them and orders its copies against the compute stream itself. */
+int mole_unimem_reserve(void *handle, int layer, int n, void **slot_ptrs_out /* [4] */);
 int mole_unimem_fetch_top(void *handle, int layer, int *n_out);
 int mole_unimem_fetch(void *handle, const void *const host_src[4], int view_base, int base, int n,
                       int prefetched, void **slot_ptrs_out /* [4] */);
+int mole_unimem_fetch_ids(void *handle, const void *const host_src[4], int view_base, const int32_t *expert_ids,
+                          int n, int prefetched, void **slot_ptrs_out /* [4] */);
 int mole_unimem_wait_params(void *handle, mole_stream_t compute_stream);
 int mole_unimem_release(void *handle, int view_base, int n, mole_stream_t compute_stream);
 int mole_unimem_sync_tran(void *handle);
@@ -254,6 +281,13 @@ int mole_unimem_copy_stats(void *handle, uint64_t *bytes, float *busy_ms);
  * since the previous read; reading resets the sums. */
 int mole_unimem_store_grads(void *handle, void *const host_dst[4], const void *const dev_src[4], int base,
                             int n, mole_stream_t compute_stream);
+/* The same for an explicit expert list: the i-th of the n experts in dev_src goes to host expert expert_ids[i].
+ * mole_unimem_zero_grads_ids writes zeros to the listed host experts instead (the gradient of an expert that
+ * received no rows), from a zeroed device slot the pool allocates on first use; it is ordered after the
+ * write-backs already enqueued and waits for no compute. */
+int mole_unimem_store_grads_ids(void *handle, void *const host_dst[4], const void *const dev_src[4],
+                                const int32_t *expert_ids, int n, mole_stream_t compute_stream);
+int mole_unimem_zero_grads_ids(void *handle, void *const host_dst[4], const int32_t *expert_ids, int n);
 int mole_unimem_sync_tranback(void *handle);
 int mole_unimem_tranback_stream(void *handle, mole_stream_t *out);
 int mole_unimem_writeback_stats(void *handle, uint64_t *bytes, float *busy_ms);

@@ -29,7 +29,8 @@ _SIGNATURES = {
     "mole_kernel_timing_read": (c_int, [c_int, POINTER(c_int), POINTER(c_float)]),
     "mole_softmax_fwd": (c_int, [_P, _P, c_int, c_int, _P, _P]),
     "mole_gate_fwd": (c_int, [_P, c_int, _P, _P, c_int, c_int, c_int, _P, _P]),
-    "mole_gate_bwd": (c_int, [_P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P, _P]),
+    "mole_softmax_bwd": (c_int, [_P, _P, c_int, c_int, _P, _P]),
+    "mole_gate_bwd": (c_int, [_P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P, _P, _P, _P]),
     "mole_gate_wgrad_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "mole_gate_wgrad": (c_int, [_P, _P, c_int, c_int, c_int, c_int, _P, _P, c_size_t, _P]),
     "mole_route_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
@@ -45,6 +46,7 @@ _SIGNATURES = {
                              _P, c_int, c_int, _P]),
     "mole_gemm_nt": (c_int, [_P, _P, c_int, c_int, c_int, c_int, _P, _P]),
     "mole_gemm_nn": (c_int, [_P, _P, c_int, c_int, c_int, c_int, _P, _P]),
+    "mole_gemm_tn": (c_int, [_P, _P, c_int, c_int, c_int, c_int, _P, _P]),
     "mole_unimem_create": (c_int, [c_int, c_int, c_int, c_int64, c_int64, POINTER(_P)]),
     "mole_unimem_destroy": (c_int, [_P]),
     "mole_unimem_clear_virtual_mem": (c_int, [_P]),
@@ -52,14 +54,19 @@ _SIGNATURES = {
     "mole_unimem_virtual_offset": (c_int, [_P, POINTER(c_int)]),
     "mole_unimem_slot_ptr": (c_int, [_P, c_int, c_int, POINTER(_P)]),
     "mole_unimem_prefetch": (c_int, [_P, c_int, POINTER(_P), c_int, c_int]),
+    "mole_unimem_prefetch_ids": (c_int, [_P, c_int, POINTER(_P), POINTER(c_int32), c_int]),
+    "mole_unimem_reserve": (c_int, [_P, c_int, c_int, POINTER(_P)]),
     "mole_unimem_fetch_top": (c_int, [_P, c_int, POINTER(c_int)]),
     "mole_unimem_fetch": (c_int, [_P, POINTER(_P), c_int, c_int, c_int, c_int, POINTER(_P)]),
+    "mole_unimem_fetch_ids": (c_int, [_P, POINTER(_P), c_int, POINTER(c_int32), c_int, c_int, POINTER(_P)]),
     "mole_unimem_wait_params": (c_int, [_P, _P]),
     "mole_unimem_release": (c_int, [_P, c_int, c_int, _P]),
     "mole_unimem_sync_tran": (c_int, [_P]),
     "mole_unimem_tran_stream": (c_int, [_P, POINTER(_P)]),
     "mole_unimem_copy_stats": (c_int, [_P, POINTER(c_uint64), POINTER(c_float)]),
     "mole_unimem_store_grads": (c_int, [_P, POINTER(_P), POINTER(_P), c_int, c_int, _P]),
+    "mole_unimem_store_grads_ids": (c_int, [_P, POINTER(_P), POINTER(_P), POINTER(c_int32), c_int, _P]),
+    "mole_unimem_zero_grads_ids": (c_int, [_P, POINTER(_P), POINTER(c_int32), c_int]),
     "mole_unimem_sync_tranback": (c_int, [_P]),
     "mole_unimem_tranback_stream": (c_int, [_P, POINTER(_P)]),
     "mole_unimem_writeback_stats": (c_int, [_P, POINTER(c_uint64), POINTER(c_float)]),

@@ -80,6 +80,22 @@ class UniMem:
                 "mole_unimem_fetch")
         return [int(p) for p in ptrs]
 
+    @staticmethod
+    def _ids(ids):
+        return (ctypes.c_int32 * max(len(ids), 1))(*[int(e) for e in ids])
+
+    def prefetch_ids(self, layer: int, host_tensors, ids):
+        """prefetch() for an explicit list of experts: ids[i] lands in the i-th reserved slot."""
+        L.check(L.lib().mole_unimem_prefetch_ids(self._h, layer, self._src(host_tensors), self._ids(ids), len(ids)),
+                "mole_unimem_prefetch_ids")
+
+    def fetch_ids(self, host_tensors, view_base: int, ids, prefetched: int) -> List[int]:
+        """fetch() for an explicit list of experts (the first `prefetched` of them are already in their slots)."""
+        ptrs = (c_void_p * 4)()
+        L.check(L.lib().mole_unimem_fetch_ids(self._h, self._src(host_tensors), view_base, self._ids(ids), len(ids),
+                                              prefetched, ptrs), "mole_unimem_fetch_ids")
+        return [int(p) for p in ptrs]
+
     def wait_params(self):
         L.check(L.lib().mole_unimem_wait_params(self._h, L.stream()), "mole_unimem_wait_params")
 
@@ -100,6 +116,20 @@ class UniMem:
         wb = torch.cuda.ExternalStream(int(out.value), device=dev_grads[0].device)
         for g in dev_grads:           # the allocator must not hand these blocks out again before the copy has run
             g.record_stream(wb)
+
+    def store_grads_ids(self, host_grads, dev_grads, ids):
+        """store_grads() with the i-th expert of dev_grads going to host expert ids[i]."""
+        L.check(L.lib().mole_unimem_store_grads_ids(self._h, self._src(host_grads), self._src(dev_grads), self._ids(ids),
+                                                    len(ids), L.stream()), "mole_unimem_store_grads_ids")
+        wb = self._side_stream("mole_unimem_tranback_stream", dev_grads[0].device)
+        for g in dev_grads:
+            g.record_stream(wb)
+
+    def zero_grads_ids(self, host_grads, ids):
+        """Zeros to the listed experts of the pinned host gradient arrays, on the write-back stream."""
+        if ids:
+            L.check(L.lib().mole_unimem_zero_grads_ids(self._h, self._src(host_grads), self._ids(ids), len(ids)),
+                    "mole_unimem_zero_grads_ids")
 
     @staticmethod
     def _arrays(tensors):
@@ -153,6 +183,11 @@ class UniMem:
         L.check(L.lib().mole_unimem_tran_stream(self._h, ctypes.byref(out)), "mole_unimem_tran_stream")
         return int(out.value or 0)
 
+    def tranback_stream_handle(self) -> int:
+        out = c_void_p()
+        L.check(L.lib().mole_unimem_tranback_stream(self._h, ctypes.byref(out)), "mole_unimem_tranback_stream")
+        return int(out.value or 0)
+
     def copy_stats(self):
         b, ms = c_uint64(), c_float()
         L.check(L.lib().mole_unimem_copy_stats(self._h, ctypes.byref(b), ctypes.byref(ms)), "mole_unimem_copy_stats")
@@ -169,11 +204,20 @@ _UniMemInst: List[UniMem] = []
 
 
 def create_UniMem(device, pool_size, dtype, sizes) -> UniMem:
-    """create_UniMem(local_rank, pool_size, "torch.float32", [[F,M],[F],[F,M],[M]]) - layer.py:43-47."""
-    if _UniMemInst:
-        return _UniMemInst[0]
+    """create_UniMem(local_rank, pool_size, "torch.float32", [[F,M],[F],[F,M],[M]]) - layer.py:43-47.
+    The pool is process-global and the first caller sizes it (umemory.cpp:77-86); a later caller whose experts
+    have another shape or dtype, or who asks for more slots, would read and write the slots at the wrong strides,
+    so that is refused here (the reference does not check)."""
     dt = _DTYPES[dtype] if isinstance(dtype, str) else dtype
     F, M = int(sizes[0][0]), int(sizes[0][1])
+    if _UniMemInst:
+        um = _UniMemInst[0]
+        if int(pool_size) > 0 and (um.dtype, um.F, um.M) != (dt, F, M):
+            raise RuntimeError(f"create_UniMem: the slot pool holds {um.dtype} experts of F={um.F}, M={um.M}; "
+                               f"a layer with {dt}, F={F}, M={M} cannot share it")
+        if int(pool_size) > um.pool_size:
+            raise RuntimeError(f"create_UniMem: the slot pool has {um.pool_size} slots, {pool_size} were asked for")
+        return um
     um = UniMem(int(device), int(pool_size), dt, F, M)
     _UniMemInst.append(um)
     return um
@@ -210,6 +254,69 @@ def default_wait_tran():
         _UniMemInst[0].wait_params()
 
 
+_multi_stream = [True]
+
+
+def disable_multi_stream():
+    """core.cpp:1402 / stream.cpp:84-95: every role runs on the compute stream.  Here: the copies still run on the
+    pool's streams (the ordering events make that invisible to results), but ExpertStreamCtx hands out the compute
+    stream for every role."""
+    _multi_stream[0] = False
+
+
+def multi_stream_enabled() -> bool:
+    return _multi_stream[0]
+
+
+def get_stream_cdata(device: int, idx: int) -> int:
+    """Raw handle of the stream with the reference's role index (stream.hpp:30-66: tran = 1, comp = 2, comm = 3,
+    tranback = 4; core.cpp:1401).  comp and comm are torch's current stream (one GPU: no exchange stream)."""
+    um = get_UniMem()
+    if idx == 1 and um is not None and _multi_stream[0]:
+        return um.tran_stream_handle()
+    if idx == 4 and um is not None and _multi_stream[0]:
+        return um.tranback_stream_handle()
+    return int(torch.cuda.current_stream(device).cuda_stream)
+
+
+def default_wait_comp():
+    """core.cpp:1403: the default stream waits for the compute stream - the same stream here, nothing to do."""
+    return None
+
+
+def default_wait_comm():
+    """core.cpp:1404: likewise for the exchange stream, which one GPU does not have."""
+    return None
+
+
+class _DeviceSpan:
+    """A stretch of device memory as an object torch.as_tensor() can wrap without copying."""
+
+    def __init__(self, ptr: int, nbytes: int):
+        self.__cuda_array_interface__ = {"shape": (nbytes,), "typestr": "|u1", "data": (ptr, False), "version": 2}
+
+
+def pool_prefetch(moe_id: int, batch_size: int):
+    """core.cpp:1425 -> _UniMem::prefetch (umemory.cpp:131-154): reserve `batch_size` slots for layer `moe_id` on
+    the prefetch stack and return the four slot tensors [batch_size, F, M], [batch_size, F], [batch_size, F, M],
+    [batch_size, M] for the caller to fill (MOLECore.prefetch_fwd does reserve + copy in one call)."""
+    um = get_UniMem()
+    if batch_size == 0 or um is None:
+        return []
+    ptrs = (c_void_p * 4)()
+    L.check(L.lib().mole_unimem_reserve(um._h, int(moe_id), int(batch_size), ptrs), "mole_unimem_reserve")
+    es = torch.empty(0, dtype=um.dtype).element_size()
+    shapes = [(batch_size, um.F, um.M), (batch_size, um.F), (batch_size, um.F, um.M), (batch_size, um.M)]
+    out = []
+    for ptr, shape in zip(ptrs, shapes):
+        n = 1
+        for d in shape:
+            n *= d
+        raw = torch.as_tensor(_DeviceSpan(int(ptr), n * es), device=torch.device("cuda", um.device))
+        out.append(raw.view(um.dtype).view(shape))
+    return out
+
+
 def fast_assign_prefetch(P: int, Fv, Ev):
     """(GPscheme, LPscheme) as core.cpp:1302-1345: GPscheme[i] = [[later_layer, count], ...]."""
     n = len(Ev)
@@ -229,12 +336,49 @@ def fast_assign_prefetch(P: int, Fv, Ev):
 # ---------------------------------------------------------------------------------------------
 # per-layer core
 # ---------------------------------------------------------------------------------------------
+def plan_chunks(n_total: int, prefetched: int, view_pool_size: int, ebatch_size: int):
+    """Chunks of the offloaded experts of one layer, in processing order -> [(first, size, already_prefetched,
+    view_base)] (core.cpp:1020-1051).  The first `prefetched` experts already sit in slots 0.. of the visible
+    pool, so a chunk that still holds some of them must start at slot == index: where the reference wraps
+    view_base to 0 regardless (core.cpp:1026-1046) - which would run such a chunk on whatever slot 0 holds - the
+    chunk is cut at the end of the visible pool instead, and the wrap happens once the prefetched experts are done."""
+    if n_total == 0:
+        return []
+    vps = int(view_pool_size)
+    if vps <= 0:
+        raise RuntimeError("slot pool exhausted by prefetches: no slot left to run offloaded experts")
+    if prefetched > vps:
+        raise RuntimeError(f"{prefetched} prefetched experts cannot sit in a visible pool of {vps} slots")
+    d_batch = min(max(int(ebatch_size), 1), vps)
+    out, view_base, i = [], 0, 0
+    while i < n_total:
+        size = min(d_batch, n_total - i)
+        if vps - view_base < size:
+            if i < prefetched:
+                size = vps - view_base
+            else:
+                view_base = 0
+        out.append((i, size, max(0, min(size, prefetched - i)), view_base))
+        view_base += size
+        i += size
+    return out
+
+
 class MOLECore:
-    """Per-layer state and the expert-batch pipeline (define.hpp:338-607, core.cpp:991-1300)."""
+    """Per-layer state and the expert-batch pipeline (define.hpp:338-607, core.cpp:991-1300).
+
+    activated_only (default): offloaded experts that routing gave no row (kept_rows[e] == 0) are neither copied to
+    the pool nor launched; their host gradient is zero.  The layer reads its E kept-row counts back once per
+    forward (one small device-to-host copy, the only host synchronisation of the path), packs the activated
+    experts into pool slots in processing order and hands the grouped FFN a compacted offsets / kept_rows pair.
+    prefetch_bwd prefetches only experts the forward pass activated; prefetch_fwd, which runs before the layer's
+    routing exists, prefetches the experts the previous step activated (none before the first step) - a wrong
+    guess costs a copy, never a result.  The reference copies and runs every expert of every chunk in index
+    order (core.cpp:41-57, 1025-1047); activated_only=False does the same."""
 
     def __init__(self, use_pool, mome_use_pool, vari_use_pool, grad_use_pool, s_experts, d_experts, ebatch_size,
                  world_size, act_name, adv_adam, acc_step, step, device, moe_id, total_experts,
-                 gelu_bwd: str = "tanh"):
+                 gelu_bwd: str = "tanh", activated_only: bool = True):
         if world_size != 1:
             raise NotImplementedError("this build covers the single-GPU hot path (world_size == 1)")
         if act_name != "gelu":
@@ -246,11 +390,24 @@ class MOLECore:
         self.device, self.moe_id, self.total_experts = device, moe_id, total_experts
         self.s_experts, self.d_experts, self.ebatch_size = s_experts, d_experts, max(int(ebatch_size), 1)
         self.world_size, self.act_name = world_size, act_name
-        self.fwd_base = self.bwd_base = 0
         self.gelu_bwd = L.GELU_BWD_TANH if gelu_bwd == "tanh" else L.GELU_BWD_EXACT
         self.gpu = [None] * 4       # (all_tensors, grad_tensors)
         self.cpu = [None] * 4       # (all_tensors, grad_)
         self._saved = None
+        self.activated_only = bool(activated_only)
+        self._pref = {"fwd": [], "bwd": []}   # experts prefetched so far for the next pass, in slot order
+        self._active = None                   # offloaded experts the last forward gave rows to (None: not known)
+        self._grad_is_zero = [False] * d_experts   # the expert's pinned host gradient is known to hold zeros
+        self.lazy_zero = True
+
+    # the reference's counters of experts prefetched so far (define.hpp:352-353)
+    @property
+    def fwd_base(self) -> int:
+        return len(self._pref["fwd"])
+
+    @property
+    def bwd_base(self) -> int:
+        return len(self._pref["bwd"])
 
     # parameter stores -------------------------------------------------------------------------
     def set_GPUParamCore(self, p_id, all_tensors, grad_tensors, bias):
@@ -268,21 +425,50 @@ class MOLECore:
     def set_hybrid_adam_count(self, hybrid_adam_count):
         self.hybrid_adam_count = self.d_experts if hybrid_adam_count == -1 else int(hybrid_adam_count)
 
+    def set_lazy_zero(self):
+        """The host gradient arrays are to be taken as zero: the next write-back overwrites them
+        (uparameter.cpp:68-83, core.cpp:1392)."""
+        for c in self.cpu:
+            if c is not None and c[1] is not None:
+                c[1].lazy_zero = True
+
+    def unset_lazy_zero(self):
+        for c in self.cpu:
+            if c is not None and c[1] is not None:
+                c[1].lazy_zero = False
+
+    def host_gradients_changed(self):
+        """Call after writing the pinned host gradient arrays from outside the pipeline (loading a checkpoint):
+        experts that get no rows in the next step are then zeroed again instead of being taken as already zero."""
+        self._grad_is_zero = [False] * self.d_experts
+
     def _host(self):
         return [c[0] for c in self.cpu]
 
     # prefetch -----------------------------------------------------------------------------------
-    def prefetch_fwd(self, batch_size: int):
-        if batch_size == 0:
+    def _prefetch(self, which: str, batch_size: int):
+        if batch_size <= 0 or self.d_experts == 0:
             return
-        get_UniMem().prefetch(self.moe_id, self._host(), self.fwd_base, batch_size)
-        self.fwd_base += batch_size
+        done = self._pref[which]
+        if not self.activated_only:
+            todo = list(range(len(done), min(self.d_experts, len(done) + batch_size)))
+            if not todo:
+                return
+            get_UniMem().prefetch(self.moe_id, self._host(), todo[0], len(todo))
+        else:
+            known = self._active if self._active is not None else []
+            seen = set(done)
+            todo = [e for e in known if e not in seen][:batch_size]
+            if not todo:
+                return
+            get_UniMem().prefetch_ids(self.moe_id, self._host(), todo)
+        done.extend(todo)
+
+    def prefetch_fwd(self, batch_size: int):
+        self._prefetch("fwd", batch_size)
 
     def prefetch_bwd(self, batch_size: int):
-        if batch_size == 0:
-            return
-        get_UniMem().prefetch(self.moe_id, self._host(), self.bwd_base, batch_size)
-        self.bwd_base += batch_size
+        self._prefetch("bwd", batch_size)
 
     def dummy_fetch(self, batch_size: int):
         """Copy `batch_size` experts into slots 0.. without reserving them (core.cpp:25-39)."""
@@ -292,26 +478,36 @@ class MOLECore:
         um.fetch(self._host(), -um.virtual_offset(), 0, batch_size, 0)
 
     # pipeline -----------------------------------------------------------------------------------
-    def _chunks(self, prefetched: int):
-        """Offloaded experts -> [(base, size, already_prefetched, view_base)] (core.cpp:1020-1051)."""
+    def _take_prefetched(self, which: str):
+        """Pops this layer's entry of the prefetch stack; returns the experts it holds, in slot order."""
         um = get_UniMem()
-        if self.d_experts == 0:
-            return []
         if not self.use_pool or um is None or um.pool_size <= 0:
             raise RuntimeError("offloaded experts need the slot pool (pool_size >= 1, use_pool=True)")
-        vps = um.view_pool_size()
-        if vps <= 0:
-            raise RuntimeError("slot pool exhausted by prefetches: no slot left to run offloaded experts")
-        d_batch = min(self.ebatch_size, vps)
-        out, view_base, i = [], 0, 0
-        while i < self.d_experts:
-            size = min(d_batch, self.d_experts - i)
-            if vps - view_base < size:
-                view_base = 0
-            out.append((i, size, max(0, min(size, prefetched - i)), view_base))
-            view_base += size
-            i += d_batch
-        return out
+        n = um.fetch_top(self.moe_id)
+        ids, self._pref[which] = self._pref[which], []
+        if n != len(ids):
+            raise RuntimeError(f"prefetch stack out of order: top holds {n}, layer expects {len(ids)}")
+        return ids
+
+    def _chunks(self, n_total: int, prefetched: int):
+        um = get_UniMem()
+        return plan_chunks(n_total, prefetched, um.view_pool_size(), self.ebatch_size)
+
+    def _order(self, resident, wanted, offsets, kept_rows, host_meta):
+        """Processing order of the offloaded experts - the resident (prefetched) ones in slot order, then the
+        wanted ones not among them - and the matching offsets / kept_rows arrays on the device."""
+        d, e0 = self.d_experts, self.s_experts
+        inres = set(resident)
+        order = list(resident) + [e for e in wanted if e not in inres]
+        if order == list(range(d)):
+            return order, offsets[e0:], kept_rows[e0:]
+        if host_meta is None:     # no host copy of the counts: gather on the device
+            sel = torch.tensor(order, dtype=torch.int64).to(offsets.device)
+            return order, offsets[e0:e0 + d][sel].contiguous(), kept_rows[e0:e0 + d][sel].contiguous()
+        off_h, kept_h = host_meta
+        comp = torch.tensor([[off_h[e] for e in order], [kept_h[e] for e in order]], dtype=torch.int32)
+        comp = comp.to(offsets.device)
+        return order, comp[0], comp[1]
 
     def forward(self, dispatched_input: torch.Tensor, requires_grad: bool, offsets=None, kept_rows=None,
                 return_saved: bool = False):
@@ -322,7 +518,8 @@ class MOLECore:
         shape = x.shape
         M = shape[-1]
         E = self.s_experts + self.d_experts
-        if offsets is None:
+        routed = offsets is not None
+        if not routed:
             assert x.dim() == 3 and shape[0] == E, f"expected [E={E}, C, M], got {tuple(shape)}"
             C = shape[1]
             offsets = torch.arange(E + 1, dtype=torch.int32, device=x.device) * C
@@ -338,19 +535,27 @@ class MOLECore:
         if self.s_experts:
             w1, b1, w2, b2 = (g[0] for g in self.gpu)
             H.ffn_fwd_into(x2, offsets, kept_rows, self.s_experts, rows, M, F, w1, b1, w2, b2, h, a, out)
+        host_meta = None
         if self.d_experts:
             um = get_UniMem()
-            prefetched = um.fetch_top(self.moe_id)
-            if prefetched != self.fwd_base:
-                raise RuntimeError(f"prefetch stack out of order: top holds {prefetched}, layer expects {self.fwd_base}")
-            self.fwd_base = 0
-            for (base, size, pref, view_base) in self._chunks(prefetched):
-                p = um.fetch(self._host(), view_base, base, size, pref)
+            resident = self._take_prefetched("fwd")
+            d, e0 = self.d_experts, self.s_experts
+            if self.activated_only and routed:
+                # the one host synchronisation of the path: E row counts (and row offsets) come back
+                meta = torch.stack([offsets[e0:e0 + d], kept_rows[e0:e0 + d]]).cpu()
+                host_meta = (meta[0].tolist(), meta[1].tolist())
+                self._active = [e for e in range(d) if host_meta[1][e] > 0]
+                wanted = self._active
+            else:
+                self._active = list(range(d))       # every expert runs
+                wanted = range(d)
+            order, off_c, kept_c = self._order(resident, wanted, offsets, kept_rows, host_meta)
+            for (lo, size, pref, view_base) in self._chunks(len(order), len(resident)):
+                p = um.fetch_ids(self._host(), view_base, order[lo:lo + size], pref)
                 um.wait_params()
-                e0 = self.s_experts + base
-                H.ffn_fwd_into(x2, offsets[e0:], kept_rows[e0:], size, rows, M, F, p[0], p[1], p[2], p[3], h, a, out)
+                H.ffn_fwd_into(x2, off_c[lo:], kept_c[lo:], size, rows, M, F, p[0], p[1], p[2], p[3], h, a, out)
                 um.release(view_base, size)
-        saved = (x2, h, a, offsets, kept_rows, requires_grad, shape)
+        saved = (x2, h, a, offsets, kept_rows, requires_grad, shape, host_meta)
         if return_saved:          # the caller (an autograd node) keeps the activations itself
             return out.view(shape), saved
         self._saved = saved       # reference behaviour: the core holds them until backward (define.hpp:594-606)
@@ -361,7 +566,7 @@ class MOLECore:
             saved, self._saved = self._saved, None
         if saved is None:
             raise RuntimeError("MOLECore.backward without a preceding forward")
-        x2, h, a, offsets, kept_rows, need_gx, shape = saved
+        x2, h, a, offsets, kept_rows, need_gx, shape, host_meta = saved
         M = shape[-1]
         go = all_output_grad.reshape(-1, M)
         if not go.is_contiguous():
@@ -378,26 +583,47 @@ class MOLECore:
                            gx, acc, self.gelu_bwd)
         if self.d_experts:
             um = get_UniMem()
-            prefetched = um.fetch_top(self.moe_id)
-            if prefetched != self.bwd_base:
-                raise RuntimeError(f"prefetch stack out of order: top holds {prefetched}, layer expects {self.bwd_base}")
-            self.bwd_base = 0
+            resident = self._take_prefetched("bwd")
+            d = self.d_experts
             host_grads = [c[1] for c in self.cpu]
             adam_now = self.adv_adam and (self.step + 1) % self.acc_step == 0
-            for (base, size, pref, view_base) in self._chunks(prefetched):
-                p = um.fetch(self._host(), view_base, base, size, pref)   # weights are fetched again (core.cpp:1203)
+            adding = self.acc_step > 1 and not getattr(host_grads[0], "lazy_zero", True)
+            if host_meta is not None:
+                active = [e for e in range(d) if host_meta[1][e] > 0]
+                # the optimizer moves every parameter it owns, also those whose gradient is zero
+                wanted = range(d) if adam_now else active
+            else:
+                active, wanted = list(range(d)), range(d)
+            order, off_c, kept_c = self._order(resident, wanted, offsets, kept_rows, host_meta)
+            for (lo, size, pref, view_base) in self._chunks(len(order), len(resident)):
+                ids = order[lo:lo + size]
+                p = um.fetch_ids(self._host(), view_base, ids, pref)   # weights are fetched again (core.cpp:1203)
                 um.wait_params()
-                e0 = self.s_experts + base
                 g = [torch.empty((size, *hg.shape[1:]), dtype=hg.dtype, device=x2.device) for hg in host_grads]
-                H.ffn_bwd_into(go, x2, h, a, offsets[e0:], kept_rows[e0:], size, rows, M, F, p[0], p[2], t, g[0], g[1],
+                H.ffn_bwd_into(go, x2, h, a, off_c[lo:], kept_c[lo:], size, rows, M, F, p[0], p[2], t, g[0], g[1],
                                g[2], g[3], gx, False, self.gelu_bwd)
                 if adam_now:
                     # the update reads the parameters in their pool slots, so the slots are released after it
-                    self._instant_adam(p, g, base, size)
+                    self._instant_adam(p, g, ids, adding)
                     um.release(view_base, size)
                 else:
                     um.release(view_base, size)
-                    self._store_grad(host_grads, g, base, size)
+                    self._store_grad(host_grads, g, ids, adding)
+            if host_meta is not None:
+                # experts that got no row: their gradient is zero.  While sums are being built up that adds
+                # nothing; otherwise the host array must read zero, which costs a copy only if it does not already
+                act = set(active)
+                if not adding:
+                    seen = set(order)
+                    stale = [e for e in range(d) if e not in seen and not self._grad_is_zero[e]]
+                    um.zero_grads_ids(host_grads, stale)
+                    for e in range(d):
+                        self._grad_is_zero[e] = e not in act
+                else:
+                    for e in act:
+                        self._grad_is_zero[e] = False
+            else:
+                self._grad_is_zero = [False] * d
             if adam_now:
                 # the next prefetch reads the host parameters that the write-back stream is still filling
                 # (the reference ends its backward with a synchronisation of the copy stream, core.cpp:1287)
@@ -408,13 +634,26 @@ class MOLECore:
                 c[1].lazy_zero = False
         return gx.view(shape) if need_gx else None
 
-    def _store_grad(self, host_grads, g, base, size):
+    @staticmethod
+    def _runs(ids):
+        """[(position of the run's first expert in ids, first expert, length)] of the runs of consecutive experts."""
+        runs, i = [], 0
+        while i < len(ids):
+            j = i + 1
+            while j < len(ids) and ids[j] == ids[j - 1] + 1:
+                j += 1
+            runs.append((i, ids[i], j - i))
+            i = j
+        return runs
+
+    def _store_grad(self, host_grads, g, ids, adding):
         """Gradients of offloaded experts go back to their pinned host buffers (core.cpp:77-103,
         uparameter.cpp:68-83): overwrite, or add when accumulating and the buffer is not lazily zero."""
-        if self.acc_step > 1 and not getattr(host_grads[0], "lazy_zero", True):
-            self._add_to_host([hg[base:base + size] for hg in host_grads], g)
+        if adding:
+            for (at, e, n) in self._runs(ids):
+                self._add_to_host([hg[e:e + n] for hg in host_grads], [gg[at:at + n] for gg in g])
         else:
-            get_UniMem().store_grads(host_grads, g, base, size)
+            get_UniMem().store_grads_ids(host_grads, g, ids)
 
     @staticmethod
     def _add_to_host(host_slices, g):
@@ -429,49 +668,52 @@ class MOLECore:
             gg += pp
         um.store_state(host_slices, g)
 
-    def _instant_adam(self, p_slots, g, base, size):
-        """Adam on the GPU for experts [base, base+size) of the offloaded set, inside the backward pipeline
-        (core.cpp:848-943): fetch their moments (and, when accumulating, the gradients of the earlier
-        micro-steps) from pinned host memory, one fused update per parameter array, write parameters and
-        moments back.  Only the first hybrid_adam_count experts are updated here; the gradients of the others
-        go to the host for the CPU optimizer.  The reference narrows the second weight from the first one when
-        it cuts a batch at hybrid_adam_count (core.cpp:859); this follows the evident intent instead."""
+    def _instant_adam(self, p_slots, g, ids, adding):
+        """Adam on the GPU for the experts `ids` of the offloaded set (one chunk, in slot order), inside the
+        backward pipeline (core.cpp:848-943): fetch their moments (and, when accumulating, the gradients of the
+        earlier micro-steps) from pinned host memory, one fused update per parameter array, write parameters and
+        moments back.  Only experts below hybrid_adam_count are updated here; the gradients of the others go to
+        the host for the CPU optimizer.  The reference narrows the second weight from the first one when it cuts
+        a batch at hybrid_adam_count (core.cpp:859); this follows the evident intent instead."""
         if self.adam is None:
             raise RuntimeError("in-pipeline Adam needs set_adam() before backward")
         if any(c[2] is None or c[3] is None for c in self.cpu):
             raise RuntimeError("in-pipeline Adam needs momentum and variance arrays (set_CPUParamCore)")
         um = get_UniMem()
         host_grads = [c[1] for c in self.cpu]
-        n = max(0, min(size, self.hybrid_adam_count - base))
-        if n < size:          # experts beyond the GPU-updated prefix: gradients only
-            rest = [gg[n:] for gg in g]
-            if self.acc_step > 1 and not getattr(host_grads[0], "lazy_zero", True):
-                self._add_to_host([hg[base + n:base + size] for hg in host_grads], rest)
-            else:
-                um.store_state([hg[base + n:base + size] for hg in host_grads], rest)
-        if n == 0:
-            return
-        beta1, beta2, t, lr, lam, eps, adamw = self.adam
-        dev = g[0].device
-        m_host = [c[2][base:base + n] for c in self.cpu]
-        v_host = [c[3][base:base + n] for c in self.cpu]
-        m = [torch.empty(mh.shape, dtype=torch.float32, device=dev) for mh in m_host]
-        v = [torch.empty(vh.shape, dtype=torch.float32, device=dev) for vh in v_host]
-        loads_dev, loads_host = m + v, m_host + v_host
-        acc = self.acc_step > 1 and not getattr(host_grads[0], "lazy_zero", True)
-        if acc:
-            g_prev = [torch.empty((n, *hg.shape[1:]), dtype=hg.dtype, device=dev) for hg in host_grads]
-            loads_dev, loads_host = loads_dev + g_prev, loads_host + [hg[base:base + n] for hg in host_grads]
-        um.load_state(loads_dev, loads_host, after_writeback=acc)
-        p_new = []
-        for k in range(4):
-            gk = g[k][:n]
-            if acc:
-                gk += g_prev[k]
-            out = torch.empty_like(gk)
-            H.adam_step(p_slots[k], gk, m[k], v[k], beta1, beta2, t + 1, lr, lam, eps, adamw, p_out=out)
-            p_new.append(out)
-        um.store_state([c[0][base:base + n] for c in self.cpu] + m_host + v_host, p_new + m + v)
+        es = g[0].element_size()
+        for (at, e0, n_run) in self._runs(ids):
+            n = max(0, min(n_run, self.hybrid_adam_count - e0))     # experts of the run updated on the GPU
+            if n < n_run:          # beyond the GPU-updated prefix: gradients only
+                rest = [gg[at + n:at + n_run] for gg in g]
+                dst = [hg[e0 + n:e0 + n_run] for hg in host_grads]
+                if adding:
+                    self._add_to_host(dst, rest)
+                else:
+                    um.store_state(dst, rest)
+            if n == 0:
+                continue
+            beta1, beta2, t, lr, lam, eps, adamw = self.adam
+            dev = g[0].device
+            m_host = [c[2][e0:e0 + n] for c in self.cpu]
+            v_host = [c[3][e0:e0 + n] for c in self.cpu]
+            m = [torch.empty(mh.shape, dtype=torch.float32, device=dev) for mh in m_host]
+            v = [torch.empty(vh.shape, dtype=torch.float32, device=dev) for vh in v_host]
+            loads_dev, loads_host = m + v, m_host + v_host
+            if adding:
+                g_prev = [torch.empty((n, *hg.shape[1:]), dtype=hg.dtype, device=dev) for hg in host_grads]
+                loads_dev, loads_host = loads_dev + g_prev, loads_host + [hg[e0:e0 + n] for hg in host_grads]
+            um.load_state(loads_dev, loads_host, after_writeback=adding)
+            p_new = []
+            for k in range(4):
+                gk = g[k][at:at + n]
+                if adding:
+                    gk += g_prev[k]
+                out = torch.empty_like(gk)
+                per_expert = gk[0].numel() * es
+                H.adam_step(p_slots[k] + at * per_expert, gk, m[k], v[k], beta1, beta2, t + 1, lr, lam, eps, adamw, p_out=out)
+                p_new.append(out)
+            um.store_state([c[0][e0:e0 + n] for c in self.cpu] + m_host + v_host, p_new + m + v)
 
 
 class BatchFusedFWD(torch.autograd.Function):

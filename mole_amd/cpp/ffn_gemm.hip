@@ -582,3 +582,17 @@ extern "C" int mole_gemm_nn(const void *a, const void *b, int dtype, int rows, i
     if (dtype == MOLE_BF16) return run_gemm<bf16_t, false, true, false, EPI_STORE>(g, rows, tiles, (hipStream_t)stream, MOLE_K_GEMM_NT);
     return launch_gemm<float, false, true, false, TBM, TBN, EPI_STORE>(g, tiles, (hipStream_t)stream, MOLE_K_GEMM_NT);
 }
+
+extern "C" int mole_gemm_tn(const void *a, const void *b, int dtype, int rows, int Mo, int N, void *c,
+                            mole_stream_t stream) {
+    MOLE_REQUIRE(dtype == MOLE_F32 || dtype == MOLE_BF16, "mole_gemm_tn: bad dtype %d", dtype);
+    const int epc = dtype == MOLE_BF16 ? 8 : 4;
+    MOLE_REQUIRE(rows >= 0 && N > 0 && Mo > 0 && Mo % epc == 0 && N % epc == 0, "mole_gemm_tn: bad sizes rows=%d Mo=%d N=%d", rows, Mo, N);
+    MOLE_REQUIRE(c && al16(c) && (rows == 0 || (a && b && al16(a) && al16(b))), "mole_gemm_tn: null or misaligned pointer");
+    GemmArgs g{};
+    g.single_rows = rows; g.E = 1;      // one group whose contraction runs over all rows (zero rows: c = 0)
+    g.A = a; g.lda = Mo; g.B = b; g.ldb = N; g.M = Mo; g.N = N; g.C = c; g.ldc = N; g.strideC = (long)Mo * N;
+    const int tiles = ceil_div(Mo, TBM) * ceil_div(N, TBN);
+    if (dtype == MOLE_BF16) return launch_gemm<bf16_t, true, true, true, TBM, TBN, EPI_WGRAD>(g, tiles, (hipStream_t)stream, MOLE_K_GEMM_NT);
+    return launch_gemm<float, true, true, true, TBM, TBN, EPI_WGRAD>(g, tiles, (hipStream_t)stream, MOLE_K_GEMM_NT);
+}

@@ -511,14 +511,48 @@ __global__ __launch_bounds__(256) void softmax_fwd_kernel(const float *__restric
     }
 }
 
+// Softmax backward on its own (the gate used outside the fused layer node): dlogits = s * (ds - sum_e ds s).
+template <int VPL>
+__global__ __launch_bounds__(256) void softmax_bwd_kernel(const float *__restrict__ dscores,
+                                                          const float *__restrict__ scores, int S, int E, int logG,
+                                                          float *__restrict__ dlogits) {
+    const int lane = threadIdx.x & 63;
+    const int G = 1 << logG;
+    const int g = lane & (G - 1), tg = lane >> logG;
+    const int tpw = 64 >> logG;
+    const int wave = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int token = wave * tpw + tg;
+    const bool tv = token < S;
+    float s[VPL], ds[VPL];
+    float dot = 0.f;
+#pragma unroll
+    for (int r = 0; r < VPL; ++r) {
+        const int e = g + (r << logG);
+        const size_t at = (size_t)min(token, S - 1) * E + min(e, E - 1);
+        s[r] = load_or_zero(scores + at, tv && e < E);
+        ds[r] = load_or_zero(dscores + at, tv && e < E);
+        dot += ds[r] * s[r];
+    }
+    dot = group_reduce(dot, logG, [](float a, float c) { return a + c; });
+#pragma unroll
+    for (int r = 0; r < VPL; ++r) {
+        const int e = g + (r << logG);
+        if (tv && e < E) dlogits[(size_t)token * E + e] = s[r] * (ds[r] - dot);
+    }
+}
+
 // dlogits[i,e] = s[i,e] * (dscore[i,e] - sum_e' dscore[i,e'] s[i,e']), dscore scattered from dgates
 // through gate_j = graw_j / max(sum graw, eps).  The token's group of lanes shares the k-sized part, then
-// writes the row.
+// writes the row.  With counts0 and d_l_aux given, dscore also carries the load-balancing loss
+// l_aux = E/S^2 sum_e (sum_i s[i,e]) counts0[e]: d l_aux / d s[i,e] = E/S^2 counts0[e], the same for every token
+// (the counts are integers and carry no gradient).
 template <int VPL>
 __global__ __launch_bounds__(256) void gate_bwd_kernel(const float *__restrict__ dgates,
                                                        const float *__restrict__ scores,
                                                        const int32_t *__restrict__ idx, int S, int E, int k,
                                                        int logG, int normalize, int through_softmax,
+                                                       const int32_t *__restrict__ counts0,
+                                                       const float *__restrict__ d_l_aux,
                                                        float *__restrict__ dlogits) {
     const int lane = threadIdx.x & 63;
     const int G = 1 << logG;
@@ -533,6 +567,11 @@ __global__ __launch_bounds__(256) void gate_bwd_kernel(const float *__restrict__
         const int e = g + (r << logG);
         s[r] = load_or_zero(scores + (size_t)min(token, S - 1) * E + min(e, E - 1), tv && e < E);
         ds[r] = 0.f;
+    }
+    if (counts0 != nullptr) {       // uniform over the grid
+        const float scale = d_l_aux[0] * ((float)E / ((float)S * (float)S));
+#pragma unroll
+        for (int r = 0; r < VPL; ++r) ds[r] = scale * (float)counts0[min(g + (r << logG), E - 1)];
     }
     // Lane j < k of the token's group fetches choice j (index, incoming gradient, raw gate value), the sums over
     // the k choices are lane reductions, and each choice is then handed round the group.  (With every lane walking
@@ -827,12 +866,30 @@ extern "C" int mole_gate_fwd(const void *x, int dtype, const float *wg, const fl
     return 0;
 }
 
+extern "C" int mole_softmax_bwd(const float *dscores, const float *scores, int S, int E, float *dlogits,
+                                mole_stream_t stream) {
+    MOLE_REQUIRE(S >= 0 && E >= 1 && E <= MOLE_MAX_EXPERTS, "mole_softmax_bwd: bad sizes S=%d E=%d", S, E);
+    if (S == 0) return 0;
+    MOLE_REQUIRE(dscores && scores && dlogits, "mole_softmax_bwd: null pointer");
+    int logG = 0;
+    while ((1 << logG) < E && logG < 6) ++logG;
+    const int vpl = ceil_div(E, 1 << logG);
+    const int tpw = 64 >> logG;
+    const dim3 grid(ceil_div(S, 4 * tpw));
+    ScopedTiming timing(MOLE_K_GATE_BWD, (hipStream_t)stream);
+    MOLE_VPL_DISPATCH(vpl, softmax_bwd_kernel, grid, (hipStream_t)stream, dscores, scores, S, E, logG, dlogits);
+    MOLE_LAUNCH_CHECK();
+    return 0;
+}
+
 extern "C" int mole_gate_bwd(const float *dgates, const float *scores, const int32_t *idx, int S, int E, int k,
-                             int normalize_gate, int through_softmax, float *dlogits, mole_stream_t stream) {
+                             int normalize_gate, int through_softmax, const int32_t *counts0, const float *d_l_aux,
+                             float *dlogits, mole_stream_t stream) {
     MOLE_REQUIRE(S >= 0 && E >= 1 && E <= MOLE_MAX_EXPERTS && k >= 1 && k <= MOLE_MAX_TOPK && k <= E,
                  "mole_gate_bwd: bad sizes S=%d E=%d k=%d", S, E, k);
     if (S == 0) return 0;
     MOLE_REQUIRE(dgates && scores && idx && dlogits, "mole_gate_bwd: null pointer");
+    MOLE_REQUIRE((counts0 == nullptr) == (d_l_aux == nullptr), "mole_gate_bwd: counts0 and d_l_aux go together");
     int logG = 0;
     while ((1 << logG) < E && logG < 6) ++logG;
     const int vpl = ceil_div(E, 1 << logG);
@@ -840,7 +897,7 @@ extern "C" int mole_gate_bwd(const float *dgates, const float *scores, const int
     const dim3 grid(ceil_div(S, 4 * tpw));
     ScopedTiming timing(MOLE_K_GATE_BWD, (hipStream_t)stream);
     MOLE_VPL_DISPATCH(vpl, gate_bwd_kernel, grid, (hipStream_t)stream, dgates, scores, idx, S, E, k, logG,
-                      normalize_gate, through_softmax, dlogits);
+                      normalize_gate, through_softmax, counts0, d_l_aux, dlogits);
     MOLE_LAUNCH_CHECK();
     return 0;
 }

@@ -37,6 +37,8 @@ struct UniMem {
     size_t wb_timers_used = 0;
     uint64_t wb_bytes_open = 0, wb_bytes_last = 0;
     float wb_ms_last = 0.f;
+    char *zeros = nullptr;           // one zeroed slot of the largest parameter kind (mole_unimem_zero_grads_ids)
+    bool zeros_ready = false;
 };
 
 // The next event pair of a copy stream's statistics.  A caller that never synchronises the stream would
@@ -56,15 +58,17 @@ static int next_timer(std::vector<std::array<hipEvent_t, 2>> &timers, size_t &us
 }
 static int next_timer(UniMem *u, std::array<hipEvent_t, 2> **out) { return next_timer(u->timers, u->timers_used, out); }
 
-// Host -> pool copy of experts [base, base+n) into slots [slot0, slot0+n).  The copy is cut at every
-// slot whose previous user has not been waited for yet, so that a prefetch trails the compute that
+// Host -> pool copy of experts ids[0..n) (or base, base+1, .. when ids is null) into slots [slot0, slot0+n).
+// Consecutive experts that go to consecutive slots travel in one copy per parameter kind.  The copy is cut at
+// every slot whose previous user has not been waited for yet, so that a prefetch trails the compute that
 // still owns the later slots instead of waiting for all of it.
-static int copy_experts(UniMem *u, const void *const host_src[4], int slot0, int base, int n) {
+static int copy_experts(UniMem *u, const void *const host_src[4], int slot0, const int32_t *ids, int base, int n) {
     if (n <= 0) return 0;
+    auto id_of = [&](int i) { return ids ? (int)ids[i] : base + i; };
     int i = 0;
     while (i < n) {
         int run = 1;
-        while (i + run < n && !u->slot_pending[slot0 + i + run]) ++run;
+        while (i + run < n && !u->slot_pending[slot0 + i + run] && id_of(i + run) == id_of(i) + run) ++run;
         if (u->slot_pending[slot0 + i]) {
             MOLE_HIP(hipStreamWaitEvent(u->tran, u->slot_event[slot0 + i], 0));
             u->slot_pending[slot0 + i] = 0;
@@ -74,7 +78,7 @@ static int copy_experts(UniMem *u, const void *const host_src[4], int slot0, int
         MOLE_HIP(hipEventRecord((*tm)[0], u->tran));
         for (int p = 0; p < 4; ++p) {
             const size_t sb = u->slot_bytes[p];
-            MOLE_HIP(hipMemcpyAsync(u->pool[p] + (size_t)(slot0 + i) * sb, (const char *)host_src[p] + (size_t)(base + i) * sb,
+            MOLE_HIP(hipMemcpyAsync(u->pool[p] + (size_t)(slot0 + i) * sb, (const char *)host_src[p] + (size_t)id_of(i) * sb,
                                     (size_t)run * sb, hipMemcpyHostToDevice, u->tran));
             u->bytes_open += (uint64_t)run * sb;
         }
@@ -84,6 +88,38 @@ static int copy_experts(UniMem *u, const void *const host_src[4], int slot0, int
     MOLE_HIP(hipEventRecord(u->para_event, u->tran));
     u->para_recorded = true;
     return 0;
+}
+
+static void destroy_members(UniMem *u) {
+    for (auto &e : u->slot_event) if (e) (void)hipEventDestroy(e);
+    for (auto &t : u->timers) { (void)hipEventDestroy(t[0]); (void)hipEventDestroy(t[1]); }
+    for (auto &t : u->wb_timers) { (void)hipEventDestroy(t[0]); (void)hipEventDestroy(t[1]); }
+    for (hipEvent_t e : {u->para_event, u->grads_ready, u->state_free, u->state_ready, u->wb_done}) if (e) (void)hipEventDestroy(e);
+    if (u->tran) (void)hipStreamDestroy(u->tran);
+    if (u->tranback) (void)hipStreamDestroy(u->tranback);
+    for (int p = 0; p < 4; ++p) if (u->pool[p]) (void)hipFree(u->pool[p]);
+    if (u->zeros) (void)hipFree(u->zeros);
+    delete u;
+}
+
+// streams, events and slot events of a freshly allocated pool
+static int create_members(UniMem *u) {
+    MOLE_HIP(hipStreamCreateWithFlags(&u->tran, hipStreamNonBlocking));
+    MOLE_HIP(hipStreamCreateWithFlags(&u->tranback, hipStreamNonBlocking));
+    MOLE_HIP(hipEventCreateWithFlags(&u->para_event, hipEventDisableTiming));
+    MOLE_HIP(hipEventCreateWithFlags(&u->grads_ready, hipEventDisableTiming));
+    MOLE_HIP(hipEventCreateWithFlags(&u->state_free, hipEventDisableTiming));
+    MOLE_HIP(hipEventCreateWithFlags(&u->state_ready, hipEventDisableTiming));
+    MOLE_HIP(hipEventCreateWithFlags(&u->wb_done, hipEventDisableTiming));
+    u->slot_event.assign(u->pool_size, nullptr);
+    u->slot_pending.assign(u->pool_size, 0);
+    for (int s = 0; s < u->pool_size; ++s) MOLE_HIP(hipEventCreateWithFlags(&u->slot_event[s], hipEventDisableTiming));
+    return 0;
+}
+
+static bool ids_ok(const int32_t *ids, int n) {
+    for (int i = 0; i < n; ++i) if (ids[i] < 0) return false;
+    return true;
 }
 
 }  // namespace mole
@@ -115,21 +151,14 @@ extern "C" int mole_unimem_create(int device, int pool_size, int dtype, int64_t 
         if (e != hipSuccess) {
             set_error("mole_unimem_create: hipMalloc of %zu bytes failed: %s", u->slot_bytes[p] * pool_size,
                       hipGetErrorString(e));
-            for (int q = 0; q < p; ++q) (void)hipFree(u->pool[q]);
-            delete u;
+            destroy_members(u);
             return MOLE_E_NOMEM;
         }
     }
-    MOLE_HIP(hipStreamCreateWithFlags(&u->tran, hipStreamNonBlocking));
-    MOLE_HIP(hipStreamCreateWithFlags(&u->tranback, hipStreamNonBlocking));
-    MOLE_HIP(hipEventCreateWithFlags(&u->para_event, hipEventDisableTiming));
-    MOLE_HIP(hipEventCreateWithFlags(&u->grads_ready, hipEventDisableTiming));
-    MOLE_HIP(hipEventCreateWithFlags(&u->state_free, hipEventDisableTiming));
-    MOLE_HIP(hipEventCreateWithFlags(&u->state_ready, hipEventDisableTiming));
-    MOLE_HIP(hipEventCreateWithFlags(&u->wb_done, hipEventDisableTiming));
-    u->slot_event.resize(pool_size);
-    u->slot_pending.assign(pool_size, 0);
-    for (int s = 0; s < pool_size; ++s) MOLE_HIP(hipEventCreateWithFlags(&u->slot_event[s], hipEventDisableTiming));
+    if (int rc = create_members(u)) {   // nothing allocated so far outlives a failure
+        destroy_members(u);
+        return rc;
+    }
     *handle = u;
     return 0;
 }
@@ -139,19 +168,7 @@ extern "C" int mole_unimem_destroy(void *handle) {
     (void)hipSetDevice(u->device);
     (void)hipStreamSynchronize(u->tran);
     (void)hipStreamSynchronize(u->tranback);
-    for (auto &e : u->slot_event) (void)hipEventDestroy(e);
-    for (auto &t : u->timers) { (void)hipEventDestroy(t[0]); (void)hipEventDestroy(t[1]); }
-    for (auto &t : u->wb_timers) { (void)hipEventDestroy(t[0]); (void)hipEventDestroy(t[1]); }
-    (void)hipEventDestroy(u->para_event);
-    (void)hipEventDestroy(u->grads_ready);
-    (void)hipEventDestroy(u->state_free);
-    (void)hipEventDestroy(u->state_ready);
-    (void)hipEventDestroy(u->wb_done);
-    (void)hipStreamDestroy(u->tran);
-    (void)hipStreamDestroy(u->tranback);
-    for (int p = 0; p < 4; ++p)
-        if (u->pool[p]) (void)hipFree(u->pool[p]);
-    delete u;
+    destroy_members(u);
     return 0;
 }
 
@@ -182,16 +199,42 @@ extern "C" int mole_unimem_slot_ptr(void *handle, int p_id, int slot, void **out
     return 0;
 }
 
-extern "C" int mole_unimem_prefetch(void *handle, int layer, const void *const host_src[4], int base, int n) {
-    UM(handle);
+static int prefetch_impl(UniMem *u, const char *who, int layer, const void *const host_src[4], const int32_t *ids, int base, int n) {
     if (n == 0) return 0;
-    MOLE_REQUIRE(n > 0 && base >= 0 && host_src && host_src[0] && host_src[1] && host_src[2] && host_src[3],
-                 "mole_unimem_prefetch: bad arguments (base=%d n=%d)", base, n);
+    MOLE_REQUIRE(n > 0 && base >= 0 && host_src && host_src[0] && host_src[1] && host_src[2] && host_src[3] && (!ids || ids_ok(ids, n)),
+                 "%s: bad arguments (base=%d n=%d)", who, base, n);
     if (n > u->view_pool_size) {
-        set_error("mole_unimem_prefetch: %d experts do not fit the %d free pool slots", n, u->view_pool_size);
+        set_error("%s: %d experts do not fit the %d free pool slots", who, n, u->view_pool_size);
         return MOLE_E_STATE;
     }
-    if (int rc = copy_experts(u, host_src, u->virtual_offset, base, n)) return rc;
+    if (int rc = copy_experts(u, host_src, u->virtual_offset, ids, base, n)) return rc;
+    if (!u->stk.empty() && u->stk.back()[0] == layer) u->stk.back()[1] += n;
+    else u->stk.push_back({layer, n});
+    u->virtual_offset += n;
+    u->view_pool_size -= n;
+    return 0;
+}
+
+extern "C" int mole_unimem_prefetch(void *handle, int layer, const void *const host_src[4], int base, int n) {
+    UM(handle);
+    return prefetch_impl(u, "mole_unimem_prefetch", layer, host_src, nullptr, base, n);
+}
+
+extern "C" int mole_unimem_prefetch_ids(void *handle, int layer, const void *const host_src[4], const int32_t *expert_ids, int n) {
+    UM(handle);
+    MOLE_REQUIRE(n == 0 || expert_ids, "mole_unimem_prefetch_ids: null expert list");
+    return prefetch_impl(u, "mole_unimem_prefetch_ids", layer, host_src, expert_ids, 0, n);
+}
+
+extern "C" int mole_unimem_reserve(void *handle, int layer, int n, void **slot_ptrs_out) {
+    UM(handle);
+    MOLE_REQUIRE(n >= 0 && slot_ptrs_out, "mole_unimem_reserve: bad arguments (n=%d)", n);
+    if (n > u->view_pool_size) {
+        set_error("mole_unimem_reserve: %d experts do not fit the %d free pool slots", n, u->view_pool_size);
+        return MOLE_E_STATE;
+    }
+    for (int p = 0; p < 4; ++p) slot_ptrs_out[p] = u->pool_size > 0 ? u->pool[p] + (size_t)u->virtual_offset * u->slot_bytes[p] : nullptr;
+    if (n == 0) return 0;
     if (!u->stk.empty() && u->stk.back()[0] == layer) u->stk.back()[1] += n;
     else u->stk.push_back({layer, n});
     u->virtual_offset += n;
@@ -213,19 +256,32 @@ extern "C" int mole_unimem_fetch_top(void *handle, int layer, int *n_out) {
     return 0;
 }
 
+static int fetch_impl(UniMem *u, const char *who, const void *const host_src[4], int view_base, const int32_t *ids, int base, int n,
+                      int prefetched, void **slot_ptrs_out) {
+    const int slot0 = view_base + u->virtual_offset;
+    MOLE_REQUIRE(n > 0 && slot0 >= 0 && base >= 0 && prefetched >= 0 && prefetched <= n && host_src && slot_ptrs_out &&
+                     (!ids || ids_ok(ids, n)),
+                 "%s: bad arguments (view_base=%d base=%d n=%d prefetched=%d)", who, view_base, base, n, prefetched);
+    if (slot0 + n > u->pool_size) {
+        set_error("%s: slots %d..%d exceed the pool of %d", who, slot0, slot0 + n, u->pool_size);
+        return MOLE_E_STATE;
+    }
+    if (int rc = copy_experts(u, host_src, slot0 + prefetched, ids ? ids + prefetched : nullptr, base + prefetched, n - prefetched)) return rc;
+    for (int p = 0; p < 4; ++p) slot_ptrs_out[p] = u->pool[p] + (size_t)slot0 * u->slot_bytes[p];
+    return 0;
+}
+
 extern "C" int mole_unimem_fetch(void *handle, const void *const host_src[4], int view_base, int base, int n,
                                  int prefetched, void **slot_ptrs_out) {
     UM(handle);
-    const int slot0 = view_base + u->virtual_offset;
-    MOLE_REQUIRE(n > 0 && slot0 >= 0 && base >= 0 && prefetched >= 0 && prefetched <= n && host_src && slot_ptrs_out,
-                 "mole_unimem_fetch: bad arguments (view_base=%d base=%d n=%d prefetched=%d)", view_base, base, n, prefetched);
-    if (slot0 + n > u->pool_size) {
-        set_error("mole_unimem_fetch: slots %d..%d exceed the pool of %d", slot0, slot0 + n, u->pool_size);
-        return MOLE_E_STATE;
-    }
-    if (int rc = copy_experts(u, host_src, slot0 + prefetched, base + prefetched, n - prefetched)) return rc;
-    for (int p = 0; p < 4; ++p) slot_ptrs_out[p] = u->pool[p] + (size_t)slot0 * u->slot_bytes[p];
-    return 0;
+    return fetch_impl(u, "mole_unimem_fetch", host_src, view_base, nullptr, base, n, prefetched, slot_ptrs_out);
+}
+
+extern "C" int mole_unimem_fetch_ids(void *handle, const void *const host_src[4], int view_base, const int32_t *expert_ids,
+                                     int n, int prefetched, void **slot_ptrs_out) {
+    UM(handle);
+    MOLE_REQUIRE(expert_ids != nullptr, "mole_unimem_fetch_ids: null expert list");
+    return fetch_impl(u, "mole_unimem_fetch_ids", host_src, view_base, expert_ids, 0, n, prefetched, slot_ptrs_out);
 }
 
 extern "C" int mole_unimem_wait_params(void *handle, mole_stream_t compute_stream) {
@@ -261,27 +317,73 @@ extern "C" int mole_unimem_sync_tran(void *handle) {
     return 0;
 }
 
-extern "C" int mole_unimem_store_grads(void *handle, void *const host_dst[4], const void *const dev_src[4], int base,
-                                       int n, mole_stream_t compute_stream) {
-    UM(handle);
-    MOLE_REQUIRE(host_dst && dev_src && base >= 0 && n >= 0, "mole_unimem_store_grads: bad arguments base=%d n=%d", base, n);
+// Device -> host copies of n experts' arrays of the four parameter kinds on the write-back stream, after the work
+// already enqueued on compute_stream.  dev_src[p] holds the n experts back to back (every expert reads the same
+// zeroed slot when zeros is set); expert i goes to host expert ids[i] (base + i when ids is null); runs of
+// consecutive experts travel in one copy.
+static int writeback_impl(UniMem *u, const char *who, void *const host_dst[4], const void *const dev_src[4], const int32_t *ids,
+                          int base, int n, bool zeros, hipStream_t compute_stream) {
+    MOLE_REQUIRE(host_dst && (zeros || dev_src) && base >= 0 && n >= 0 && (!ids || ids_ok(ids, n)), "%s: bad arguments base=%d n=%d", who, base, n);
     if (n == 0) return 0;
     for (int p = 0; p < 4; ++p)
-        MOLE_REQUIRE(host_dst[p] && dev_src[p], "mole_unimem_store_grads: null buffer for parameter kind %d", p);
-    MOLE_HIP(hipEventRecord(u->grads_ready, (hipStream_t)compute_stream));
-    MOLE_HIP(hipStreamWaitEvent(u->tranback, u->grads_ready, 0));
+        MOLE_REQUIRE(host_dst[p] && (zeros || dev_src[p]), "%s: null buffer for parameter kind %d", who, p);
+    if (!zeros) {
+        MOLE_HIP(hipEventRecord(u->grads_ready, compute_stream));
+        MOLE_HIP(hipStreamWaitEvent(u->tranback, u->grads_ready, 0));
+    }
     std::array<hipEvent_t, 2> *tmp;
     if (int rc = next_timer(u->wb_timers, u->wb_timers_used, &tmp)) return rc;
     auto &tm = *tmp;
     MOLE_HIP(hipEventRecord(tm[0], u->tranback));
-    for (int p = 0; p < 4; ++p) {
-        const size_t sb = u->slot_bytes[p];
-        MOLE_HIP(hipMemcpyAsync((char *)host_dst[p] + (size_t)base * sb, dev_src[p], (size_t)n * sb, hipMemcpyDeviceToHost,
-                                u->tranback));
-        u->wb_bytes_open += (uint64_t)n * sb;
+    auto id_of = [&](int i) { return ids ? (int)ids[i] : base + i; };
+    for (int i = 0; i < n;) {
+        int run = 1;
+        if (!zeros) while (i + run < n && id_of(i + run) == id_of(i) + run) ++run;
+        for (int p = 0; p < 4; ++p) {
+            const size_t sb = u->slot_bytes[p];
+            const char *src = zeros ? u->zeros : (const char *)dev_src[p] + (size_t)i * sb;
+            MOLE_HIP(hipMemcpyAsync((char *)host_dst[p] + (size_t)id_of(i) * sb, src, (size_t)run * sb, hipMemcpyDeviceToHost, u->tranback));
+            u->wb_bytes_open += (uint64_t)run * sb;
+        }
+        i += run;
     }
     MOLE_HIP(hipEventRecord(tm[1], u->tranback));
     return 0;
+}
+
+extern "C" int mole_unimem_store_grads(void *handle, void *const host_dst[4], const void *const dev_src[4], int base,
+                                       int n, mole_stream_t compute_stream) {
+    UM(handle);
+    return writeback_impl(u, "mole_unimem_store_grads", host_dst, dev_src, nullptr, base, n, false, (hipStream_t)compute_stream);
+}
+
+extern "C" int mole_unimem_store_grads_ids(void *handle, void *const host_dst[4], const void *const dev_src[4],
+                                           const int32_t *expert_ids, int n, mole_stream_t compute_stream) {
+    UM(handle);
+    MOLE_REQUIRE(n == 0 || expert_ids, "mole_unimem_store_grads_ids: null expert list");
+    return writeback_impl(u, "mole_unimem_store_grads_ids", host_dst, dev_src, expert_ids, 0, n, false, (hipStream_t)compute_stream);
+}
+
+extern "C" int mole_unimem_zero_grads_ids(void *handle, void *const host_dst[4], const int32_t *expert_ids, int n) {
+    UM(handle);
+    MOLE_REQUIRE(n == 0 || expert_ids, "mole_unimem_zero_grads_ids: null expert list");
+    if (n == 0) return 0;
+    if (!u->zeros_ready) {
+        // one zeroed slot of the largest kind, made on first use and kept until the pool is destroyed; the fill runs
+        // on the write-back stream, ahead of the copies that read it
+        MOLE_HIP(hipSetDevice(u->device));
+        if (!u->zeros) {
+            hipError_t e = hipMalloc((void **)&u->zeros, u->slot_bytes[0]);
+            if (e != hipSuccess) {
+                u->zeros = nullptr;
+                set_error("mole_unimem_zero_grads_ids: hipMalloc of %zu bytes failed: %s", u->slot_bytes[0], hipGetErrorString(e));
+                return MOLE_E_NOMEM;
+            }
+        }
+        MOLE_HIP(hipMemsetAsync(u->zeros, 0, u->slot_bytes[0], u->tranback));
+        u->zeros_ready = true;
+    }
+    return writeback_impl(u, "mole_unimem_zero_grads_ids", host_dst, nullptr, expert_ids, 0, n, true, nullptr);
 }
 
 extern "C" int mole_unimem_load_state(void *handle, void *const dev_dst[], const void *const host_src[],

@@ -68,15 +68,67 @@ def gate_fwd(x: torch.Tensor, wg: torch.Tensor, logit_bias: Optional[torch.Tenso
 
 
 def gate_bwd(dgates: torch.Tensor, scores: torch.Tensor, idx: torch.Tensor, normalize_gate: bool,
-             through_softmax: bool = True) -> torch.Tensor:
-    """d(logits) (through_softmax) or d(scores) from d(gates)."""
+             through_softmax: bool = True, counts0: Optional[torch.Tensor] = None,
+             d_l_aux: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """d(logits) (through_softmax) or d(scores) from d(gates); with counts0 [E] int32 and d_l_aux [1] fp32 (both on
+    the device) the result also carries the gradient of l_aux = E/S^2 sum_e (sum_i scores[i,e]) counts0[e]."""
     _dev(dgates), _dev(scores), _dev(idx)
     S, E = scores.shape
     k = idx.shape[0]
+    if (counts0 is None) != (d_l_aux is None):
+        raise RuntimeError("gate_bwd: counts0 and d_l_aux go together")
+    if d_l_aux is not None:
+        _dev(counts0)
+        d_l_aux = _dev(d_l_aux.reshape(1).float())
     dlogits = torch.empty_like(scores)
-    L.check(L.lib().mole_gate_bwd(L.ptr(dgates), L.ptr(scores), L.ptr(idx), S, E, k, int(normalize_gate), int(through_softmax), L.ptr(dlogits),
-                                  L.stream()), "mole_gate_bwd")
+    L.check(L.lib().mole_gate_bwd(L.ptr(dgates), L.ptr(scores), L.ptr(idx), S, E, k, int(normalize_gate), int(through_softmax),
+                                  L.ptr(counts0), L.ptr(d_l_aux), L.ptr(dlogits), L.stream()), "mole_gate_bwd")
     return dlogits
+
+
+def softmax_bwd(dscores: torch.Tensor, scores: torch.Tensor) -> torch.Tensor:
+    """dlogits = scores * (dscores - sum_e dscores scores)."""
+    _dev(dscores), _dev(scores)
+    S, E = scores.shape
+    dlogits = torch.empty_like(scores)
+    L.check(L.lib().mole_softmax_bwd(L.ptr(dscores), L.ptr(scores), S, E, L.ptr(dlogits), L.stream()), "mole_softmax_bwd")
+    return dlogits
+
+
+def gemm_tn(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """c[Mo,N] = a[rows,Mo].T @ b[rows,N] in the operands' dtype."""
+    _dev(a), _dev(b)
+    rows, Mo = a.shape
+    N = b.shape[1]
+    c = torch.empty(Mo, N, dtype=a.dtype, device=a.device)
+    L.check(L.lib().mole_gemm_tn(L.ptr(a), L.ptr(b), L.dtype_code(a.dtype), rows, Mo, N, L.ptr(c), L.stream()), "mole_gemm_tn")
+    return c
+
+
+def _pad_cols(t: torch.Tensor, mult: int) -> torch.Tensor:
+    """t [rows, n] with zero columns appended up to a multiple of `mult` (a copy only when needed)."""
+    n = t.shape[1]
+    if n % mult == 0:
+        return t.contiguous()
+    out = torch.zeros(t.shape[0], (n + mult - 1) // mult * mult, dtype=t.dtype, device=t.device)
+    out[:, :n] = t
+    return out
+
+
+def gate_input_grad(dlogits: torch.Tensor, wg: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """dx [S,M] = dlogits[S,E] @ wg[E,M] in `dtype` on the grouped-GEMM tiles (the gate's share of the input
+    gradient when it is not folded into the dispatch backward).  E is padded with zeros to the tile's granule."""
+    epc = 8 if dtype == torch.bfloat16 else 4
+    M = wg.shape[1]
+    if M % epc:
+        raise RuntimeError(f"gate_input_grad: M={M} must be a multiple of {epc}")
+    a = _pad_cols(dlogits.to(dtype), epc)
+    w = wg.to(dtype)
+    if a.shape[1] != w.shape[0]:
+        wp = torch.zeros(a.shape[1], M, dtype=dtype, device=w.device)
+        wp[:w.shape[0]] = w
+        w = wp
+    return gemm_nn(a, w.contiguous())
 
 
 def gate_wgrad(dlogits: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
@@ -88,7 +140,12 @@ def gate_wgrad(dlogits: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
     M = x.shape[1]
     mfma = x.dtype == torch.bfloat16 and E <= 256 and M % 64 == 0 and S > 0
     if not mfma and (E > 32 or M % 4 != 0):
-        return (dlogits.t().to(x.dtype) @ x).float()
+        # shapes neither gate kernel takes: the transposed product of the grouped-GEMM tiles (one tile per block,
+        # the contraction over all tokens inside it), E padded to the tile's granule
+        epc = 8 if x.dtype == torch.bfloat16 else 4
+        if M % epc:
+            raise RuntimeError(f"gate_wgrad: M={M} must be a multiple of {epc}")
+        return gemm_tn(_pad_cols(dlogits.to(x.dtype), epc), x)[:E].float()
     dwg = torch.empty(E, M, dtype=torch.float32, device=x.device)
     nbytes = L.lib().mole_gate_wgrad_workspace_bytes(S, E, M)
     ws = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
@@ -158,7 +215,7 @@ def dispatch_fwd(x: torch.Tensor, row: torch.Tensor, total_rows: int, out: Optio
 def dispatch_bwd(dxd: torch.Tensor, row: torch.Tensor, dlogits: Optional[torch.Tensor] = None,
                  wg: Optional[torch.Tensor] = None) -> torch.Tensor:
     """dx = gather-sum of dxd rows (+ dlogits @ wg, the gate's share of the input gradient).  Small gates
-    are folded into the gather kernel; for larger ones the product runs first on the MFMA GEMM."""
+    are folded into the gather kernel; for larger ones the product runs first on the grouped-GEMM tiles."""
     _dev(dxd), _dev(row)
     k, S = row.shape
     M = dxd.shape[-1]
@@ -173,8 +230,8 @@ def dispatch_bwd(dxd: torch.Tensor, row: torch.Tensor, dlogits: Optional[torch.T
         if wg.dtype != torch.float32 or dlogits.dtype != torch.float32:
             raise TypeError("gate tensors are fp32")
         epc = 8 if dxd.dtype == torch.bfloat16 else 4
-        if E > 32 and E % epc == 0 and M % epc == 0:
-            dx_add = gemm_nn(dlogits.to(dxd.dtype), wg.to(dxd.dtype))
+        if E > 32 and M % epc == 0:
+            dx_add = gate_input_grad(dlogits, wg, dxd.dtype)
             dlogits, wg, E = None, None, 0
     L.check(L.lib().mole_dispatch_bwd(L.ptr(dxd), L.dtype_code(dxd.dtype), L.ptr(row), S, M, k, L.ptr(dlogits), L.ptr(wg),
                                       E, L.ptr(dx_add), L.ptr(dx), L.stream()), "mole_dispatch_bwd")

@@ -19,22 +19,27 @@ class Critical(tuple):
 
 
 class _RouteFn(torch.autograd.Function):
-    """scores [S,E] -> gates [k,S]; differentiable through the gate normalisation."""
+    """scores [S,E] -> gates [k,S] and l_aux; differentiable through the gate normalisation and through
+    l_aux = E/S^2 sum_e (sum_i scores[i,e]) counts[0,e] (tutel's gshard_loss, whose gradient the reference's
+    loss reaches through autograd)."""
 
     @staticmethod
     def forward(ctx, scores, top_k, capacity_factor, normalize_gate, alignment, layout, holder):
         r = H.route(scores.detach().contiguous(), top_k, capacity_factor, normalize_gate, alignment, layout)
         holder.append(r)
-        ctx.save_for_backward(scores, r.idx)
+        ctx.save_for_backward(scores, r.idx, r.counts)
         ctx.normalize_gate = normalize_gate
         ctx.mark_non_differentiable(r.idx, r.loc)
-        return r.gates, r.idx, r.loc
+        return r.gates, r.idx, r.loc, r.l_aux[0].clone()
 
     @staticmethod
-    def backward(ctx, dgates, _di, _dl):
-        scores, idx = ctx.saved_tensors
+    def backward(ctx, dgates, _di, _dl, d_l_aux):
+        scores, idx, counts = ctx.saved_tensors
+        if dgates is None:
+            dgates = torch.zeros(idx.shape, dtype=torch.float32, device=scores.device)
+        aux = {} if d_l_aux is None else dict(counts0=counts[0].contiguous(), d_l_aux=d_l_aux)
         dscores = H.gate_bwd(dgates.contiguous(), scores.detach().contiguous(), idx, ctx.normalize_gate,
-                             through_softmax=False)
+                             through_softmax=False, **aux)
         return dscores, None, None, None, None, None, None
 
 
@@ -50,8 +55,8 @@ def extract_critical(scores, top_k, loss_fn=None, capacity_factor=1.0, batch_pri
     S, E = scores.shape
     k = min(int(top_k), E)
     holder = []
-    gates, idx, loc = _RouteFn.apply(scores.float(), k, float(capacity_factor), bool(normalize_gate), int(alignment),
-                                     int(layout), holder)
+    gates, idx, loc, l_aux_diff = _RouteFn.apply(scores.float(), k, float(capacity_factor), bool(normalize_gate),
+                                                 int(alignment), int(layout), holder)
     r = holder[0]
     if capacity_factor > 0:
         cap = k * int(capacity_factor * ((S + E - 1) // E))
@@ -62,7 +67,7 @@ def extract_critical(scores, top_k, loss_fn=None, capacity_factor=1.0, batch_pri
     crit = Critical((E, [idx[j] for j in range(k)], [loc[j] for j in range(k)], [gates[j] for j in range(k)], cap))
     crit.route = r
     crit.gates = gates
-    l_aux = r.l_aux[0] if loss_fn is None else loss_fn(scores, idx.t())
+    l_aux = l_aux_diff if loss_fn is None else loss_fn(scores, idx.t())
     return crit, l_aux
 
 

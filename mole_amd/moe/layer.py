@@ -12,7 +12,9 @@ Two execution shapes, same results:
 
 New, optional keyword arguments (all defaulting to the reference's behaviour): dtype,
 normalize_gate, gelu_bwd ("tanh" = the derivative the reference compiles, MOLE/cpp/define.hpp:6;
-"exact" = erf derivative), gate_logit_bias, reference_layout.
+"exact" = erf derivative), gate_logit_bias, reference_layout, activated_only (offloaded experts that
+received no token are neither copied to the pool nor launched; False restores the reference's
+every-expert-in-index-order behaviour).
 """
 import time
 
@@ -23,7 +25,7 @@ from .. import core
 from .. import hip_ops as H
 from ..core import BatchFusedFWD, MOLECore
 from ..utils import Ugate
-from ..utils.Uparam import CPUHostBatchedParameter, GPUHostBatchedParameter
+from ..utils.Uparam import CPUHostBatchedParameter, GPUHostBatchedParameter, UnifiedCPUTensor
 from . import fast_dispatch as tutel_fast_dispatcher
 
 
@@ -65,20 +67,22 @@ class _FusedMoE(torch.autograd.Function):
         xd = H.dispatch_fwd(x, r.row, max(rows, 1))
         out, saved = m.MOLECore.forward(xd, True, r.offsets, r.kept_rows, return_saved=True)
         y = H.combine_fwd(out, r.row, r.gates)
-        m.l_aux = r.l_aux[0]
         m.last_route = r
         ctx.m, ctx.r, ctx.saved = m, r, saved
         ctx.save_for_backward(x, wg, scores, out)
-        return y
+        return y, r.l_aux[0].clone()
 
     @staticmethod
-    def backward(ctx, dy):
+    def backward(ctx, dy, d_l_aux):
         m, r = ctx.m, ctx.r
         x, wg, scores, out = ctx.saved_tensors
         d_o, dgates = H.combine_bwd(dy.contiguous(), out, r.row, r.gates)
         gxd = m.MOLECore.backward(d_o, saved=ctx.saved)
         ctx.saved = None
-        dlogits = H.gate_bwd(dgates, scores, r.idx, m.normalize_gate, through_softmax=True)
+        # l_aux reaches the gate only when the caller added it to the loss (an unused output arrives as zeros,
+        # which costs nothing: the term rides along in the same kernel)
+        aux = {} if d_l_aux is None else dict(counts0=r.counts[0], d_l_aux=d_l_aux)
+        dlogits = H.gate_bwd(dgates, scores, r.idx, m.normalize_gate, through_softmax=True, **aux)
         wg32 = wg.detach().float().contiguous()
         dx = H.dispatch_bwd(gxd, r.row, dlogits, wg32)
         dwg = H.gate_wgrad(dlogits, x).to(wg.dtype)
@@ -99,7 +103,8 @@ class MOLEModule(torch.nn.Module):
     def __init__(self, total_d_experts, total_s_experts, embed_dim, ffn_dim, pool_size, topk, ebatch_size, dist, act,
                  acc_step, adv_adam, use_pool, pool_for_extra=[False, False, False], overlap=True,
                  gate_control_by_umoe=True, hybrid_adam=False, device_s_experts=-1, dtype=torch.float32,
-                 normalize_gate=True, gelu_bwd="tanh", gate_logit_bias=None, reference_layout=False):
+                 normalize_gate=True, gelu_bwd="tanh", gate_logit_bias=None, reference_layout=False,
+                 activated_only=True):
         super().__init__()
         if not torch.cuda.is_available():
             raise RuntimeError("MOLEModule needs an MI355X: the expert path exists only as HIP kernels")
@@ -122,7 +127,8 @@ class MOLEModule(torch.nn.Module):
         self.MOLECore = MOLECore(use_pool, pool_for_extra[0], pool_for_extra[1], pool_for_extra[2],
                                  total_s_experts // self.world_size, total_d_experts // self.world_size, ebatch_size,
                                  dist["world_size"], act, adv_adam, acc_step, 0, dist["local_rank"],
-                                 len(MOLEModule._instance), total_d_experts + total_s_experts, gelu_bwd=gelu_bwd)
+                                 len(MOLEModule._instance), total_d_experts + total_s_experts, gelu_bwd=gelu_bwd,
+                                 activated_only=activated_only)
 
         # only EP = DP; on one GPU every expert is local
         self.d_experts = total_d_experts // self.world_size
@@ -156,6 +162,10 @@ class MOLEModule(torch.nn.Module):
                                                  transposed=True, **gp)
         self.FC2_B_GPU = GPUHostBatchedParameter(size=[embed_dim], count=self.s_experts, bias=True, p_id=3,
                                                  fan_in=ffn_dim, **gp)
+        # device_s_experts > 0: the offloaded experts of all layers share one pinned host pool (layer.py:98-100)
+        UnifiedCPUTensor()
+        UnifiedCPUTensor.init([[ffn_dim, embed_dim], [ffn_dim], [ffn_dim, embed_dim], [embed_dim]], device_s_experts,
+                              dtype, with_adam_state=bool(adv_adam))
         cp = dict(dtype=dtype, moe=self.MOLECore, device_s_experts=device_s_experts)
         self.FC1_W_CPU = CPUHostBatchedParameter(size=[ffn_dim, embed_dim], count=self.d_experts, p_id=0, **cp)
         self.FC1_B_CPU = CPUHostBatchedParameter(size=[ffn_dim], count=self.d_experts, p_id=1, bias=True,
@@ -240,8 +250,8 @@ class MOLEModule(torch.nn.Module):
             experts_output = BatchFusedFWD.apply(dispatched_input, self, self.dummy_param, time_it, prefetch)
             expert_output = tutel_fast_dispatcher.fast_decode(data=experts_output, critial_data=crit)
         else:
-            expert_output = _FusedMoE.apply(resized_input, self.gate[0].linear.weight, self.dummy_param, self,
-                                            float(capacity_factor))
+            expert_output, self.l_aux = _FusedMoE.apply(resized_input, self.gate[0].linear.weight, self.dummy_param,
+                                                        self, float(capacity_factor))
 
         expert_output = expert_output.reshape(original_shape)
         out = expert_output.to(original_dtype)
@@ -265,6 +275,9 @@ class MOLEModule(torch.nn.Module):
     def unset_lazy_zero(self):
         for p in (self.FC1_W_CPU, self.FC1_B_CPU, self.FC2_W_CPU, self.FC2_B_CPU):
             p.unset_lazy_zero()
+
+    def set_lazy_zero(self):
+        self.MOLECore.set_lazy_zero()
 
     # ---- layer state for checkpoints (layer.py:350-427) ------------------------------------------
     def _expert_stores(self):
@@ -316,6 +329,7 @@ class MOLEModule(torch.nn.Module):
                     for st, t in zip(self._expert_stores(), gs[j]):
                         st[which].fetch_single_grad(i).copy_(t)
                     j += 1
+            self.MOLECore.host_gradients_changed()
             lin.weight.grad = None if gs[j] is None else gs[j].to(lin.weight.device)
             if lin.bias is not None and gs[j + 1] is not None:
                 lin.bias.grad = gs[j + 1].to(lin.bias.device)
@@ -342,3 +356,4 @@ class MOLEModule(torch.nn.Module):
         """Forget all layers and free the process-global slot pool (tests, benchmarks)."""
         cls._instance = []
         core.destroy_UniMem()
+        UnifiedCPUTensor.reset()

@@ -2,8 +2,9 @@
 
 Mirror of MOLE/utils/Ugate.py:5-14 (same class name, same `linear` attribute).  For bf16 tokens the scores
 come from one fused kernel of the C ABI (mole_gate_fwd); otherwise the logits come from the MFMA NT GEMM
-(mole_gemm_nt) and the softmax from mole_softmax_fwd.  The backward is the textbook softmax/linear
-backward on device tensors.  `logit_bias` ([E], optional, not trained) is
+(mole_gemm_nt) and the softmax from mole_softmax_fwd.  The backward is the softmax/linear backward in the
+same library: mole_softmax_bwd, then dlogits . Wg and dlogits^T . x on the grouped-GEMM tiles / the gate
+weight-gradient kernel.  `logit_bias` ([E], optional, not trained) is
 added to the logits before the softmax - the reference gate has none.
 """
 import torch
@@ -21,9 +22,10 @@ class _GateFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dscores):
         x, weight, scores = ctx.saved_tensors
-        dlogits = scores * (dscores - (dscores * scores).sum(dim=-1, keepdim=True))
-        dx = (dlogits @ weight).to(x.dtype) if ctx.needs_input_grad[0] else None
-        dw = (dlogits.t().to(x.dtype) @ x).to(weight.dtype) if ctx.needs_input_grad[1] else None
+        dlogits = H.softmax_bwd(dscores.float().contiguous(), scores)
+        xc = x.detach().contiguous()
+        dx = H.gate_input_grad(dlogits, weight.detach().float(), x.dtype) if ctx.needs_input_grad[0] else None
+        dw = H.gate_wgrad(dlogits, xc).to(weight.dtype) if ctx.needs_input_grad[1] else None
         return dx, dw, None
 
 

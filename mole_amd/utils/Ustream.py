@@ -1,10 +1,11 @@
 """Stream roles of the expert pipeline.
 
 Mirror of MOLE/utils/Ustream.py:6-73 and MOLE/cpp/stream.cpp:84-144.  The reference owns 16 streams
-and makes stream 2 ("comp") torch's current stream; here compute simply stays on torch's current
-stream and the only extra stream is the slot pool's copy stream ("tran"), created at default
-priority by mole_unimem_create.  comm / tranback have no work on one GPU and alias the compute
-stream.
+and makes stream 2 ("comp") torch's current stream; here compute stays on torch's current stream and
+the slot pool owns the two copy streams, both created at default priority by mole_unimem_create:
+"tran" (host -> pool prefetches and state loads) and "tranback" (gradient / parameter / moment
+write-backs).  "comm" has no work on one GPU and is the compute stream.  With multi-stream switched
+off (core.disable_multi_stream, stream.cpp:84-95) every role hands out the compute stream.
 """
 import torch
 
@@ -20,24 +21,34 @@ class ExpertStreamCtx(object):
             cls._instance.disable = kw.get("disable", False)
             cls._instance.device = kw.get("device", "cuda:0")
             cls._instance.default = torch.cuda.current_stream(device=cls._instance.device)
+            if cls._instance.disable:
+                core.disable_multi_stream()
         return cls._instance
 
     def __init__(self, *args, **kw):
         pass
 
     @staticmethod
-    def tran_stream():
+    def _pool_stream(handle_of):
         um = core.get_UniMem()
-        if um is None or ExpertStreamCtx._instance.disable:
+        inst = ExpertStreamCtx._instance
+        if um is None or inst.disable or not core.multi_stream_enabled():
             return ExpertStreamCtx.comp_stream()
-        return torch.cuda.ExternalStream(um.tran_stream_handle(), device=ExpertStreamCtx._instance.device)
+        return torch.cuda.ExternalStream(handle_of(um), device=inst.device)
+
+    @staticmethod
+    def tran_stream():
+        return ExpertStreamCtx._pool_stream(lambda um: um.tran_stream_handle())
+
+    @staticmethod
+    def tran_back_stream():
+        return ExpertStreamCtx._pool_stream(lambda um: um.tranback_stream_handle())
 
     @staticmethod
     def comp_stream():
         return torch.cuda.current_stream(device=ExpertStreamCtx._instance.device)
 
     comm_stream = comp_stream
-    tran_back_stream = comp_stream
 
     @staticmethod
     def default_stream():

@@ -206,6 +206,14 @@ def gshard_loss(scores: np.ndarray, top1_idx: np.ndarray) -> float:
     return float((me * ce).sum() * (E / (S * S)))
 
 
+def gshard_loss_bwd(S: int, counts0: np.ndarray, d_l_aux: float = 1.0) -> torch.Tensor:
+    """d l_aux / d scores, [S,E]: E/S^2 * counts0[e] for every token (the counts are integers and carry no
+    gradient; tutel detaches them the same way by building them from the top-k indices)."""
+    E = len(counts0)
+    row = torch.from_numpy(np.asarray(counts0, dtype=np.float64)) * (d_l_aux * E / (S * S))
+    return row.unsqueeze(0).expand(S, E).clone()
+
+
 # --------------------------------------------------------------------------------------------
 # A7 / A8  dispatch (encode) and combine (decode), forward and backward
 # --------------------------------------------------------------------------------------------
@@ -411,13 +419,15 @@ class LayerResult:
 
 def moe_layer(x, wg, w1, b1, w2, b2, top_k: int, capacity_factor: float = 1.0, dy=None,
               logit_bias=None, normalize_gate: bool = True, gelu_bwd: str = "tanh",
-              scores_override=None) -> LayerResult:
+              scores_override=None, d_l_aux: float = 0.0) -> LayerResult:
     """One MoE layer forward (and backward when dy is given) on the ragged layout.
 
     The ragged layout computes exactly the kept rows; the reference's padded [E,C,M] layout gives
     the same y and the same gradients because padded rows are never read by decode and receive
     zero output gradient (tests pin that equivalence).  `scores_override` lets a test feed the
-    scores produced on the GPU so that routing is compared bit for bit on identical inputs.
+    scores produced on the GPU so that routing is compared bit for bit on identical inputs.  d_l_aux is the
+    weight with which l_aux enters the loss (loss = <dy, y> + d_l_aux * l_aux): its gradient reaches dx and dwg
+    through the scores.
     """
     scores = gate_scores(x, wg, logit_bias) if scores_override is None else scores_override
     crit = extract_critical(scores.detach().numpy(), top_k, capacity_factor, normalize_gate)
@@ -431,6 +441,8 @@ def moe_layer(x, wg, w1, b1, w2, b2, top_k: int, capacity_factor: float = 1.0, d
     g_w1, g_b1, g_w2, g_b2, gxd = ffn_bwd_ragged(do, xd, x1, crit.offsets, w1, w2, gelu_bwd)
     dx = fast_encode_bwd(gxd, crit, ragged=True)
     dscores = gate_normalize_bwd(dgates, scores, crit, normalize_gate)
+    if d_l_aux != 0.0 and x.shape[0] > 0:
+        dscores = dscores + gshard_loss_bwd(x.shape[0], crit.counts[0], d_l_aux).to(dscores.dtype)
     dlogits = softmax_bwd(dscores, scores)
     dx = dx + dlogits @ wg
     res.dx, res.dwg = dx, dlogits.t() @ x
@@ -487,10 +499,17 @@ class UniMemModel:
 
 
 def plan_offloaded_chunks(d_experts: int, ebatch_size: int, use_pool: bool, view_pool_size: int,
-                          prefetched: int):
+                          prefetched: int, as_reference: bool = False):
     """Chunking of the offloaded experts of one layer into batch records and launch groups
     (core.cpp:1020-1051).  Returns a list of groups, each a list of
-    (expert_base, size, already_prefetched, view_base)."""
+    (expert_base, size, already_prefetched, view_base).
+
+    as_reference=True restates the reference literally.  It wraps view_base to 0 whenever the next chunk does not
+    fit the visible pool, also while that chunk still holds prefetched experts (core.cpp:1026-1046), which then
+    are looked for in slots that hold other experts - e.g. (d=6, ebatch=2, pool=5, prefetched=5) yields the chunk
+    (4, 2, 1, 0): expert 4 is taken to be in slot 0, which holds expert 0.  The default cuts such a chunk at the
+    end of the visible pool instead, so that prefetched experts are always used where they lie;
+    simulate_chunk_slots() checks exactly that."""
     groups, cur = [], []
     d_batch = min(ebatch_size, 10000 if not use_pool else view_pool_size)
     view_base = 0
@@ -498,16 +517,36 @@ def plan_offloaded_chunks(d_experts: int, ebatch_size: int, use_pool: bool, view
     while i < d_experts:
         size = min(d_batch, d_experts - i)
         if use_pool and view_pool_size - view_base < size:
-            view_base = 0
-            groups.append(cur)
-            cur = []
+            if i < prefetched and not as_reference:
+                size = view_pool_size - view_base
+            else:
+                view_base = 0
+                groups.append(cur)
+                cur = []
         cur_pref = min(size, prefetched - i) if prefetched > i else 0
         cur.append((i, size, cur_pref, view_base))
         view_base += size
-        i += d_batch
+        i += d_batch if as_reference else size
     if cur:
         groups.append(cur)
     return groups
+
+
+def simulate_chunk_slots(chunks, prefetched: int, pool_size: int) -> bool:
+    """Plays a chunk plan [(expert_base, size, already_prefetched, view_base)] against the slot pool: slots
+    0..prefetched-1 start out holding experts 0..prefetched-1, each chunk copies its not-yet-prefetched experts
+    into its slots and then runs on what the slots hold.  True iff every chunk finds exactly its own experts."""
+    slots = [None] * pool_size
+    for e in range(prefetched):
+        slots[e] = e
+    for (base, size, pref, vb) in chunks:
+        if vb < 0 or vb + size > pool_size:
+            return False
+        for j in range(pref, size):
+            slots[vb + j] = base + j
+        if any(slots[vb + j] != base + j for j in range(size)):
+            return False
+    return True
 
 
 def fast_assign_prefetch(P: int, Fv: Sequence[int], Ev: Sequence[int]):

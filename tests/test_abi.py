@@ -72,7 +72,9 @@ def test_every_entry_point_rejects_bad_arguments_on_the_host():
         ("mole_gate_fwd", lambda: lib.mole_gate_fwd(ok, L.MOLE_F32, ok, None, 10, 64, 128, ok, None)),      # fp32: E <= 32
         ("mole_gate_fwd", lambda: lib.mole_gate_fwd(bad16, L.MOLE_F32, ok, None, 10, 8, 128, ok, None)),    # fp32: alignment
         ("mole_gate_fwd", lambda: lib.mole_gate_fwd(ok, L.MOLE_BF16, ok, None, 10, 8, 100, ok, None)),
-        ("mole_gate_bwd", lambda: lib.mole_gate_bwd(ok, ok, ok, 10, 4, 5, 1, 1, ok, None)),
+        ("mole_softmax_bwd", lambda: lib.mole_softmax_bwd(ok, ok, 10, 0, ok, None)),
+        ("mole_gate_bwd", lambda: lib.mole_gate_bwd(ok, ok, ok, 10, 4, 5, 1, 1, None, None, ok, None)),
+        ("mole_gate_bwd", lambda: lib.mole_gate_bwd(ok, ok, ok, 10, 4, 2, 1, 1, ok, None, ok, None)),      # counts0 without d_l_aux
         ("mole_gate_wgrad", lambda: lib.mole_gate_wgrad(ok, ok, L.MOLE_F32, 10, 64, 128, ok, ok, 1 << 30, None)),
         ("mole_gate_wgrad", lambda: lib.mole_gate_wgrad(ok, ok, L.MOLE_BF16, 10, 8, 128, ok, ok, 16, None)),
         ("mole_route", lambda: lib.mole_route(ok, 10, 4, 5, 1.0, 1, 1, 1, ok, ok, ok, ok, ok, ok, ok, ok, ok, ok, 1 << 20, None)),
@@ -87,11 +89,17 @@ def test_every_entry_point_rejects_bad_arguments_on_the_host():
         ("mole_ffn_bwd", lambda: lib.mole_ffn_bwd(ok, ok, ok, ok, 5, ok, ok, 2, 16, 16, 16, ok, ok, ok, ok, ok, ok, ok, ok, 0, 0, None)),
         ("mole_gemm_nt", lambda: lib.mole_gemm_nt(ok, ok, 4, 16, 16, 16, ok, None)),
         ("mole_gemm_nn", lambda: lib.mole_gemm_nn(ok, ok, 4, 16, 16, 16, ok, None)),
+        ("mole_gemm_tn", lambda: lib.mole_gemm_tn(ok, ok, L.MOLE_F32, 16, 6, 16, ok, None)),                  # Mo % 4
         ("mole_adam_step", lambda: lib.mole_adam_step(ok, ok, ok, ok, ok, 64, L.MOLE_F32, 0.9, 0.999, 0, 1e-3, 0.0, 1e-8, 0, None)),
         ("mole_adam_step", lambda: lib.mole_adam_step(ok, bad16, ok, ok, ok, 64, L.MOLE_BF16, 0.9, 0.999, 1, 1e-3, 0.0, 1e-8, 0, None)),
         ("mole_adam_step", lambda: lib.mole_adam_step(ok, ok, ok, ok, ok, 64, L.MOLE_F32, 1.0, 0.999, 1, 1e-3, 0.0, 1e-8, 0, None)),
         ("mole_unimem_prefetch", lambda: lib.mole_unimem_prefetch(None, 0, None, 0, 1)),
         ("mole_unimem_fetch", lambda: lib.mole_unimem_fetch(None, None, 0, 0, 1, 0, None)),
+        ("mole_unimem_prefetch_ids", lambda: lib.mole_unimem_prefetch_ids(None, 0, None, None, 1)),
+        ("mole_unimem_fetch_ids", lambda: lib.mole_unimem_fetch_ids(None, None, 0, None, 1, 0, None)),
+        ("mole_unimem_reserve", lambda: lib.mole_unimem_reserve(None, 0, 1, None)),
+        ("mole_unimem_store_grads_ids", lambda: lib.mole_unimem_store_grads_ids(None, None, None, None, 1, None)),
+        ("mole_unimem_zero_grads_ids", lambda: lib.mole_unimem_zero_grads_ids(None, None, None, 1)),
         ("mole_unimem_store_grads", lambda: lib.mole_unimem_store_grads(None, None, None, 0, 1, None)),
         ("mole_unimem_load_state", lambda: lib.mole_unimem_load_state(None, None, None, None, 1, 0, None)),
         ("mole_unimem_store_state", lambda: lib.mole_unimem_store_state(None, None, None, None, 1, None)),

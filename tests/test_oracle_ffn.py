@@ -108,7 +108,8 @@ def test_whole_layer_against_dense_autograd(k, cf):
     w1, b1 = torch.randn(E, Fd, M, dtype=dt) * 0.2, torch.randn(E, Fd, dtype=dt) * 0.1
     w2, b2 = torch.randn(E, Fd, M, dtype=dt) * 0.2, torch.randn(E, M, dtype=dt) * 0.1
     dy = torch.randn(S, M, dtype=dt)
-    res = O.moe_layer(x, wg, w1, b1, w2, b2, k, cf, dy=dy, gelu_bwd="exact")
+    aux_w = 0.7 * k                      # the load-balancing loss enters the loss with this weight
+    res = O.moe_layer(x, wg, w1, b1, w2, b2, k, cf, dy=dy, gelu_bwd="exact", d_l_aux=aux_w)
     crit = res.crit
     # dense autograd version
     leaves = [t.clone().requires_grad_(True) for t in (x, wg, w1, b1, w2, b2)]
@@ -128,7 +129,12 @@ def test_whole_layer_against_dense_autograd(k, cf):
             y = y + F.one_hot(torch.tensor(i), S).to(dt)[:, None] * (gates[j, i] * (F.gelu(h) @ w2q[e] + b2q[e]))[None, :]
     # gates pass through fp32 inside extract_critical (as in the reference), hence 1e-6
     torch.testing.assert_close(res.y, y.detach(), rtol=1e-6, atol=1e-7)
-    (y * dy).sum().backward()
+    # l_aux by its definition (mean score per expert times the fraction of first choices, times E), differentiable
+    # in the scores only: autograd through it pins gshard_loss_bwd, a term the layer's own loss does not exercise
+    frac = torch.bincount(idx[0], minlength=E).to(dt) / S
+    l_aux = E * (scores.mean(dim=0) * frac).sum()
+    assert abs(float(l_aux.detach()) - crit.l_aux) < 1e-6
+    ((y * dy).sum() + aux_w * l_aux).backward()
     for got, leaf in zip((res.dx, res.dwg, res.g_w1, res.g_b1, res.g_w2, res.g_b2), leaves):
         torch.testing.assert_close(got, leaf.grad, rtol=1e-5, atol=1e-6)
 
@@ -172,6 +178,34 @@ def test_chunk_plan_covers_every_expert_once_and_respects_the_pool():
                 seen += list(range(base, base + size))
                 assert p == max(0, min(size, pref - base))
         assert seen == list(range(d))
+
+
+def test_chunk_plans_use_prefetched_experts_where_they_lie():
+    """Brute force over (experts, batch, pool, prefetched): played against a model of the slots, every chunk of
+    the oracle's plan and of the product's plan finds its own experts in its slots; the literal reference plan
+    does not (two hand-checked cases), which is why neither follows it there."""
+    from mole_amd import core
+    bad_ref = 0
+    for d, eb, pool in itertools.product(range(0, 9), range(1, 6), range(1, 8)):
+        for pref in range(0, min(d, pool) + 1):
+            flat = [c for g in O.plan_offloaded_chunks(d, eb, True, pool, pref) for c in g]
+            assert O.simulate_chunk_slots(flat, pref, pool), (d, eb, pool, pref, flat)
+            assert [e for (b, n, _, _) in flat for e in range(b, b + n)] == list(range(d))
+            mine = core.plan_chunks(d, pref, pool, eb)
+            assert O.simulate_chunk_slots(mine, pref, pool), (d, eb, pool, pref, mine)
+            assert [e for (b, n, _, _) in mine for e in range(b, b + n)] == list(range(d))
+            for (b, n, p, vb) in mine:
+                assert n <= min(eb, pool) and (p == 0 or vb == b)
+            ref = [c for g in O.plan_offloaded_chunks(d, eb, True, pool, pref, as_reference=True) for c in g]
+            bad_ref += not O.simulate_chunk_slots(ref, pref, pool)
+    assert bad_ref > 0
+    ref = [c for g in O.plan_offloaded_chunks(6, 2, True, 5, 5, as_reference=True) for c in g]
+    assert (4, 2, 1, 0) in ref and not O.simulate_chunk_slots(ref, 5, 5)
+    ref = [c for g in O.plan_offloaded_chunks(6, 3, True, 4, 4, as_reference=True) for c in g]
+    assert (3, 3, 1, 0) in ref and not O.simulate_chunk_slots(ref, 4, 4)
+    assert core.plan_chunks(6, 5, 5, 2) == [(0, 2, 2, 0), (2, 2, 2, 2), (4, 1, 1, 4), (5, 1, 0, 0)]
+    with pytest.raises(RuntimeError):
+        core.plan_chunks(3, 0, 0, 2)
 
 
 def _brute_assign_ok(P, Fv, Ev, gp, lp):
