@@ -270,3 +270,61 @@ def test_ffn_fine_grained_full_size_against_fp32_products():
         assert rel_err(gx[lo:hi], t32 @ w1[e].float()) < t
         assert rel_err(g_b1[e], t32.sum(0)) < t
         assert rel_err(g_b2[e], go32.sum(0)) < t
+
+
+def _bf16_grid(limit=8.0, min_exp=-14):
+    """Every bf16 value v with 2^min_exp <= |v| <= limit, and zero."""
+    bits = torch.arange(0, 1 << 15, dtype=torch.int32)
+    v = (bits << 16).view(torch.float32)
+    v = v[torch.isfinite(v) & (v <= limit) & (v >= 2.0 ** min_exp)]
+    return torch.cat([torch.zeros(1), v, -v])
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_fused_activation_math_on_a_dense_grid(dtype):
+    """The GELU of the forward epilogue and both GELU derivatives of the backward epilogue, pinned through the
+    FFN entry points themselves on every bf16 value of magnitude 2^-14 .. 8 (about 4400 points): one-hot rows in
+    w1 make h an exact copy of xd, one-hot rows in w2 make go . w2^T exactly 1, so a = gelu(h) and t = gelu'(h)
+    rounded once to the buffer dtype.  bf16 results come from polynomial fits (stated absolute error 6e-5 for the
+    GELU's erf part, 2e-4 for the derivatives); the bound is that error plus the rounding of the result (half an
+    ulp of bf16: 2^-9 relative).  fp32 results come from the closed forms and are held to 2e-6."""
+    from mole_amd import hip_ops as H, _lib as L
+    grid = _bf16_grid()
+    M, Fd = 64, 256
+    rows = (grid.numel() + M - 1) // M
+    vals = torch.zeros(rows * M)
+    vals[:grid.numel()] = grid
+    xd = vals.view(rows, M).to(dtype).cuda()
+    w1 = torch.zeros(1, Fd, M)
+    w1[0, torch.arange(Fd), torch.arange(Fd) % M] = 1.0          # h[r, f] = xd[r, f mod M]
+    w2 = torch.zeros(1, Fd, M)
+    w2[0, :, 0] = 1.0                                             # (go . w2^T)[r, f] = go[r, 0]
+    b1, b2 = torch.zeros(1, Fd), torch.zeros(1, M)
+    go = torch.zeros(rows, M)
+    go[:, 0] = 1.0
+    off = torch.tensor([0, rows], dtype=torch.int32).cuda()
+    n = torch.tensor([rows], dtype=torch.int32).cuda()
+    dev = lambda t: t.to(dtype).cuda()
+    w1d, w2d = dev(w1), dev(w2)
+    out, h, a = H.ffn_fwd(xd, off, n, w1d, dev(b1), w2d, dev(b2))
+    h64 = xd.double().cpu().repeat(1, Fd // M)
+    assert torch.equal(h.double().cpu(), h64)                     # the set-up: h is xd, exactly
+    gelu64 = 0.5 * h64 * (1.0 + torch.erf(h64 / 2.0 ** 0.5))
+    half_ulp = 2.0 ** -9 if dtype == torch.bfloat16 else 2.0 ** -24
+    poly = 6e-5 if dtype == torch.bfloat16 else 2e-6
+    err = (a.double().cpu() - gelu64).abs()
+    bound = poly * torch.clamp(h64.abs(), min=1.0) + half_ulp * gelu64.abs() * 1.01 + 1e-30
+    worst = float((err - half_ulp * gelu64.abs()).max())
+    print(f"fused GELU {dtype}: worst error beyond rounding {worst:.2e}", flush=True)
+    assert bool((err <= bound).all()), f"GELU off by {float((err / bound).max()):.2f}x its bound"
+    for variant, fn, code in (("tanh", O.d_gelu_tanh, L.GELU_BWD_TANH), ("exact", O.d_gelu_exact, L.GELU_BWD_EXACT)):
+        g_w1, g_b1, g_w2, g_b2 = (torch.empty_like(t) for t in (w1d, dev(b1), w2d, dev(b2)))
+        t = torch.empty(rows, Fd, dtype=dtype, device="cuda")
+        H.ffn_bwd_into(dev(go), xd, h, a, off, n, 1, rows, M, Fd, w1d, w2d, t, g_w1, g_b1, g_w2, g_b2, None, False, code)
+        d64 = fn(h64)
+        err = (t.double().cpu() - d64).abs()
+        polyd = 2e-4 if dtype == torch.bfloat16 else 2e-6
+        bound = polyd + half_ulp * d64.abs() * 1.01
+        worst = float((err - half_ulp * d64.abs()).max())
+        print(f"fused GELU' ({variant}) {dtype}: worst error beyond rounding {worst:.2e}", flush=True)
+        assert bool((err <= bound).all()), f"GELU' ({variant}) off by {float((err / bound).max()):.2f}x its bound"

@@ -48,13 +48,20 @@ def _grads(m, E):
     return out
 
 
-def _run_and_compare(m, x, ref, k, cf, dtype, gelu_bwd="tanh", normalize=True):
+def _run_and_compare(m, x, ref, k, cf, dtype, gelu_bwd="tanh", normalize=True, aux_w=0.0):
+    """aux_w: weight of the load-balancing loss in the loss (loss = mean(y^2) + aux_w * l_aux)."""
+    from mole_amd import core
     from mole_amd.utils import Ugate
     x = x.clone().requires_grad_(True)
     y = m(x, capacity_factor=cf)
     dy = (2.0 * y.detach().float() / y.numel()).to(dtype)       # d/dy of mean(y^2): the MSE-vs-zero loss
-    y.backward(dy)
+    if aux_w:
+        assert m.l_aux.requires_grad
+        torch.autograd.backward([y, m.l_aux], [dy, torch.tensor(aux_w, device=y.device)])
+    else:
+        y.backward(dy)
     torch.cuda.synchronize()
+    core.synchronize_tran()                # gradients of offloaded experts are on their way to the host
     t = tol(dtype)
     # gate scores: GPU vs oracle within tolerance; then the oracle re-routes on the GPU's own scores so that
     # every routing decision is compared on identical inputs
@@ -62,7 +69,8 @@ def _run_and_compare(m, x, ref, k, cf, dtype, gelu_bwd="tanh", normalize=True):
     bias = m.gate[0].logit_bias.cpu() if m.gate[0].logit_bias is not None else None
     assert rel_err(scores_gpu, O.gate_scores(ref["x"], ref["wg"], bias)) < (1e-5 if dtype == torch.float32 else 2e-2)
     res = O.moe_layer(ref["x"], ref["wg"], ref["w1"], ref["b1"], ref["w2"], ref["b2"], k, cf, dy=dy.float().cpu(),
-                      logit_bias=bias, normalize_gate=normalize, gelu_bwd=gelu_bwd, scores_override=scores_gpu)
+                      logit_bias=bias, normalize_gate=normalize, gelu_bwd=gelu_bwd, scores_override=scores_gpu,
+                      d_l_aux=aux_w)
     assert rel_err(y, res.y) < t
     assert rel_err(x.grad, res.dx) < t
     assert rel_err(m.gate[0].linear.weight.grad, res.dwg) < t
@@ -85,12 +93,31 @@ def test_layer_static_experts(S, M, E, k, Fd, cf, reference_layout, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("d_experts,pool,ebatch,prefetch_n", [(8, 8, 4, 0), (6, 3, 2, 0), (8, 5, 2, 3), (4, 2, 4, 2)])
-def test_layer_offloaded_experts(d_experts, pool, ebatch, prefetch_n, dtype):
-    """Some or all experts live in pinned host memory and stream through a pool smaller than the layer."""
-    print(f"layer offload d={d_experts} pool={pool} ebatch={ebatch} prefetch={prefetch_n} {dtype}", flush=True)
+@pytest.mark.parametrize("reference_layout", [False, True])
+def test_layer_l_aux_carries_a_gradient(reference_layout, dtype):
+    """loss = mean(y^2) + w * l_aux: the load-balancing term reaches the gate weight and the input through the
+    scores (d l_aux / d scores[i,e] = E/S^2 counts0[e]), in both execution shapes of the module; the oracle's
+    version of that term is pinned against autograd in tests/test_oracle_ffn.py."""
+    print(f"layer l_aux gradient ref_layout={reference_layout} {dtype}", flush=True)
+    m, x, ref = _build(500, 64, 8, 2, 128, dtype, reference_layout=reference_layout, seed=4)
+    res0 = _run_and_compare(m, x, ref, 2, 1.0, dtype)
+    m.gate[0].linear.weight.grad = None
+    res1 = _run_and_compare(m, x, ref, 2, 1.0, dtype, aux_w=25.0)
+    assert rel_err(res1.dwg, res0.dwg) > 0.05           # the term is not lost in the comparison's tolerance
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("activated_only", [True, False])
+@pytest.mark.parametrize("d_experts,pool,ebatch,prefetch_n", [(8, 8, 4, 0), (6, 3, 2, 0), (8, 5, 2, 3), (4, 2, 4, 2),
+                                                              (6, 5, 2, 5), (6, 4, 3, 4)])
+def test_layer_offloaded_experts(d_experts, pool, ebatch, prefetch_n, activated_only, dtype):
+    """Some or all experts live in pinned host memory and stream through a pool smaller than the layer.  The last
+    two cases prefetch as many experts as the pool holds, so that a chunk which still contains prefetched
+    experts reaches the end of the pool (the chunk is cut there, not wrapped onto slot 0)."""
+    print(f"layer offload d={d_experts} pool={pool} ebatch={ebatch} prefetch={prefetch_n} act_only={activated_only} {dtype}", flush=True)
     E, k = 8, 2
-    m, x, ref = _build(400, 64, E, k, 128, dtype, d_experts=d_experts, pool=pool, ebatch=ebatch)
+    m, x, ref = _build(400, 64, E, k, 128, dtype, d_experts=d_experts, pool=pool, ebatch=ebatch,
+                       activated_only=activated_only)
     if prefetch_n:
         m.set_prefetch(prefetch_n, prefetch_n)
         m.prefetch_fwd(prefetch_n)             # what the scheduler does before the first layer
@@ -103,16 +130,156 @@ def test_layer_offloaded_experts(d_experts, pool, ebatch, prefetch_n, dtype):
                 gp.grad_tensors.zero_()
         m.gate[0].linear.weight.grad = None
         m.prefetch_fwd(prefetch_n)
+        assert m.MOLECore.fwd_base == prefetch_n
     _run_and_compare(m, x, ref, k, 0.0, dtype)
+    from mole_amd import core
+    um = core.get_UniMem()
+    assert um.virtual_offset() == 0 and um.view_pool_size() == pool
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("unified", [False, True])
+def test_layer_activated_only_skips_experts_without_rows(unified, dtype):
+    """Twelve tokens, top-1, eight offloaded experts: several experts get no row.  Only the activated ones are
+    copied (the pool's byte counter says so exactly, forward and backward), the results equal the oracle's, the
+    host gradients of the others read zero - also when they held a gradient from an earlier step - and a run
+    with activated_only=False (every expert copied and launched, as the reference does) gives the same bits."""
+    from mole_amd import core
+    print(f"layer activated-only unified={unified} {dtype}", flush=True)
+    S, M, E, k, Fd = 12, 64, 8, 1, 128
+    kw = dict(device_s_experts=E) if unified else {}
+    es = 4 if dtype == torch.float32 else 2
+    expert_bytes = (2 * Fd * M + Fd + M) * es
+
+    def run(activated_only, x_override=None):
+        m, x, ref = _build(S, M, E, k, Fd, dtype, d_experts=E, pool=4, ebatch=2, seed=8, activated_only=activated_only, **kw)
+        if x_override is not None:
+            x = x_override
+        um = core.get_UniMem()
+        # an earlier step in which every expert was active leaves gradients behind in the host arrays
+        big = torch.randn(4 * S * E, M, generator=torch.Generator().manual_seed(1)).to(dtype).cuda().requires_grad_(True)
+        yb = m(big, capacity_factor=0.0)
+        yb.backward(torch.ones_like(yb) * 1e-2)
+        torch.cuda.synchronize(); core.synchronize_tran()
+        assert all(float(m.FC1_W_CPU.all_tensors.grad_[e].abs().max()) > 0 for e in range(E))
+        um.copy_stats()
+        m.gate[0].linear.weight.grad = None
+        res = _run_and_compare(m, x, ref, k, 0.0, dtype)
+        nbytes, _ = um.copy_stats()
+        return m, res, nbytes, _grads(m, E)
+
+    m, res, nbytes, grads = run(True)
+    active = [e for e in range(E) if res.crit.kept_rows[e] > 0]
+    assert 0 < len(active) < E
+    assert nbytes == 2 * len(active) * expert_bytes          # forward + backward, activated experts only
+    for e in range(E):
+        if e not in active:
+            assert all(float(g[e].abs().max()) == 0.0 for g in grads)
+    if unified:
+        from mole_amd.utils.Uparam import UnifiedCPUTensor
+        pool_t = UnifiedCPUTensor.get_cpu_experts()[0]
+        assert pool_t.is_pinned() and pool_t.numel() == E * (2 * Fd * M + Fd + M)
+        assert m.FC1_W_CPU.all_tensors.data_ptr() == pool_t.data_ptr()
+        assert m.FC1_B_CPU.all_tensors.data_ptr() == pool_t.data_ptr() + E * Fd * M * es
+    m2, res2, nbytes2, grads2 = run(False)
+    assert nbytes2 == 2 * E * expert_bytes
+    for a, b in zip(grads, grads2):
+        assert torch.equal(a, b)
+
+
+def test_pool_guards_and_reserve():
+    """The process-wide pool refuses a second layer whose experts have another shape (it would read the slots at the
+    wrong strides), and pool_prefetch hands out the reserved slots as tensors (core.cpp:1425)."""
+    from mole_amd import core
+    from mole_amd.moe.layer import MOLEModule
+    m, x, ref = _build(100, 64, 4, 2, 128, torch.float32, d_experts=4, pool=4, ebatch=2)
+    dist = {"local_rank": 0, "world_size": 1, "rank": 0}
+    with pytest.raises(RuntimeError, match="cannot share"):
+        MOLEModule(2, 0, 64, 256, 4, 2, 2, dist, "gelu", 1, False, True, dtype=torch.float32)
+    with pytest.raises(RuntimeError, match="slots"):
+        core.create_UniMem(0, 9, torch.float32, [[128, 64], [128], [128, 64], [64]])
+    MOLEModule._instance = MOLEModule._instance[:1]
+    slots = core.pool_prefetch(0, 3)
+    assert [tuple(t.shape) for t in slots] == [(3, 128, 64), (3, 128), (3, 128, 64), (3, 64)]
+    um = core.get_UniMem()
+    assert um.view_pool_size() == 1 and um.virtual_offset() == 3
+    assert slots[0].data_ptr() == um.slot_tensor(0, 0, 3)
+    slots[0].fill_(1.5)
+    assert core.fetch_top_prefetched_batch(0) == 3 and um.view_pool_size() == 4
+    assert core.get_stream_cdata(0, 1) == um.tran_stream_handle() != core.get_stream_cdata(0, 2)
+    assert core.get_stream_cdata(0, 4) == um.tranback_stream_handle()
+    from mole_amd.utils.Ustream import ExpertStreamCtx
+    ExpertStreamCtx(device="cuda:0")
+    assert ExpertStreamCtx.tran_back_stream().cuda_stream == um.tranback_stream_handle()
+    assert ExpertStreamCtx.tran_stream().cuda_stream == um.tran_stream_handle()
+    MOLEModule.reset_instances()
 
 
 def test_layer_config1_exact():
     """BASELINE config 1 as specified: 4096 x 512 fp32, 8 experts, top-2, F = 2048, N(0, 0.02) weights,
-    MSE against zero, seed 0; with the reference's default capacity factor and without dropping."""
+    MSE against zero, seed 0; with the reference's default capacity factor and without dropping.  Besides the
+    max-norm tolerance, every row of y and dx is held to it relative to the row's own largest element."""
+    from tests.util import row_rel_err
     for cf in (1.0, 0.0):
         print(f"layer config1 cf={cf}", flush=True)
         m, x, ref = _build(4096, 512, 8, 2, 2048, torch.float32, seed=0)
-        _run_and_compare(m, x, ref, 2, cf, torch.float32)
+        xin = x.clone().requires_grad_(True)
+        y = m(xin, capacity_factor=cf)
+        dy = (2.0 * y.detach() / y.numel())
+        y.backward(dy)
+        res = _run_and_compare(m, x, ref, 2, cf, torch.float32)
+        ry, rdx = row_rel_err(y, res.y), row_rel_err(xin.grad, res.dx)
+        print(f"layer config1 cf={cf}: per-row relative error y {ry:.2e}, dx {rdx:.2e}", flush=True)
+        assert ry < 1e-5 and rdx < 1e-5
+
+
+def _near_tie_report(scores64, idx_gpu, idx_cpu, k, bound):
+    """Tokens whose chosen expert sets differ between the GPU and the oracle, each checked to be a genuine near
+    tie: the scores (fp64 reference) of the experts the two sides disagree about lie within `bound` (relative)."""
+    diff = (idx_gpu != idx_cpu).any(axis=0).nonzero()[0]
+    for i in diff:
+        a, b = idx_gpu[:, i], idx_cpu[:, i]
+        involved = sorted(set(a.tolist()) ^ set(b.tolist())) or sorted(set(a.tolist()))   # same set, other order
+        vals = scores64[i, involved]
+        assert float(vals.max() - vals.min()) <= bound * float(vals.max()), \
+            f"token {i}: GPU chose {a.tolist()}, oracle {b.tolist()}, scores {scores64[i, sorted(set(a.tolist()) | set(b.tolist()))]}"
+    return len(diff)
+
+
+@pytest.mark.parametrize("name,S,M,E,k,cf,dtype", [("c1", 4096, 512, 8, 2, 1.0, torch.float32),
+                                                   ("c2", 16384, 1024, 16, 1, 1.25, torch.bfloat16)])
+def test_routing_from_tokens_matches_oracle(name, S, M, E, k, cf, dtype):
+    """Routing end to end from x (gate product, softmax, top-k, locations, capacity, permutation) against the
+    oracle run on the same seeded x and Wg with no help from the GPU's scores.  The two gates sum their products
+    in different orders (and the bf16 gate multiplies bf16-rounded operands exactly into fp32), so scores differ
+    in the last bits; an index may differ only where the competing scores are that close, and such tokens
+    are counted.  With none, every routing output must be equal bit for bit."""
+    from mole_amd import hip_ops as H
+    from mole_amd.utils import Ugate
+    print(f"routing from tokens {name}", flush=True)
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(S, M, generator=g)
+    wg = torch.randn(E, M, generator=g) * 0.02
+    xr = x.to(dtype)
+    wr = wg if dtype == torch.float32 else wg.bfloat16().float()      # the bf16 gate kernel rounds Wg
+    scores_gpu = Ugate.gate_scores(xr.cuda(), wg.cuda())
+    r = H.route(scores_gpu, k, cf)
+    scores_cpu = O.gate_scores(xr.float(), wr)
+    c = O.extract_critical(scores_cpu.numpy(), k, cf)
+    idx_gpu, idx_cpu = r.idx.cpu().numpy(), np.stack(c.indices_s)
+    scores64 = torch.softmax(xr.double() @ wr.double().t(), dim=-1).numpy()
+    # a few ulp of fp32 relative to the score
+    flips = _near_tie_report(scores64, idx_gpu, idx_cpu, k, bound=8 * 1.2e-7)
+    print(f"routing from tokens {name}: {flips} of {S} tokens routed differently (near ties)", flush=True)
+    assert flips <= 2
+    if flips == 0:
+        np.testing.assert_array_equal(idx_gpu, idx_cpu)
+        np.testing.assert_array_equal(r.counts.cpu().numpy(), c.counts)
+        np.testing.assert_array_equal(r.loc.cpu().numpy(), np.stack(c.locations_s))
+        np.testing.assert_array_equal(r.row.cpu().numpy(), c.rows(True))
+        np.testing.assert_array_equal(r.kept_rows.cpu().numpy(), c.kept_rows)
+        assert int(r.capacity.cpu()) == c.capacity
+        assert rel_err(r.gates.cpu(), torch.from_numpy(np.stack(c.gates_s))) < 1e-5
 
 
 def test_layer_gelu_exact_switch_and_gate_bias():

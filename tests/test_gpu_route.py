@@ -82,6 +82,19 @@ def test_softmax_and_gate_bwd(S, E):
         idx = torch.from_numpy(np.stack(c.indices_s)).cuda()
         got = H.gate_bwd(dg.cuda(), sc, idx, norm)
         assert rel_err(got, want_dl) < 1e-5
+        # the load-balancing loss rides along: d l_aux / d scores = E/S^2 counts0[e] on every token
+        w = 0.37 * (k + 1)
+        extra = O.gshard_loss_bwd(S, c.counts[0], w).float()
+        want_aux = O.softmax_bwd(O.gate_normalize_bwd(dg, scores, c, norm) + extra, scores)
+        counts0 = torch.from_numpy(c.counts[0].astype(np.int32)).cuda()
+        got = H.gate_bwd(dg.cuda(), sc, idx, norm, counts0=counts0, d_l_aux=torch.tensor([w], device="cuda"))
+        assert rel_err(got, want_aux) < 1e-5
+        got = H.gate_bwd(dg.cuda(), sc, idx, norm, through_softmax=False, counts0=counts0,
+                         d_l_aux=torch.tensor([w], device="cuda"))
+        assert rel_err(got, O.gate_normalize_bwd(dg, scores, c, norm) + extra) < 1e-5
+    # the softmax's backward as its own entry point
+    ds = torch.randn(S, E, generator=g)
+    assert rel_err(H.softmax_bwd(ds.cuda(), sc), O.softmax_bwd(ds, sc.cpu())) < 1e-5
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -96,8 +109,37 @@ def test_gate_wgrad(S, E, M, dtype):
     got = H.gate_wgrad(dl.cuda(), x.cuda())
     want = dl.double().t() @ x.double()
     # fp32 sums of exact products (VALU kernel) or of products with dlogits split into two bf16 parts (matrix
-    # cores, bf16 tokens); fp32 tokens with a large gate go through a library GEMM in fp32
+    # cores, bf16 tokens); fp32 tokens with a large gate take the transposed product of the grouped-GEMM tiles
+    assert got.shape == (E, M)
     assert rel_err(got, want) < 2e-5
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,Mo,N", [(1, 4, 8), (300, 64, 192), (1000, 8, 520), (129, 128, 256), (0, 8, 16)])
+def test_gemm_tn_and_gate_input_grad(rows, Mo, N, dtype):
+    """c = a^T . b on the grouped-GEMM tiles (the gate weight gradient of shapes its own kernels do not take) and
+    the gate's input gradient dlogits . Wg with E padded to the tile granule."""
+    from mole_amd import hip_ops as H
+    print(f"gemm_tn rows={rows} Mo={Mo} N={N} {dtype}", flush=True)
+    g = torch.Generator().manual_seed(rows + Mo)
+    ep = 8 if dtype == torch.bfloat16 else 4
+    Mo = (Mo + ep - 1) // ep * ep
+    a = torch.randn(rows, Mo, generator=g).to(dtype)
+    b = torch.randn(rows, N, generator=g).to(dtype)
+    got = H.gemm_tn(a.cuda(), b.cuda())
+    want = a.double().t() @ b.double()
+    t = 1e-5 if dtype == torch.float32 else 1e-2
+    if rows == 0:
+        assert float(got.abs().max()) == 0.0
+        return
+    assert rel_err(got, want) < t
+    for E in (3, 8, 37):
+        dl = torch.randn(rows, E, generator=g) * 0.1
+        wg = torch.randn(E, N, generator=g) * 0.05
+        got = H.gate_input_grad(dl.cuda(), wg.cuda(), dtype)
+        want = dl.to(dtype).double() @ wg.to(dtype).double()
+        assert got.shape == (rows, N) and got.dtype == dtype
+        assert rel_err(got, want) < t
 
 
 @pytest.mark.parametrize("S,E,M,bias", [(100, 16, 128, False), (1000, 8, 256, True), (513, 64, 384, False),

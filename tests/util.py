@@ -14,6 +14,28 @@ def rel_err(got: torch.Tensor, want: torch.Tensor) -> float:
     return float((got - want).abs().max()) / denom
 
 
+def rel_err_dev(got: torch.Tensor, want: torch.Tensor) -> float:
+    """rel_err evaluated where the tensors live (fp32 arithmetic on the GPU): for comparisons of hundreds of
+    megabytes, where the trip through fp64 on the host would dominate the test."""
+    got, want = got.detach().float(), want.detach().float().to(got.device)
+    denom = float(want.abs().max()) if want.numel() else 0.0
+    diff = float((got - want).abs().max()) if want.numel() else 0.0
+    return diff if denom == 0.0 else diff / denom
+
+
+def row_rel_err(got: torch.Tensor, want: torch.Tensor) -> float:
+    """max over rows of max_j |got[i,j] - want[i,j]| / max_j |want[i,j]|: every row is held to the tolerance
+    relative to its own magnitude, so that a row of small values cannot hide behind a large one elsewhere.
+    Rows whose reference is all zero count with their absolute error."""
+    got = got.detach().double().cpu().reshape(-1, got.shape[-1])
+    want = want.detach().double().cpu().reshape(-1, want.shape[-1])
+    if want.numel() == 0:
+        return 0.0
+    diff = (got - want).abs().amax(dim=1)
+    mag = want.abs().amax(dim=1)
+    return float(torch.where(mag > 0, diff / mag.clamp_min(1e-300), diff).max())
+
+
 FP32_TOL = 1e-5
 BF16_TOL = 2e-2
 
