@@ -233,7 +233,11 @@ int mole_gemm_tn(const void *a, const void *b, int dtype, int rows, int Mo, int 
  *                                 view_base+virtual_offset .. : waits for the last compute that
  *                                 used those slots, copies the part not yet prefetched, records the
  *                                 event.
- *   wait_params(stream)           the compute stream waits for the last fetch/prefetch.
+ *   wait_params(stream)           the compute stream waits for every copy issued so far.
+ *   wait_slots(view_base, n, stream)
+ *                                 the compute stream waits for the experts in slots view_base+virtual_offset ..
+ *                                 only (each expert carries an event of its own): a chunk starts computing
+ *                                 while the rest of a large prefetch is still arriving.
  *   release(view_base, n, stream) records that compute on `stream` has finished with the slots.
  *
  * prefetch_ids / fetch_ids are the same two calls for an explicit list of experts instead of a range:
@@ -262,6 +266,7 @@ int mole_unimem_fetch(void *handle, const void *const host_src[4], int view_base
 int mole_unimem_fetch_ids(void *handle, const void *const host_src[4], int view_base, const int32_t *expert_ids,
                           int n, int prefetched, void **slot_ptrs_out /* [4] */);
 int mole_unimem_wait_params(void *handle, mole_stream_t compute_stream);
+int mole_unimem_wait_slots(void *handle, int view_base, int n, mole_stream_t compute_stream);
 int mole_unimem_release(void *handle, int view_base, int n, mole_stream_t compute_stream);
 int mole_unimem_sync_tran(void *handle);
 int mole_unimem_tran_stream(void *handle, mole_stream_t *out);

@@ -60,6 +60,7 @@ _SIGNATURES = {
     "mole_unimem_fetch": (c_int, [_P, POINTER(_P), c_int, c_int, c_int, c_int, POINTER(_P)]),
     "mole_unimem_fetch_ids": (c_int, [_P, POINTER(_P), c_int, POINTER(c_int32), c_int, c_int, POINTER(_P)]),
     "mole_unimem_wait_params": (c_int, [_P, _P]),
+    "mole_unimem_wait_slots": (c_int, [_P, c_int, c_int, _P]),
     "mole_unimem_release": (c_int, [_P, c_int, c_int, _P]),
     "mole_unimem_sync_tran": (c_int, [_P]),
     "mole_unimem_tran_stream": (c_int, [_P, POINTER(_P)]),

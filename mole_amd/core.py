@@ -99,6 +99,10 @@ class UniMem:
     def wait_params(self):
         L.check(L.lib().mole_unimem_wait_params(self._h, L.stream()), "mole_unimem_wait_params")
 
+    def wait_slots(self, view_base: int, n: int):
+        """The current stream waits for the experts in slots view_base.. (of the visible pool) to have arrived."""
+        L.check(L.lib().mole_unimem_wait_slots(self._h, view_base, n, L.stream()), "mole_unimem_wait_slots")
+
     def release(self, view_base: int, n: int):
         L.check(L.lib().mole_unimem_release(self._h, view_base, n, L.stream()), "mole_unimem_release")
 
@@ -552,7 +556,7 @@ class MOLECore:
             order, off_c, kept_c = self._order(resident, wanted, offsets, kept_rows, host_meta)
             for (lo, size, pref, view_base) in self._chunks(len(order), len(resident)):
                 p = um.fetch_ids(self._host(), view_base, order[lo:lo + size], pref)
-                um.wait_params()
+                um.wait_slots(view_base, size)
                 H.ffn_fwd_into(x2, off_c[lo:], kept_c[lo:], size, rows, M, F, p[0], p[1], p[2], p[3], h, a, out)
                 um.release(view_base, size)
         saved = (x2, h, a, offsets, kept_rows, requires_grad, shape, host_meta)
@@ -598,7 +602,7 @@ class MOLECore:
             for (lo, size, pref, view_base) in self._chunks(len(order), len(resident)):
                 ids = order[lo:lo + size]
                 p = um.fetch_ids(self._host(), view_base, ids, pref)   # weights are fetched again (core.cpp:1203)
-                um.wait_params()
+                um.wait_slots(view_base, size)
                 g = [torch.empty((size, *hg.shape[1:]), dtype=hg.dtype, device=x2.device) for hg in host_grads]
                 H.ffn_bwd_into(go, x2, h, a, off_c[lo:], kept_c[lo:], size, rows, M, F, p[0], p[2], t, g[0], g[1],
                                g[2], g[3], gx, False, self.gelu_bwd)
