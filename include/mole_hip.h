@@ -147,6 +147,21 @@ int mole_route(const float *scores, int S, int E, int k, double capacity_factor,
                int32_t *counts, int32_t *kept_rows, int32_t *offsets, int32_t *capacity,
                float *l_aux, void *workspace, size_t workspace_bytes, mole_stream_t stream);
 
+/* mole_route for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): the same routing with the same outputs, but without the workspace argument.
+ * No counterpart in the reference.  The scratch the routing kernels need (per-block histograms, per-choice bases,
+ * column sums of the scores) lives in a static device array of mole_route_static_max_bytes() = 8 MiB inside the
+ * library, one copy per GPU, held until the process ends; the call allocates nothing, on the host side neither.
+ * Problem sizes whose mole_route_workspace_bytes(S, E, k) exceeds the array are rejected with MOLE_E_WORKSPACE
+ * (the five BASELINE configurations need at most 4.6 MiB).  All calls on one GPU share the array: calls that
+ * overlap on one GPU (two streams, two threads) race on it and must be serialised by the caller.  The first
+ * call on a device looks up the array's address (hipGetSymbolAddress) and must not run under stream capture. */
+size_t mole_route_static_max_bytes(void);
+int mole_route_static(const float *scores, int S, int E, int k, double capacity_factor, int normalize_gate,
+                      int alignment, int layout, int32_t *idx, int32_t *loc, float *gates, int32_t *row,
+                      int32_t *counts, int32_t *kept_rows, int32_t *offsets, int32_t *capacity,
+                      float *l_aux, mole_stream_t stream);
+
 /* ------------------------------------------------------------------------------------------
  * Dispatch / combine.  Replace tutel fast_encode / fast_decode and their backward
  * (call sites MOLE/moe/layer.py:448-449, 457-458).  `row` is mole_route's permutation.

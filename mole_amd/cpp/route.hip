@@ -18,6 +18,8 @@
 #include <limits.h>
 #include <math.h>
 
+#include <mutex>
+
 namespace mole {
 
 constexpr int RT_THREADS = 256;
@@ -465,6 +467,58 @@ extern "C" int mole_route(const float *scores, int S, int E, int k, double capac
         MOLE_LAUNCH_CHECK();
     }
     return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
+// mole_route without a workspace argument and without any allocation: the per-block histograms, the per-choice
+// bases and the column sums of the scores live in a file-scope device array.  Each GPU the library runs on holds
+// its own copy of the array until the process ends.  The array's name is only a host-side handle; the address
+// the kernels get is looked up once per device with hipGetSymbolAddress and kept.
+// ---------------------------------------------------------------------------------------------
+#define MOLE_ROUTE_SCRATCH_BYTES (8u << 20)
+static __device__ __align__(256) unsigned char scratch[MOLE_ROUTE_SCRATCH_BYTES];
+
+namespace mole {
+constexpr int MAX_SCRATCH_DEVICES = 64;
+static void *g_scratch_ptr[MAX_SCRATCH_DEVICES];
+static std::mutex g_scratch_mu;
+
+// device address of `scratch` on the current device
+static int route_scratch(void **out) {
+    int dev = 0;
+    MOLE_HIP(hipGetDevice(&dev));
+    MOLE_REQUIRE(dev >= 0 && dev < MAX_SCRATCH_DEVICES, "mole_route_static: device %d out of range", dev);
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void *p = nullptr;
+        MOLE_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        MOLE_REQUIRE(p != nullptr, "mole_route_static: hipGetSymbolAddress returned no address");
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return 0;
+}
+}  // namespace mole
+
+extern "C" size_t mole_route_static_max_bytes(void) { return MOLE_ROUTE_SCRATCH_BYTES; }
+
+extern "C" int mole_route_static(const float *scores, int S, int E, int k, double capacity_factor, int normalize_gate,
+                                 int alignment, int layout, int32_t *idx, int32_t *loc, float *gates, int32_t *row,
+                                 int32_t *counts, int32_t *kept_rows, int32_t *offsets, int32_t *capacity, float *l_aux,
+                                 mole_stream_t stream) {
+    const size_t need = mole_route_workspace_bytes(S, E, k);
+    if (need == 0 || need > MOLE_ROUTE_SCRATCH_BYTES) {
+        set_error("mole_route_static: S=%d E=%d k=%d needs %zu bytes of scratch, the static array holds %zu "
+                  "(use mole_route with a workspace of your own)", S, E, k, need, (size_t)MOLE_ROUTE_SCRATCH_BYTES);
+        return need == 0 ? MOLE_E_INVALID : MOLE_E_WORKSPACE;
+    }
+    void *ptr = nullptr;
+    if (int rc = route_scratch(&ptr)) return rc;
+    // every word of the scratch that a kernel of the route reads has been written by an earlier kernel of the
+    // same call (the histograms by the top-k blocks, the bases and column sums by the scan / finish kernels), so
+    // nothing needs clearing between calls; calls that overlap on one GPU would race on it
+    return mole_route(scores, S, E, k, capacity_factor, normalize_gate, alignment, layout, idx, loc, gates, row, counts,
+                      kept_rows, offsets, capacity, l_aux, ptr, MOLE_ROUTE_SCRATCH_BYTES, stream);
 }
 
 // ---------------------------------------------------------------------------------------------
