@@ -7,7 +7,11 @@ default workload is BASELINE.json's configuration 2: Switch-style layer, bf16 wi
 16384 tokens x 1024, 16 experts of 1024 -> 4096 -> 1024, top-1, capacity factor 1.25.
 
 Prints ONE JSON line: the metric (tokens/s), the roofline of the dominant kernel measured with HIP
-events on the stream the kernel runs on, and the CPU oracle timed on this box's host cores.
+events on the stream the kernel runs on, the same figures for configuration 1 (fp32, the CPU-runnable
+case) on the GPU, and the CPU oracle timed on configuration 1 on this box's host cores.
+
+--probe prints a different line: what the matrix cores sustain on their own (zero and random operands)
+and what the product's K loop sustains without its epilogue, at the default workload's shape.
 """
 import argparse
 import json
@@ -30,11 +34,16 @@ PEAK_MFMA_TFLOPS = {"bf16": 2500.0, "f32": 157.3}   # MI355X dense peaks
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch (read + write) of the grouped GEMMs at workload c2, from rocprofv3 FETCH_SIZE and
 # WRITE_SIZE runs of this script scaled by the same counters' readings for a copy of known size
-# (profiles/bench_c2_hbm_traffic.txt); other workloads have no counter run and report null
+# (profiles/bench_c2_hbm_traffic.txt, profiles/bench_c3_c5_hbm_traffic.txt); c1 has no counter run and reports null
 MEASURED_TRAFFIC_BYTES = {
-    "c2": {"ffn_fwd1": 751.8e6, "ffn_fwd2": 383.9e6, "ffn_gw2": 546.7e6, "ffn_da": 741.5e6, "ffn_gw1": 546.7e6,
-           "ffn_gx": 385.0e6},
+    "c2": {"ffn_fwd1": 758.2e6, "ffn_fwd2": 373.2e6, "ffn_gw2": 547.0e6, "ffn_da": 748.5e6, "ffn_gw1": 547.0e6,
+           "ffn_gx": 383.2e6},
+    "c3": {"ffn_fwd1": 3816.1e6, "ffn_fwd2": 2214.7e6, "ffn_gw2": 3085.4e6, "ffn_da": 3824.1e6, "ffn_gw1": 3085.4e6,
+           "ffn_gx": 2219.6e6},
+    "c5": {"ffn_fwd1": 4371.8e6, "ffn_fwd2": 3329.5e6, "ffn_gw2": 5971.4e6, "ffn_da": 4378.7e6, "ffn_gw1": 5971.4e6,
+           "ffn_gx": 3306.4e6},
 }
+PEAK_HBM_BYTES = PEAK_HBM_GBS * 1e9
 
 
 def make_layer(w, seed=0):
@@ -65,33 +74,43 @@ def step(m, x, dy, cf):
     m.gate[0].linear.weight.grad = None
 
 
-def cpu_baseline(w, budget_s=12.0):
-    """The CPU oracle's layer (fp32 torch on the host cores), forward + backward, on a bounded
-    sample of the workload: the same layer shape at a token count that keeps the run near budget_s."""
+def cpu_baseline(budget_s=12.0):
+    """The CPU oracle's layer (fp32 torch on the host cores), forward + backward, on BASELINE configuration 1
+    exactly as specified: 4096 tokens x 512 ~N(0,1), gate 512 -> 8 ~N(0,0.02), top-2, experts
+    Linear(512 -> 2048) + GELU + Linear(2048 -> 512) ~N(0,0.02), fp32, seed 0, MSE against zero, the reference's
+    default capacity factor 1.0.  Three warm-up steps, then at least ten timed ones (until budget_s), median."""
     import torch
     from oracle import moe_oracle as O
+    w = WORKLOADS["c1"]
     cores = min(16, os.cpu_count() or 1)
     torch.set_num_threads(cores)
-    S = min(w["S"], 4096)
     g = torch.Generator().manual_seed(0)
-    E, M, F = w["E"], w["M"], w["F"]
+    S, E, M, F = w["S"], w["E"], w["M"], w["F"]
     x = torch.randn(S, M, generator=g)
     wg = torch.randn(E, M, generator=g) * 0.02
     w1, b1 = torch.randn(E, F, M, generator=g) * 0.02, torch.randn(E, F, generator=g) * 0.02
     w2, b2 = torch.randn(E, F, M, generator=g) * 0.02, torch.randn(E, M, generator=g) * 0.02
-    dy = torch.randn(S, M, generator=g) * 1e-3
-    run = lambda: O.moe_layer(x, wg, w1, b1, w2, b2, w["k"], w["cf"], dy=dy)
-    run()
+
+    y = O.moe_layer(x, wg, w1, b1, w2, b2, w["k"], w["cf"]).y
+    dy = 2.0 * y / y.numel()                      # gradient of mean(y^2); the inputs are fixed, so it is too
+
+    def run():
+        return O.moe_layer(x, wg, w1, b1, w2, b2, w["k"], w["cf"], dy=dy)
+
+    for _ in range(3):
+        run()
     times = []
     t_start = time.perf_counter()
-    while len(times) < 3 or (time.perf_counter() - t_start < budget_s and len(times) < 20):
+    while len(times) < 10 or (time.perf_counter() - t_start < budget_s and len(times) < 40):
         t0 = time.perf_counter()
         run()
         times.append(time.perf_counter() - t0)
     times.sort()
     med = times[len(times) // 2]
-    return {"value": S / med, "unit": "tokens/s", "cores": cores, "kind": "port",
-            "sample": f"{len(times)} steps of the {w['name']} layer shape at {S} tokens, fp32 torch-CPU oracle, median"}
+    return {"value": round(S / med, 1), "unit": "tokens/s", "cores": cores, "kind": "port", "ms_per_step": round(med * 1e3, 2),
+            "sample": f"{len(times)} steps of configuration c1 exactly (S={S} M={M} E={E} top-{w['k']} F={F} fp32, seed 0, "
+                      f"capacity factor {w['cf']}, MSE against zero), forward + backward, "
+                      f"fp32 torch-CPU oracle on {cores} threads, median"}
 
 
 def bench_offloaded_stack(args):
@@ -184,6 +203,190 @@ def bench_offloaded_stack(args):
     print(json.dumps(out))
 
 
+def measure_layer(name, steps, warmup, with_adam=True):
+    """Times `steps` forward + backward passes of one MoE layer of workload `name` (inputs resident in HBM), then the
+    same steps again with the library's per-kernel events on.  Returns the JSON fields of that workload."""
+    import torch
+    from mole_amd import _lib as L
+    w = dict(WORKLOADS[name], name=name)
+    m, x, dy = make_layer(w)
+    cf = w["cf"]
+    for _ in range(warmup):
+        step(m, x, dy, cf)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step(m, x, dy, cf)
+    torch.cuda.synchronize()
+    dt_s = time.perf_counter() - t0
+    ms_per_step = dt_s / steps * 1e3
+    value = w["S"] / (dt_s / steps)
+
+    # per-kernel durations: a second pass of the same steps with start/stop events attached to every kernel
+    # launch, on the stream the kernel is launched on
+    L.kernel_timing_enable(True)
+    for _ in range(steps):
+        step(m, x, dy, cf)
+    torch.cuda.synchronize()
+    timing = L.kernel_timing_read()
+    L.kernel_timing_enable(False)
+
+    R = int(m.last_route.offsets[-1].item())       # kept (token, choice) rows
+    S, M, F, k = w["S"], w["M"], w["F"], w["k"]
+    b = 2 if w["dtype"] == "bf16" else 4
+    gemm_flop = 2.0 * R * M * F                     # every one of the six grouped products
+    # algorithmic HBM bytes of the products (operands once, results once; kept rows only)
+    act, wts = R * (M + 0.0) * b, w["E"] * F * M * b * 1.0
+    gemm_bytes = {"ffn_fwd1": act + wts + 2 * R * F * b, "ffn_fwd2": R * F * b + wts + act,
+                  "ffn_gw2": R * F * b + act + wts, "ffn_da": act + wts + 2 * R * F * b,
+                  "ffn_gw1": R * F * b + act + wts, "ffn_gx": R * F * b + wts + act}
+    work = {  # algorithmic work per launch: flop for the GEMMs, bytes for the permutes
+        "ffn_fwd1": gemm_flop, "ffn_fwd2": gemm_flop, "ffn_gw2": gemm_flop, "ffn_da": gemm_flop, "ffn_gw1": gemm_flop,
+        "ffn_gx": gemm_flop,
+        # the combine backward is one fused kernel (d_o scatter and the gate dot products read dy and o once)
+        "dispatch_fwd": 2.0 * R * M * b, "combine_fwd": (R + S) * M * b, "combine_bwd": (S + 2.0 * R) * M * b,
+        "dispatch_bwd": (R + S) * M * b,
+    }
+    kernels = {}
+    for kname, (cnt, ms) in timing.items():
+        if cnt == 0:
+            continue
+        avg_us = ms / cnt * 1e3
+        entry = {"avg_us": round(avg_us, 2), "launches_per_step": cnt / steps}
+        if kname in work:
+            if kname.startswith("ffn_"):
+                entry["tflops"] = round(work[kname] / (avg_us * 1e-6) / 1e12, 1)
+            else:
+                entry["gbs"] = round(work[kname] / (avg_us * 1e-6) / 1e9, 1)
+        kernels[kname] = entry
+    gemms = [n for n in kernels if n in gemm_bytes]
+    dom = max(gemms, key=lambda n: kernels[n]["avg_us"])
+    peak = PEAK_MFMA_TFLOPS[w["dtype"]]
+    dom_s = kernels[dom]["avg_us"] * 1e-6
+    gemm_total_us = sum(kernels[n]["avg_us"] for n in gemms)
+    traffic = MEASURED_TRAFFIC_BYTES.get(name, {}).get(dom)
+    mfma_frac = kernels[dom]["tflops"] / peak
+    hbm_alg_frac = gemm_bytes[dom] / dom_s / PEAK_HBM_BYTES
+    hbm_meas_frac = traffic / dom_s / PEAK_HBM_BYTES if traffic else None
+    # the roof the kernel is nearer to, judged by the bytes it really moves when a counter run gave them
+    hbm_side = hbm_meas_frac if hbm_meas_frac is not None else hbm_alg_frac
+    if hbm_side > mfma_frac:
+        roofline = {"bound": "hbm", "kernel": dom, "achieved": round(gemm_bytes[dom] / dom_s / 1e9, 1), "peak": PEAK_HBM_GBS,
+                    "unit": "GB/s", "frac": round(hbm_alg_frac, 4)}
+    else:
+        roofline = {"bound": "mfma", "kernel": dom, "achieved": kernels[dom]["tflops"], "peak": peak, "unit": "TFLOP/s",
+                    "frac": round(mfma_frac, 4)}
+    roofline.update({"traffic": traffic, "mfma_frac": round(mfma_frac, 4), "hbm_frac_algorithmic_bytes": round(hbm_alg_frac, 4),
+                     "hbm_frac_measured_traffic": round(hbm_meas_frac, 4) if hbm_meas_frac is not None else None,
+                     "all_ffn_gemms_frac": round(6 * gemm_flop / (gemm_total_us * 1e-6) / 1e12 / peak, 4)})
+    out = {
+        "value": round(value, 1), "ms_per_step": round(ms_per_step, 4), "dtype": w["dtype"],
+        "config": {"workload": f"{name}: single MoE layer fwd+bwd, S={S} M={M} E={w['E']} top-{k} F={F} "
+                               f"capacity_factor={cf}, kept rows R={R}"},
+        "roofline": roofline,
+        "hbm_permutes": {n: {"achieved": kernels[n]["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                             "frac": round(kernels[n]["gbs"] / PEAK_HBM_GBS, 4)}
+                         for n in ("dispatch_fwd", "combine_fwd", "combine_bwd", "dispatch_bwd") if n in kernels},
+        "kernels": kernels,
+    }
+    if with_adam:
+        # the fused Adam update on one weight array of this layer ([E, F, M] parameters and gradients in the
+        # layer's dtype, fp32 moments): not part of the step above, measured for its own HBM roofline
+        from mole_amd import hip_ops as H
+        pdt = torch.bfloat16 if w["dtype"] == "bf16" else torch.float32
+        n_adam = w["E"] * w["F"] * w["M"]
+        ap_, ag_ = (torch.randn(n_adam, device="cuda") * 0.02).to(pdt), (torch.randn(n_adam, device="cuda") * 1e-3).to(pdt)
+        am_, av_ = torch.zeros(n_adam, device="cuda"), torch.zeros(n_adam, device="cuda")
+        H.adam_step(ap_, ag_, am_, av_, 0.9, 0.999, 1, 1e-3, 0.0, 1e-8, False)
+        torch.cuda.synchronize()
+        L.kernel_timing_enable(True)
+        for i in range(5):
+            H.adam_step(ap_, ag_, am_, av_, 0.9, 0.999, 2 + i, 1e-3, 0.0, 1e-8, False)
+        torch.cuda.synchronize()
+        adam_cnt, adam_ms = L.kernel_timing_read()["adam"]
+        L.kernel_timing_enable(False)
+        del ap_, ag_, am_, av_
+        adam_bytes = n_adam * (22.0 if pdt == torch.bfloat16 else 28.0)   # read p, g, m, v; write p, m, v
+        adam_gbs = adam_bytes / (adam_ms / adam_cnt * 1e-3) / 1e9
+        out["hbm_optimizer"] = {"adam_step": {"achieved": round(adam_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                              "frac": round(adam_gbs / PEAK_HBM_GBS, 4), "elements": n_adam,
+                                              "avg_us": round(adam_ms / adam_cnt * 1e3, 2)}}
+    from mole_amd.moe.layer import MOLEModule
+    del m, x, dy
+    MOLEModule.reset_instances()
+    torch.cuda.empty_cache()
+    return out
+
+
+def run_probes(args):
+    """What bounds the grouped products at the default workload's shape, from tracked code: the matrix cores alone
+    (operands in registers, zero and random data, all CUs), the product's K loop without its epilogue, the full
+    first product, and a library GEMM of the same shape as a yardstick."""
+    import torch
+    from ctypes import byref, c_double
+    from mole_amd import _lib as L, hip_ops as H
+    w = WORKLOADS["c2"]
+    S, M, E, F = w["S"], w["M"], w["E"], w["F"]
+    dev = "cuda"
+    n_cu = torch.cuda.get_device_properties(0).multi_processor_count
+    nb = L.lib().mole_probe_mfma_operand_bytes()
+    sink = torch.zeros(n_cu * 512, device=dev)
+    res = {}
+
+    def timed(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        L.kernel_timing_enable(True)
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        t = L.kernel_timing_read()
+        L.kernel_timing_enable(False)
+        return t
+
+    flop = c_double()
+    for kind in ("zeros", "random"):
+        ops = torch.zeros(nb // 2, dtype=torch.bfloat16, device=dev) if kind == "zeros" else \
+            (torch.randn(nb // 2, device=dev) * 0.5).bfloat16()
+        iters = 4000
+        t = timed(lambda: L.check(L.lib().mole_probe_mfma(L.ptr(ops), n_cu, iters, L.ptr(sink), byref(flop), L.stream()),
+                                  "mole_probe_mfma"), 5)
+        cnt, ms = t["probe"]
+        res[f"mfma_only_{kind}_operands"] = {"avg_us": round(ms / cnt * 1e3, 1), "tflops": round(flop.value / (ms / cnt * 1e-3) / 1e12, 1)}
+    xd = torch.randn(S, M, device=dev).bfloat16()
+    w1 = (torch.randn(E, F, M, device=dev) * 0.02).bfloat16()
+    b1 = (torch.randn(E, F, device=dev) * 0.02).bfloat16()
+    w2 = (torch.randn(E, F, M, device=dev) * 0.02).bfloat16()
+    b2 = (torch.randn(E, M, device=dev) * 0.02).bfloat16()
+    rows = S // E
+    kept = torch.full((E,), rows, dtype=torch.int32, device=dev)
+    off = torch.arange(E + 1, dtype=torch.int32, device=dev) * rows
+    gflop = 2.0 * S * M * F
+    t = timed(lambda: L.check(L.lib().mole_probe_kloop(L.ptr(xd), L.ptr(w1), L.ptr(off), L.ptr(kept), E, S, F, M, L.ptr(sink),
+                                                       L.stream()), "mole_probe_kloop"), 20)
+    cnt, ms = t["probe"]
+    res["k_loop_without_epilogue"] = {"avg_us": round(ms / cnt * 1e3, 1), "tflops": round(gflop / (ms / cnt * 1e-3) / 1e12, 1)}
+    t = timed(lambda: H.ffn_fwd(xd, off, kept, w1, b1, w2, b2), 20)
+    for kname in ("ffn_fwd1", "ffn_fwd2"):
+        cnt, ms = t[kname]
+        res[kname] = {"avg_us": round(ms / cnt * 1e3, 1), "tflops": round(gflop / (ms / cnt * 1e-3) / 1e12, 1)}
+    # yardstick: the vendor library's GEMM of the same shape (not used by the product)
+    wt = w1[0].t().contiguous()
+    for _ in range(5):
+        torch.matmul(xd, wt)
+    torch.cuda.synchronize()
+    a, b_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(20):
+        torch.matmul(xd, wt)
+    b_.record()
+    torch.cuda.synchronize()
+    us = a.elapsed_time(b_) / 20 * 1e3
+    res["library_gemm_same_shape"] = {"avg_us": round(us, 1), "tflops": round(gflop / (us * 1e-6) / 1e12, 1)}
+    print(json.dumps({"probe": f"grouped product h = xd . w1^T at S={S} M={M} E={E} F={F}, bf16, {E} experts of {rows} rows",
+                      "peak_tflops": PEAK_MFMA_TFLOPS["bf16"], "compute_units": n_cu, "results": res}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -194,6 +397,8 @@ def main():
     ap.add_argument("--adam", action="store_true",
                     help="c4 only: update the offloaded experts with the in-pipeline Adam (adds 30 GB of pinned moments per layer)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-c1", action="store_true", help="skip the configuration-1 (fp32) figures beside the headline")
+    ap.add_argument("--probe", action="store_true", help="run the matrix-core and K-loop probes instead of the layer")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures the single-GPU MoE-layer hot path: this build has no multi-GPU path, run with --gpus 1",
@@ -201,101 +406,25 @@ def main():
         sys.exit(2)
 
     import torch
-    from mole_amd import _lib as L
     assert torch.cuda.is_available(), "bench.py needs an MI355X"
+    if args.probe:
+        return run_probes(args)
     if args.workload == "c4":
         return bench_offloaded_stack(args)
-    w = dict(WORKLOADS[args.workload], name=args.workload)
-    m, x, dy = make_layer(w)
-    cf = w["cf"]
-
-    for _ in range(args.warmup):
-        step(m, x, dy, cf)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step(m, x, dy, cf)
-    torch.cuda.synchronize()
-    dt_s = time.perf_counter() - t0
-    ms_per_step = dt_s / args.steps * 1e3
-    value = w["S"] / (dt_s / args.steps)
-
-    # per-kernel durations: a second pass of the same steps with an event pair around every kernel,
-    # recorded on the stream the kernel is launched on
-    L.kernel_timing_enable(True)
-    for _ in range(args.steps):
-        step(m, x, dy, cf)
-    torch.cuda.synchronize()
-    timing = L.kernel_timing_read()
-    L.kernel_timing_enable(False)
-
-    # the fused Adam update on one weight array of this layer ([E, F, M] parameters and gradients in the
-    # layer's dtype, fp32 moments): not part of the step above, measured for its own HBM roofline
-    from mole_amd import hip_ops as H
-    pdt = torch.bfloat16 if w["dtype"] == "bf16" else torch.float32
-    n_adam = w["E"] * w["F"] * w["M"]
-    ap_, ag_ = (torch.randn(n_adam, device="cuda") * 0.02).to(pdt), (torch.randn(n_adam, device="cuda") * 1e-3).to(pdt)
-    am_, av_ = torch.zeros(n_adam, device="cuda"), torch.zeros(n_adam, device="cuda")
-    H.adam_step(ap_, ag_, am_, av_, 0.9, 0.999, 1, 1e-3, 0.0, 1e-8, False)
-    torch.cuda.synchronize()
-    L.kernel_timing_enable(True)
-    for i in range(5):
-        H.adam_step(ap_, ag_, am_, av_, 0.9, 0.999, 2 + i, 1e-3, 0.0, 1e-8, False)
-    torch.cuda.synchronize()
-    adam_cnt, adam_ms = L.kernel_timing_read()["adam"]
-    L.kernel_timing_enable(False)
-    del ap_, ag_, am_, av_
-    adam_bytes = n_adam * (22.0 if pdt == torch.bfloat16 else 28.0)   # read p, g, m, v; write p, m, v
-    adam_gbs = adam_bytes / (adam_ms / adam_cnt * 1e-3) / 1e9
-
-    R = int(m.last_route.offsets[-1].item())       # kept (token, choice) rows
-    S, M, F, k = w["S"], w["M"], w["F"], w["k"]
-    b = 2 if w["dtype"] == "bf16" else 4
-    gemm_flop = 2.0 * R * M * F                     # every one of the six grouped products
-    work = {  # algorithmic work per launch: flop for the GEMMs, bytes for the permutes
-        "ffn_fwd1": gemm_flop, "ffn_fwd2": gemm_flop, "ffn_gw2": gemm_flop, "ffn_da": gemm_flop, "ffn_gw1": gemm_flop,
-        "ffn_gx": gemm_flop,
-        "dispatch_fwd": 2.0 * R * M * b, "combine_fwd": (R + S) * M * b, "combine_bwd": (S + 3.0 * R) * M * b,
-        "dispatch_bwd": (R + S) * M * b,
-    }
-    kernels = {}
-    for name, (cnt, ms) in timing.items():
-        if cnt == 0:
-            continue
-        avg_us = ms / cnt * 1e3
-        entry = {"avg_us": round(avg_us, 2), "launches_per_step": cnt / args.steps}
-        if name in work:
-            if name.startswith("ffn_"):
-                entry["tflops"] = round(work[name] / (avg_us * 1e-6) / 1e12, 1)
-            else:
-                entry["gbs"] = round(work[name] / (avg_us * 1e-6) / 1e9, 1)
-        kernels[name] = entry
-    gemms = [n for n in kernels if n in ("ffn_fwd1", "ffn_fwd2", "ffn_gw2", "ffn_da", "ffn_gw1", "ffn_gx")]
-    dom = max(gemms, key=lambda n: kernels[n]["avg_us"])
-    peak = PEAK_MFMA_TFLOPS[w["dtype"]]
-    gemm_total_us = sum(kernels[n]["avg_us"] for n in gemms)
-    roofline = {"bound": "mfma", "kernel": dom, "achieved": kernels[dom]["tflops"], "peak": peak, "unit": "TFLOP/s",
-                "frac": round(kernels[dom]["tflops"] / peak, 4),
-                "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload, {}).get(dom),
-                "all_ffn_gemms_frac": round(6 * gemm_flop / (gemm_total_us * 1e-6) / 1e12 / peak, 4)}
-
+    res = measure_layer(args.workload, args.steps, args.warmup)
     out = {
-        "metric": "MoE layer tokens/sec fwd+bwd on 1 MI355X", "value": round(value, 1), "unit": "tokens/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": w["dtype"], "data": "synthetic",
-        "config": {"workload": f"{args.workload}: single MoE layer fwd+bwd, S={S} M={M} E={w['E']} top-{k} F={F} "
-                               f"capacity_factor={cf}, kept rows R={R}"},
-        "roofline": roofline,
-        "hbm_permutes": {n: {"achieved": kernels[n]["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                             "frac": round(kernels[n]["gbs"] / PEAK_HBM_GBS, 4)}
-                         for n in ("dispatch_fwd", "combine_fwd", "combine_bwd", "dispatch_bwd") if n in kernels},
-        "hbm_optimizer": {"adam_step": {"achieved": round(adam_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                        "frac": round(adam_gbs / PEAK_HBM_GBS, 4), "elements": n_adam,
-                                        "avg_us": round(adam_ms / adam_cnt * 1e3, 2)}},
-        "kernels": kernels,
+        "metric": "MoE layer tokens/sec fwd+bwd on 1 MI355X", "value": res.pop("value"), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": res.pop("ms_per_step"),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": res.pop("dtype"), "data": "synthetic",
     }
+    out.update(res)
+    if args.workload != "c1" and not args.no_c1:
+        # configuration 1 (fp32, the case the CPU baseline runs) on the GPU, beside the headline
+        c1 = measure_layer("c1", args.steps, args.warmup, with_adam=False)
+        out["c1"] = {"tokens_per_s": c1["value"], "ms_per_step": c1["ms_per_step"], "dtype": c1["dtype"],
+                     "workload": c1["config"]["workload"], "roofline": c1["roofline"], "hbm_permutes": c1["hbm_permutes"]}
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(w)
+        out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
 
 

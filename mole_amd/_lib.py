@@ -19,7 +19,7 @@ LAYOUT_PADDED, LAYOUT_RAGGED = 0, 1
 GELU_BWD_TANH, GELU_BWD_EXACT = 0, 1
 MAX_TOPK, MAX_EXPERTS = 16, 1024
 KERNEL_IDS = ("ffn_fwd1", "ffn_fwd2", "ffn_gw2", "ffn_da", "ffn_gw1", "ffn_gx", "ffn_gb", "dispatch_fwd", "dispatch_bwd",
-              "combine_fwd", "combine_bwd", "route", "gemm_nt", "adam", "gate_fwd", "gate_bwd", "gate_wgrad")
+              "combine_fwd", "combine_bwd", "route", "gemm_nt", "adam", "gate_fwd", "gate_bwd", "gate_wgrad", "probe")
 
 _P = c_void_p
 _SIGNATURES = {
@@ -27,6 +27,9 @@ _SIGNATURES = {
     "mole_last_error_string": (c_char_p, []),
     "mole_kernel_timing_enable": (c_int, [c_int]),
     "mole_kernel_timing_read": (c_int, [c_int, POINTER(c_int), POINTER(c_float)]),
+    "mole_probe_mfma_operand_bytes": (c_size_t, []),
+    "mole_probe_mfma": (c_int, [_P, c_int, c_int, _P, POINTER(c_double), _P]),
+    "mole_probe_kloop": (c_int, [_P, _P, _P, _P, c_int, c_int, c_int, c_int, _P, _P]),
     "mole_softmax_fwd": (c_int, [_P, _P, c_int, c_int, _P, _P]),
     "mole_gate_fwd": (c_int, [_P, c_int, _P, _P, c_int, c_int, c_int, _P, _P]),
     "mole_softmax_bwd": (c_int, [_P, _P, c_int, c_int, _P, _P]),

@@ -32,7 +32,8 @@ __device__ __forceinline__ float d_gelu_exact(float x) {
     return cdf + x * pdf;
 }
 
-enum { EPI_STORE = 0, EPI_BIAS = 1, EPI_BIAS_GELU = 2, EPI_DGELU = 3, EPI_WGRAD = 4, EPI_F32 = 5 };
+enum { EPI_STORE = 0, EPI_BIAS = 1, EPI_BIAS_GELU = 2, EPI_DGELU = 3, EPI_WGRAD = 4, EPI_F32 = 5,
+       EPI_NONE = 6 /* measurement only: the K loop runs, nothing is stored */ };
 
 struct GemmArgs {
     const void *A, *B;      // operands (see A_KS / B_KS for their layout)
@@ -54,6 +55,7 @@ struct GemmArgs {
     int n_blocks;           // real number of tiles in the launch (grid is rounded up to 8)
     void *colsum;           // weight gradients, 256-wide kernel: [E][M] (side 1) or [E][N] (side 2) sums of an operand
     int colsum_side;        //   over the expert's rows: 1 = the m-side operand (A), 2 = the n-side operand (B)
+    int m_fastest;          // row-ragged products, 256-wide kernel: number an expert's tiles m-tile first (see gemm256.hip)
 };
 
 

@@ -472,6 +472,21 @@ __device__ __forceinline__ void epilogue(const GemmArgs &g, f32x16 (&acc)[Tile<T
         }
     };
 
+    if constexpr (EPI == EPI_NONE) {
+        // the K loop alone (mole_probe_kloop): results leave only under a condition that never holds, which is
+        // enough to keep the accumulation alive
+        if (g.K < 0) {
+            float s = 0.f;
+#pragma unroll
+            for (int tm = 0; tm < TMC; ++tm)
+#pragma unroll
+                for (int tn = 0; tn < 2; ++tn)
+#pragma unroll
+                    for (int q = 0; q < 16; ++q) s += acc[tm][tn][q];
+            ((float *)g.C)[threadIdx.x] = s;
+        }
+        return;
+    }
     if constexpr (EPI == EPI_F32) {
 #pragma unroll
         for (int tn = 0; tn < 2; ++tn)
@@ -618,9 +633,10 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
         // That order runs an expert's light tile long after its heavy ones, whose weight panels have left the L2 by
         // then; with many rounds of tiles the order matters little and the re-read does, so beyond 16 rounds
         // all tiles count as one class, in expert order.
+        auto tiles_of = [&](int r) { return (r + Q_BM - 1) / Q_BM; };     // m-tiles of an expert with r rows
         bool split = true;
         auto heavy_of = [&](int r) {
-            const int cnt = (r + Q_BM - 1) / Q_BM;
+            const int cnt = tiles_of(r);
             if (cnt == 0 || !split) return cnt;
             if (TMB == 10) return ((((r + cnt - 1) / cnt) + 31) & ~31) > Q_BM / 2 ? cnt : 0;
             return cnt - 1 + ((r - (cnt - 1) * Q_BM) > Q_BM / 2 ? 1 : 0);
@@ -630,7 +646,7 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
             const int r = ee < WAVE ? rows_lane : rows_of(ee);
             const int hv = heavy_of(r);
             n_h += hv;
-            n_l += (r + Q_BM - 1) / Q_BM - hv;
+            n_l += tiles_of(r) - hv;
         }
         for (int d = WAVE / 2; d >= 1; d >>= 1) { n_h += __shfl_xor(n_h, d, WAVE); n_l += __shfl_xor(n_l, d, WAVE); }
         if ((n_h + n_l) * n_tiles > 16 * 256) { split = false; n_h += n_l; n_l = 0; }
@@ -640,15 +656,22 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
         const bool heavy = slot < per_h;
         const int t = heavy ? xcd * per_h + slot : xcd * per_l + (slot - per_h);
         if (heavy ? t >= total_h : (slot - per_h >= per_l || t >= total_l)) return;
-        const int target = t / n_tiles;        // index among the m-tiles of the class
+        // Order of an XCD's tiles.  n-tile first: tile t = (m-tile t / n_tiles, n-tile t % n_tiles); the blocks that
+        // run side by side on an XCD are then a few m-tiles times all n-tiles, i.e. they stream the expert's whole
+        // weight matrix through the L2 once per group of m-tiles.  m-tile first (m_fastest): an expert's tiles are
+        // numbered n-tile by n-tile, all its m-tiles of the class inside; the blocks side by side are then all
+        // m-tiles of the expert times a few n-tiles, and every weight panel is fetched once.
+        const bool mf = g.m_fastest != 0;
+        const int unit = mf ? n_tiles : 1;       // tiles per counted m-tile
+        const int target = mf ? t : t / n_tiles;
         nt = t % n_tiles;
         // the expert whose running count (of the class) passes `target`
-        int run = 0, found = -1, before = 0;
+        int run = 0, found = -1, before = 0, cnt_found = 1;
         for (int base = 0; base < nE && found < 0; base += WAVE) {
             const int ee = base + lane;
             const int r = base == 0 ? rows_lane : (ee < nE ? rows_of(ee) : 0);
             const int hv = heavy_of(r);
-            const int cnt = heavy ? hv : (r + Q_BM - 1) / Q_BM - hv;
+            const int cnt = (heavy ? hv : tiles_of(r) - hv) * unit;
             int incl = cnt;
             for (int d = 1; d < WAVE; d <<= 1) {
                 const int y = __shfl_up(incl, d, WAVE);
@@ -659,13 +682,20 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
                 const int src = __ffsll(hit) - 1;
                 found = base + src;
                 before = run + __shfl(incl - cnt, src, WAVE);
+                cnt_found = __shfl(cnt, src, WAVE);
             }
             run += __shfl(incl, WAVE - 1, WAVE);
         }
         if (found < 0) return;
         e = found;
         m_ext = found < WAVE ? __shfl(rows_lane, found, WAVE) : rows_of(e);
-        mt = target - before + (heavy ? 0 : heavy_of(m_ext));   // an expert's light tiles follow its heavy ones
+        int mt_class = target - before;
+        if (mf) {
+            const int c_e = cnt_found / n_tiles;      // the expert's m-tiles of this class
+            nt = mt_class / c_e;
+            mt_class = mt_class % c_e;
+        }
+        mt = mt_class + (heavy ? 0 : heavy_of(m_ext));   // an expert's light tiles follow its heavy ones
         const int t_e = (m_ext + Q_BM - 1) / Q_BM;
         tile_h = TMB == 10 ? ((((m_ext + t_e - 1) / t_e) + 31) & ~31) : Q_BM;
         row0 = single ? 0 : (found < WAVE ? __shfl(off_lane, found, WAVE) : g.offsets[e]);
@@ -779,6 +809,16 @@ static int launch256(GemmArgs g, int tiles, hipStream_t st, int kid) {
     return 0;
 }
 
+// Which products number their tiles m-tile first (bit = MOLE_K_* id).  MOLE_MFAST in the environment overrides
+// the default (tuning aid).
+static int m_fastest_mask() {
+    static const int mask = [] {
+        const char *v = getenv("MOLE_MFAST");
+        return v ? atoi(v) : 0;
+    }();
+    return mask;
+}
+
 template <int TMB, int WM>
 static int dispatch256(const GemmArgs &g, bool b_ks, bool wg, int epi, int max_rows, hipStream_t st, int kid) {
     constexpr int BM = Tile<TMB, WM>::BM;
@@ -793,6 +833,7 @@ static int dispatch256(const GemmArgs &g, bool b_ks, bool wg, int epi, int max_r
     // block slots: the worst-case number of m-tiles (an expert with r rows has ceil(r / BM) of them)
     const int rows_bound = g.offsets ? max_rows : g.single_rows;
     GemmArgs gg = g;
+    gg.m_fastest = (m_fastest_mask() >> kid) & 1;
     // (+ 16: the heavy and the light tiles of an XCD are rounded up to whole slots separately)
     const int tiles = (((rows_bound / BM + (g.offsets ? g.E : 1)) * n_tiles + 7) & ~7) + 16;
     if (wg) return -100;
@@ -801,6 +842,7 @@ static int dispatch256(const GemmArgs &g, bool b_ks, bool wg, int epi, int max_r
             if (epi == EPI_DGELU) return launch256<TMB, WM, false, false, EPI_DGELU>(gg, tiles, st, kid);
             if (epi == EPI_BIAS_GELU) return launch256<TMB, WM, false, false, EPI_BIAS_GELU>(gg, tiles, st, kid);
             if (epi == EPI_F32) return launch256<TMB, WM, false, false, EPI_F32>(gg, tiles, st, kid);
+            if (epi == EPI_NONE) return launch256<TMB, WM, false, false, EPI_NONE>(gg, tiles, st, kid);
         }
     } else {
         if (epi == EPI_BIAS) return launch256<TMB, WM, true, false, EPI_BIAS>(gg, tiles, st, kid);

@@ -30,7 +30,7 @@ class _RouteFn(torch.autograd.Function):
         ctx.save_for_backward(scores, r.idx, r.counts)
         ctx.normalize_gate = normalize_gate
         ctx.mark_non_differentiable(r.idx, r.loc)
-        return r.gates, r.idx, r.loc, r.l_aux[0].clone()
+        return r.gates, r.idx, r.loc, r.l_aux.view(())
 
     @staticmethod
     def backward(ctx, dgates, _di, _dl, d_l_aux):

@@ -70,7 +70,7 @@ class _FusedMoE(torch.autograd.Function):
         m.last_route = r
         ctx.m, ctx.r, ctx.saved = m, r, saved
         ctx.save_for_backward(x, wg, scores, out)
-        return y, r.l_aux[0].clone()
+        return y, r.l_aux.view(())
 
     @staticmethod
     def backward(ctx, dy, d_l_aux):
