@@ -131,7 +131,8 @@ def bench_offloaded_stack(args):
     for i in range(n_layers):
         print(f"[c4] building layer {i} (pinned host weights)", file=sys.stderr, flush=True)
         try:
-            layers.append(MOLEModule(E, 0, M, F, pool, k, ebatch, dist, "gelu", 1, bool(args.adam), True, dtype=torch.bfloat16))
+            layers.append(MOLEModule(E, 0, M, F, pool, k, ebatch, dist, "gelu", 1, bool(args.adam), True, dtype=torch.bfloat16,
+                                     resident=not args.no_resident))
         except RuntimeError as exc:     # pinned host memory is capped well below the machine's RAM on some boxes
             print(f"[c4] layer {i} could not be built ({str(exc).splitlines()[0]}): lower --layers", file=sys.stderr)
             sys.exit(3)
@@ -171,6 +172,7 @@ def bench_offloaded_stack(args):
     wall = (time.perf_counter() - t0) / args.steps
     h2d_bytes, h2d_ms = um.copy_stats()
     h2d_bytes /= args.steps; h2d_ms /= args.steps
+    resident = all(m.MOLECore.resident and m.MOLECore._home_base() is not None for m in layers)
     d2h_bytes, d2h_ms = um.writeback_stats()
     d2h_bytes /= args.steps; d2h_ms /= args.steps
     L.kernel_timing_enable(True)
@@ -188,11 +190,15 @@ def bench_offloaded_stack(args):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"c4: {n_layers}-layer offloaded-expert stack fwd+bwd, S={S} M={M} E={E} top-{k} F={F}, "
                                f"experts in pinned host memory, pool {pool} slots, chunks of {ebatch} experts"
+                               + (", experts kept in the pool from forward to backward" if resident else ", experts fetched for every pass")
                                + (", in-pipeline AdamW on the GPU (fp32 moments in pinned host memory)" if args.adam else "")},
         "prefetch": {"h2d_bytes_per_step": int(h2d_bytes), "h2d_busy_ms": round(h2d_ms, 2),
                      "h2d_gbs": round(h2d_bytes / (h2d_ms * 1e-3) / 1e9, 2),
                      "h2d_busy_frac_of_step": round(h2d_ms / (wall * 1e3), 4),
-                     "expected_h2d_bytes": (2 + (4 if args.adam else 0)) * n_layers * E * expert_bytes,
+                     # every activated expert once per pass, or once per step when the pool keeps it from the
+                     # forward pass to the backward pass (plus the fp32 moments for the in-pipeline optimizer)
+                     "expected_h2d_bytes": ((1 if resident else 2) + (4 if args.adam else 0)) * n_layers * E * expert_bytes,
+                     "experts_resident_from_forward_to_backward": resident,
                      "d2h_gradient_bytes_per_step": int(d2h_bytes), "d2h_busy_ms": round(d2h_ms, 2),
                      "d2h_gbs": round(d2h_bytes / (d2h_ms * 1e-3) / 1e9, 2)},
         "kernel_ms_per_step": round(kernel_ms, 2),
@@ -396,6 +402,8 @@ def main():
     ap.add_argument("--layers", type=int, default=2, help="depth of the c4 stack (12 in the configuration)")
     ap.add_argument("--adam", action="store_true",
                     help="c4 only: update the offloaded experts with the in-pipeline Adam (adds 30 GB of pinned moments per layer)")
+    ap.add_argument("--no-resident", action="store_true",
+                    help="c4 only: fetch the experts again for every backward pass, as the reference does")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-c1", action="store_true", help="skip the configuration-1 (fp32) figures beside the headline")
     ap.add_argument("--probe", action="store_true", help="run the matrix-core and K-loop probes instead of the layer")

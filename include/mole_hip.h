@@ -273,7 +273,12 @@ int mole_gemm_tn(const void *a, const void *b, int dtype, int rows, int Mo, int 
  * host side can bring in only the experts that routing activated (kept_rows[e] > 0) and hand the grouped
  * FFN a compacted offsets / kept_rows pair in the same order.  The reference always copies whole index
  * ranges (MOLE/cpp/core.cpp:41-57, 1025-1047); these two have no counterpart there.  Consecutive ids that
- * go to consecutive slots still travel as one copy per parameter kind.
+ * `tag` (0: none) lets a slot keep what it holds: a slot last filled under the same non-zero tag from the same
+ * host expert is not copied again.  The caller vouches that the host arrays are unchanged since that copy; the
+ * host side hands out one tag per forward pass of a layer and uses it again only for that pass's backward, so
+ * that experts still resident from the forward are not fetched a second time (the reference always fetches
+ * again, MOLE/cpp/core.cpp:1203).  mole_unimem_reuse_stats: bytes of the requests answered that way since the last
+ * read (an expert asked for twice while in place counts twice).
  * ------------------------------------------------------------------------------------------ */
 int mole_unimem_create(int device, int pool_size, int dtype, int64_t F, int64_t M, void **handle);
 int mole_unimem_destroy(void *handle);
@@ -283,7 +288,7 @@ int mole_unimem_virtual_offset(void *handle, int *out);
 int mole_unimem_slot_ptr(void *handle, int p_id, int slot, void **out);
 int mole_unimem_prefetch(void *handle, int layer, const void *const host_src[4], int base, int n);
 int mole_unimem_prefetch_ids(void *handle, int layer, const void *const host_src[4], const int32_t *expert_ids,
-                             int n);
+                             int n, uint64_t tag);
 /* The bookkeeping half of prefetch alone (_UniMem::prefetch, MOLE/cpp/umemory.cpp:131-154, exported by the
  * reference as pool_prefetch, MOLE/cpp/core.cpp:1425): reserve n slots for `layer` and return their addresses;
  * the caller fills them and orders its copies against the compute stream itself. */
@@ -292,7 +297,7 @@ int mole_unimem_fetch_top(void *handle, int layer, int *n_out);
 int mole_unimem_fetch(void *handle, const void *const host_src[4], int view_base, int base, int n,
                       int prefetched, void **slot_ptrs_out /* [4] */);
 int mole_unimem_fetch_ids(void *handle, const void *const host_src[4], int view_base, const int32_t *expert_ids,
-                          int n, int prefetched, void **slot_ptrs_out /* [4] */);
+                          int n, int prefetched, uint64_t tag, void **slot_ptrs_out /* [4] */);
 int mole_unimem_wait_params(void *handle, mole_stream_t compute_stream);
 int mole_unimem_wait_slots(void *handle, int view_base, int n, mole_stream_t compute_stream);
 int mole_unimem_release(void *handle, int view_base, int n, mole_stream_t compute_stream);
@@ -302,6 +307,7 @@ int mole_unimem_tran_stream(void *handle, mole_stream_t *out);
  * that mole_unimem_sync_tran() calls have waited for since the previous mole_unimem_copy_stats(); reading
  * resets the sums */
 int mole_unimem_copy_stats(void *handle, uint64_t *bytes, float *busy_ms);
+int mole_unimem_reuse_stats(void *handle, uint64_t *bytes);
 
 /* Gradient write-back of offloaded experts; replaces _MOLECore::store_grad / _CPUParamCore::store_grad
  * (MOLE/cpp/core.cpp:77-103, MOLE/cpp/uparameter.cpp:68-83) and the "tranback" stream

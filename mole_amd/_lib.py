@@ -60,17 +60,18 @@ _SIGNATURES = {
     "mole_unimem_virtual_offset": (c_int, [_P, POINTER(c_int)]),
     "mole_unimem_slot_ptr": (c_int, [_P, c_int, c_int, POINTER(_P)]),
     "mole_unimem_prefetch": (c_int, [_P, c_int, POINTER(_P), c_int, c_int]),
-    "mole_unimem_prefetch_ids": (c_int, [_P, c_int, POINTER(_P), POINTER(c_int32), c_int]),
+    "mole_unimem_prefetch_ids": (c_int, [_P, c_int, POINTER(_P), POINTER(c_int32), c_int, c_uint64]),
     "mole_unimem_reserve": (c_int, [_P, c_int, c_int, POINTER(_P)]),
     "mole_unimem_fetch_top": (c_int, [_P, c_int, POINTER(c_int)]),
     "mole_unimem_fetch": (c_int, [_P, POINTER(_P), c_int, c_int, c_int, c_int, POINTER(_P)]),
-    "mole_unimem_fetch_ids": (c_int, [_P, POINTER(_P), c_int, POINTER(c_int32), c_int, c_int, POINTER(_P)]),
+    "mole_unimem_fetch_ids": (c_int, [_P, POINTER(_P), c_int, POINTER(c_int32), c_int, c_int, c_uint64, POINTER(_P)]),
     "mole_unimem_wait_params": (c_int, [_P, _P]),
     "mole_unimem_wait_slots": (c_int, [_P, c_int, c_int, _P]),
     "mole_unimem_release": (c_int, [_P, c_int, c_int, _P]),
     "mole_unimem_sync_tran": (c_int, [_P]),
     "mole_unimem_tran_stream": (c_int, [_P, POINTER(_P)]),
     "mole_unimem_copy_stats": (c_int, [_P, POINTER(c_uint64), POINTER(c_float)]),
+    "mole_unimem_reuse_stats": (c_int, [_P, POINTER(c_uint64)]),
     "mole_unimem_store_grads": (c_int, [_P, POINTER(_P), POINTER(_P), c_int, c_int, _P]),
     "mole_unimem_store_grads_ids": (c_int, [_P, POINTER(_P), POINTER(_P), POINTER(c_int32), c_int, _P]),
     "mole_unimem_zero_grads_ids": (c_int, [_P, POINTER(_P), POINTER(c_int32), c_int]),

@@ -84,17 +84,24 @@ class UniMem:
     def _ids(ids):
         return (ctypes.c_int32 * max(len(ids), 1))(*[int(e) for e in ids])
 
-    def prefetch_ids(self, layer: int, host_tensors, ids):
-        """prefetch() for an explicit list of experts: ids[i] lands in the i-th reserved slot."""
-        L.check(L.lib().mole_unimem_prefetch_ids(self._h, layer, self._src(host_tensors), self._ids(ids), len(ids)),
+    def prefetch_ids(self, layer: int, host_tensors, ids, tag: int = 0):
+        """prefetch() for an explicit list of experts: ids[i] lands in the i-th reserved slot.  tag != 0: slots
+        that were filled under the same tag from the same host expert keep what they hold."""
+        L.check(L.lib().mole_unimem_prefetch_ids(self._h, layer, self._src(host_tensors), self._ids(ids), len(ids), tag),
                 "mole_unimem_prefetch_ids")
 
-    def fetch_ids(self, host_tensors, view_base: int, ids, prefetched: int) -> List[int]:
+    def fetch_ids(self, host_tensors, view_base: int, ids, prefetched: int, tag: int = 0) -> List[int]:
         """fetch() for an explicit list of experts (the first `prefetched` of them are already in their slots)."""
         ptrs = (c_void_p * 4)()
         L.check(L.lib().mole_unimem_fetch_ids(self._h, self._src(host_tensors), view_base, self._ids(ids), len(ids),
-                                              prefetched, ptrs), "mole_unimem_fetch_ids")
+                                              prefetched, tag, ptrs), "mole_unimem_fetch_ids")
         return [int(p) for p in ptrs]
+
+    def reuse_stats(self) -> int:
+        """Bytes that were not copied because their slot still held the expert (since the last read)."""
+        b = c_uint64()
+        L.check(L.lib().mole_unimem_reuse_stats(self._h, ctypes.byref(b)), "mole_unimem_reuse_stats")
+        return b.value
 
     def wait_params(self):
         L.check(L.lib().mole_unimem_wait_params(self._h, L.stream()), "mole_unimem_wait_params")
@@ -378,11 +385,21 @@ class MOLECore:
     prefetch_bwd prefetches only experts the forward pass activated; prefetch_fwd, which runs before the layer's
     routing exists, prefetches the experts the previous step activated (none before the first step) - a wrong
     guess costs a copy, never a result.  The reference copies and runs every expert of every chunk in index
-    order (core.cpp:41-57, 1025-1047); activated_only=False does the same."""
+    order (core.cpp:41-57, 1025-1047); activated_only=False does the same.
+
+    resident (default): what a layer's forward pass brought into the pool is not fetched again for its backward
+    pass while it is still there.  Every forward pass copies under a tag of its own and the backward pass asks
+    for its experts under the same tag; the pool skips a slot that still holds that expert under that tag.  When
+    the pool has a slot for every offloaded expert of every layer (an MI355X holds 288 GB), each layer keeps a
+    fixed stretch of slots, expert e at its base + e, nothing is ever displaced between a forward and its
+    backward, and the host-to-device traffic of a step halves; with a smaller pool the slots are recycled
+    through the prefetch stack as in the reference (umemory.cpp:131-183) and only what happens to survive (the last
+    layer's experts, whose backward follows its forward directly) is reused.  The reference fetches the weights
+    again for every backward (core.cpp:1203)."""
 
     def __init__(self, use_pool, mome_use_pool, vari_use_pool, grad_use_pool, s_experts, d_experts, ebatch_size,
                  world_size, act_name, adv_adam, acc_step, step, device, moe_id, total_experts,
-                 gelu_bwd: str = "tanh", activated_only: bool = True):
+                 gelu_bwd: str = "tanh", activated_only: bool = True, resident: bool = True):
         if world_size != 1:
             raise NotImplementedError("this build covers the single-GPU hot path (world_size == 1)")
         if act_name != "gelu":
@@ -403,6 +420,10 @@ class MOLECore:
         self._active = None                   # offloaded experts the last forward gave rows to (None: not known)
         self._grad_is_zero = [False] * d_experts   # the expert's pinned host gradient is known to hold zeros
         self.lazy_zero = True
+        self.resident = bool(resident)
+        self._passes = 0            # forward passes so far: part of the tag under which a pass fills pool slots
+        self._tag = 0               # tag of the pass in preparation or in flight (0: none yet)
+        self._tag_used = True       # a forward pass has run under _tag: the next prefetch_fwd / forward takes a new one
 
     # the reference's counters of experts prefetched so far (define.hpp:352-353)
     @property
@@ -450,22 +471,56 @@ class MOLECore:
         return [c[0] for c in self.cpu]
 
     # prefetch -----------------------------------------------------------------------------------
+    def _forward_tag(self) -> int:
+        """The tag of the coming (or running) forward pass: a new one unless a prefetch already took it."""
+        if not self.resident:
+            return 0
+        if self._tag_used:
+            self._passes += 1
+            self._tag = ((self.moe_id + 1) << 40) | self._passes
+            self._tag_used = False
+        return self._tag
+
+    def _home_base(self):
+        """First slot of this layer's fixed stretch of the pool, or None when the pool cannot give every offloaded
+        expert of every layer a slot of its own (then the slots are recycled through the prefetch stack)."""
+        if not self.resident or self.d_experts == 0 or not self.use_pool:
+            return None
+        um = get_UniMem()
+        from .moe.layer import MOLEModule
+        layers = [m.MOLECore for m in MOLEModule._instance]
+        if um is None or self not in layers or not all(c.resident for c in layers):
+            return None
+        if sum(c.d_experts for c in layers) > um.pool_size or um.virtual_offset() != 0:
+            return None
+        return sum(c.d_experts for c in layers[:layers.index(self)])
+
+    def _home_fetch(self, home: int, ids, tag: int):
+        """Bring the experts `ids` into their own slots (home + e); runs of consecutive experts in one call."""
+        um = get_UniMem()
+        for (at, e0, n) in self._runs(list(ids)):
+            um.fetch_ids(self._host(), home + e0, ids[at:at + n], 0, tag)
+
     def _prefetch(self, which: str, batch_size: int):
         if batch_size <= 0 or self.d_experts == 0:
             return
         done = self._pref[which]
+        tag = self._forward_tag() if which == "fwd" else self._tag
         if not self.activated_only:
             todo = list(range(len(done), min(self.d_experts, len(done) + batch_size)))
-            if not todo:
-                return
-            get_UniMem().prefetch(self.moe_id, self._host(), todo[0], len(todo))
         else:
             known = self._active if self._active is not None else []
             seen = set(done)
             todo = [e for e in known if e not in seen][:batch_size]
-            if not todo:
-                return
-            get_UniMem().prefetch_ids(self.moe_id, self._host(), todo)
+        if not todo:
+            return
+        home = self._home_base()
+        if home is not None:
+            self._home_fetch(home, todo, tag)
+        elif not self.activated_only:
+            get_UniMem().prefetch(self.moe_id, self._host(), todo[0], len(todo))
+        else:
+            get_UniMem().prefetch_ids(self.moe_id, self._host(), todo, tag)
         done.extend(todo)
 
     def prefetch_fwd(self, batch_size: int):
@@ -482,13 +537,16 @@ class MOLECore:
         um.fetch(self._host(), -um.virtual_offset(), 0, batch_size, 0)
 
     # pipeline -----------------------------------------------------------------------------------
-    def _take_prefetched(self, which: str):
-        """Pops this layer's entry of the prefetch stack; returns the experts it holds, in slot order."""
+    def _take_prefetched(self, which: str, home):
+        """The experts prefetched for this pass, in slot order; pops this layer's entry of the prefetch stack
+        (experts with slots of their own never enter the stack)."""
         um = get_UniMem()
         if not self.use_pool or um is None or um.pool_size <= 0:
             raise RuntimeError("offloaded experts need the slot pool (pool_size >= 1, use_pool=True)")
-        n = um.fetch_top(self.moe_id)
         ids, self._pref[which] = self._pref[which], []
+        if home is not None:
+            return ids
+        n = um.fetch_top(self.moe_id)
         if n != len(ids):
             raise RuntimeError(f"prefetch stack out of order: top holds {n}, layer expects {len(ids)}")
         return ids
@@ -512,6 +570,17 @@ class MOLECore:
         comp = torch.tensor([[off_h[e] for e in order], [kept_h[e] for e in order]], dtype=torch.int32)
         comp = comp.to(offsets.device)
         return order, comp[0], comp[1]
+
+    def _home_chunks(self, home: int, wanted):
+        """Expert ranges [e0, e0 + size) of at most ebatch_size experts that hold a wanted expert, with the device
+        addresses of their slots."""
+        um = get_UniMem()
+        want = set(wanted)
+        for e0 in range(0, self.d_experts, self.ebatch_size):
+            size = min(self.ebatch_size, self.d_experts - e0)
+            ids = [e for e in range(e0, e0 + size) if e in want]
+            if ids:
+                yield e0, size, ids, [um.slot_tensor(p, home + e0, size) for p in range(4)]
 
     def forward(self, dispatched_input: torch.Tensor, requires_grad: bool, offsets=None, kept_rows=None,
                 return_saved: bool = False):
@@ -539,10 +608,13 @@ class MOLECore:
         if self.s_experts:
             w1, b1, w2, b2 = (g[0] for g in self.gpu)
             H.ffn_fwd_into(x2, offsets, kept_rows, self.s_experts, rows, M, F, w1, b1, w2, b2, h, a, out)
-        host_meta = None
+        host_meta, tag = None, 0
         if self.d_experts:
             um = get_UniMem()
-            resident = self._take_prefetched("fwd")
+            home = self._home_base()
+            resident = self._take_prefetched("fwd", home)
+            tag = self._forward_tag()
+            self._tag_used = True
             d, e0 = self.d_experts, self.s_experts
             if self.activated_only and routed:
                 # the one host synchronisation of the path: E row counts (and row offsets) come back
@@ -553,13 +625,22 @@ class MOLECore:
             else:
                 self._active = list(range(d))       # every expert runs
                 wanted = range(d)
-            order, off_c, kept_c = self._order(resident, wanted, offsets, kept_rows, host_meta)
-            for (lo, size, pref, view_base) in self._chunks(len(order), len(resident)):
-                p = um.fetch_ids(self._host(), view_base, order[lo:lo + size], pref)
-                um.wait_slots(view_base, size)
-                H.ffn_fwd_into(x2, off_c[lo:], kept_c[lo:], size, rows, M, F, p[0], p[1], p[2], p[3], h, a, out)
-                um.release(view_base, size)
-        saved = (x2, h, a, offsets, kept_rows, requires_grad, shape, host_meta)
+            if home is not None:
+                # every expert has a slot of its own: the copies of all wanted experts are issued now, each chunk
+                # waits for its own, and experts without rows are simply not copied (the kernel skips them)
+                self._home_fetch(home, list(wanted), tag)
+                for (c0, size, _, p) in self._home_chunks(home, wanted):
+                    um.wait_slots(home + c0, size)
+                    H.ffn_fwd_into(x2, offsets[e0 + c0:], kept_rows[e0 + c0:], size, rows, M, F, p[0], p[1], p[2], p[3], h, a, out)
+                    um.release(home + c0, size)
+            else:
+                order, off_c, kept_c = self._order(resident, wanted, offsets, kept_rows, host_meta)
+                for (lo, size, pref, view_base) in self._chunks(len(order), len(resident)):
+                    p = um.fetch_ids(self._host(), view_base, order[lo:lo + size], pref, tag)
+                    um.wait_slots(view_base, size)
+                    H.ffn_fwd_into(x2, off_c[lo:], kept_c[lo:], size, rows, M, F, p[0], p[1], p[2], p[3], h, a, out)
+                    um.release(view_base, size)
+        saved = (x2, h, a, offsets, kept_rows, requires_grad, shape, host_meta, tag)
         if return_saved:          # the caller (an autograd node) keeps the activations itself
             return out.view(shape), saved
         self._saved = saved       # reference behaviour: the core holds them until backward (define.hpp:594-606)
@@ -570,7 +651,7 @@ class MOLECore:
             saved, self._saved = self._saved, None
         if saved is None:
             raise RuntimeError("MOLECore.backward without a preceding forward")
-        x2, h, a, offsets, kept_rows, need_gx, shape, host_meta = saved
+        x2, h, a, offsets, kept_rows, need_gx, shape, host_meta, tag = saved
         M = shape[-1]
         go = all_output_grad.reshape(-1, M)
         if not go.is_contiguous():
@@ -587,38 +668,56 @@ class MOLECore:
                            gx, acc, self.gelu_bwd)
         if self.d_experts:
             um = get_UniMem()
-            resident = self._take_prefetched("bwd")
-            d = self.d_experts
+            home = self._home_base()
+            resident = self._take_prefetched("bwd", home)
+            d, e0 = self.d_experts, self.s_experts
             host_grads = [c[1] for c in self.cpu]
             adam_now = self.adv_adam and (self.step + 1) % self.acc_step == 0
             adding = self.acc_step > 1 and not getattr(host_grads[0], "lazy_zero", True)
             if host_meta is not None:
                 active = [e for e in range(d) if host_meta[1][e] > 0]
                 # the optimizer moves every parameter it owns, also those whose gradient is zero
-                wanted = range(d) if adam_now else active
+                wanted = list(range(d)) if adam_now else active
             else:
-                active, wanted = list(range(d)), range(d)
-            order, off_c, kept_c = self._order(resident, wanted, offsets, kept_rows, host_meta)
-            for (lo, size, pref, view_base) in self._chunks(len(order), len(resident)):
-                ids = order[lo:lo + size]
-                p = um.fetch_ids(self._host(), view_base, ids, pref)   # weights are fetched again (core.cpp:1203)
-                um.wait_slots(view_base, size)
-                g = [torch.empty((size, *hg.shape[1:]), dtype=hg.dtype, device=x2.device) for hg in host_grads]
-                H.ffn_bwd_into(go, x2, h, a, off_c[lo:], kept_c[lo:], size, rows, M, F, p[0], p[2], t, g[0], g[1],
-                               g[2], g[3], gx, False, self.gelu_bwd)
-                if adam_now:
-                    # the update reads the parameters in their pool slots, so the slots are released after it
-                    self._instant_adam(p, g, ids, adding)
-                    um.release(view_base, size)
-                else:
-                    um.release(view_base, size)
-                    self._store_grad(host_grads, g, ids, adding)
+                active, wanted = list(range(d)), list(range(d))
+            new_g = lambda n: [torch.empty((n, *hg.shape[1:]), dtype=hg.dtype, device=x2.device) for hg in host_grads]
+            if home is not None:
+                self._home_fetch(home, wanted, tag)       # what the forward left in place is not copied again
+                for (c0, size, ids, p) in self._home_chunks(home, wanted):
+                    um.wait_slots(home + c0, size)
+                    g = new_g(size)
+                    H.ffn_bwd_into(go, x2, h, a, offsets[e0 + c0:], kept_rows[e0 + c0:], size, rows, M, F, p[0], p[2], t,
+                                   g[0], g[1], g[2], g[3], gx, False, self.gelu_bwd)
+                    if adam_now:
+                        self._instant_adam(p, g, list(range(c0, c0 + size)), adding)
+                        um.release(home + c0, size)
+                    else:
+                        um.release(home + c0, size)
+                        for (at, r0, n) in self._runs(ids):       # the experts of the chunk that got rows
+                            self._store_grad(host_grads, [gg[r0 - c0:r0 - c0 + n] for gg in g], list(range(r0, r0 + n)), adding)
+                seen = set(wanted)
+            else:
+                order, off_c, kept_c = self._order(resident, wanted, offsets, kept_rows, host_meta)
+                for (lo, size, pref, view_base) in self._chunks(len(order), len(resident)):
+                    ids = order[lo:lo + size]
+                    p = um.fetch_ids(self._host(), view_base, ids, pref, tag)   # the reference fetches again (core.cpp:1203)
+                    um.wait_slots(view_base, size)
+                    g = new_g(size)
+                    H.ffn_bwd_into(go, x2, h, a, off_c[lo:], kept_c[lo:], size, rows, M, F, p[0], p[2], t, g[0], g[1],
+                                   g[2], g[3], gx, False, self.gelu_bwd)
+                    if adam_now:
+                        # the update reads the parameters in their pool slots, so the slots are released after it
+                        self._instant_adam(p, g, ids, adding)
+                        um.release(view_base, size)
+                    else:
+                        um.release(view_base, size)
+                        self._store_grad(host_grads, g, ids, adding)
+                seen = set(order)
             if host_meta is not None:
                 # experts that got no row: their gradient is zero.  While sums are being built up that adds
                 # nothing; otherwise the host array must read zero, which costs a copy only if it does not already
                 act = set(active)
                 if not adding:
-                    seen = set(order)
                     stale = [e for e in range(d) if e not in seen and not self._grad_is_zero[e]]
                     um.zero_grads_ids(host_grads, stale)
                     for e in range(d):

@@ -28,6 +28,9 @@ struct UniMem {
     std::vector<char> slot_pending;  // slot_event[s] was recorded and not yet waited on
     std::vector<hipEvent_t> landed_event;   // recorded on the copy stream once the slot's expert has arrived
     std::vector<char> landed_valid;
+    std::vector<uint64_t> slot_tag;         // the caller's tag under which the slot was last filled (0: none)
+    std::vector<const void *> slot_src;     // host address of the expert (its first parameter array) the slot holds
+    uint64_t bytes_reused = 0;
     std::vector<std::array<int, 2>> stk;  // (layer, n)
     int virtual_offset = 0, view_pool_size = 0;
     // copy statistics
@@ -66,14 +69,29 @@ static int next_timer(UniMem *u, std::array<hipEvent_t, 2> **out) { return next_
 // prefetch made a layer wait for all of it: 134 ms for 32 experts of 235 MB).  Before a slot is overwritten the
 // copy stream waits for the compute that last used it, slot by slot, so that a prefetch trails the compute
 // that still owns the later slots instead of waiting for all of it.
-static int copy_experts(UniMem *u, const void *const host_src[4], int slot0, const int32_t *ids, int base, int n) {
+//
+// tag != 0: a slot that was last filled under the same tag from the same host expert is left as it is (nothing is
+// copied, its earlier "landed" event still stands): the caller vouches that the host arrays have not changed since -
+// the host side hands out one tag per forward pass of a layer and uses it again for that pass's backward only.
+static int copy_experts(UniMem *u, const void *const host_src[4], int slot0, const int32_t *ids, int base, int n,
+                        uint64_t tag = 0) {
     if (n <= 0) return 0;
     auto id_of = [&](int i) { return ids ? (int)ids[i] : base + i; };
     int i = 0;
     while (i < n) {
-        // a run: experts up to the next slot that is still waited for (one pair of timing events per run)
+        auto resident = [&](int j) {
+            return tag != 0 && u->slot_tag[slot0 + j] == tag &&
+                   u->slot_src[slot0 + j] == (const char *)host_src[0] + (size_t)id_of(j) * u->slot_bytes[0];
+        };
+        if (resident(i)) {
+            for (int p = 0; p < 4; ++p) u->bytes_reused += u->slot_bytes[p];
+            ++i;
+            continue;
+        }
+        // a run: experts up to the next slot that is still waited for or already holds its expert (one pair of
+        // timing events per run)
         int run = 1;
-        while (i + run < n && !u->slot_pending[slot0 + i + run]) ++run;
+        while (i + run < n && !u->slot_pending[slot0 + i + run] && !resident(i + run)) ++run;
         if (u->slot_pending[slot0 + i]) {
             MOLE_HIP(hipStreamWaitEvent(u->tran, u->slot_event[slot0 + i], 0));
             u->slot_pending[slot0 + i] = 0;
@@ -90,6 +108,8 @@ static int copy_experts(UniMem *u, const void *const host_src[4], int slot0, con
             }
             MOLE_HIP(hipEventRecord(u->landed_event[slot0 + j], u->tran));
             u->landed_valid[slot0 + j] = 1;
+            u->slot_tag[slot0 + j] = tag;
+            u->slot_src[slot0 + j] = (const char *)host_src[0] + (size_t)id_of(j) * u->slot_bytes[0];
         }
         MOLE_HIP(hipEventRecord((*tm)[1], u->tran));
         i += run;
@@ -126,6 +146,8 @@ static int create_members(UniMem *u) {
     for (int s = 0; s < u->pool_size; ++s) MOLE_HIP(hipEventCreateWithFlags(&u->slot_event[s], hipEventDisableTiming));
     u->landed_event.assign(u->pool_size, nullptr);
     u->landed_valid.assign(u->pool_size, 0);
+    u->slot_tag.assign(u->pool_size, 0);
+    u->slot_src.assign(u->pool_size, nullptr);
     for (int s = 0; s < u->pool_size; ++s) MOLE_HIP(hipEventCreateWithFlags(&u->landed_event[s], hipEventDisableTiming));
     return 0;
 }
@@ -212,7 +234,8 @@ extern "C" int mole_unimem_slot_ptr(void *handle, int p_id, int slot, void **out
     return 0;
 }
 
-static int prefetch_impl(UniMem *u, const char *who, int layer, const void *const host_src[4], const int32_t *ids, int base, int n) {
+static int prefetch_impl(UniMem *u, const char *who, int layer, const void *const host_src[4], const int32_t *ids, int base, int n,
+                         uint64_t tag) {
     if (n == 0) return 0;
     MOLE_REQUIRE(n > 0 && base >= 0 && host_src && host_src[0] && host_src[1] && host_src[2] && host_src[3] && (!ids || ids_ok(ids, n)),
                  "%s: bad arguments (base=%d n=%d)", who, base, n);
@@ -220,7 +243,7 @@ static int prefetch_impl(UniMem *u, const char *who, int layer, const void *cons
         set_error("%s: %d experts do not fit the %d free pool slots", who, n, u->view_pool_size);
         return MOLE_E_STATE;
     }
-    if (int rc = copy_experts(u, host_src, u->virtual_offset, ids, base, n)) return rc;
+    if (int rc = copy_experts(u, host_src, u->virtual_offset, ids, base, n, tag)) return rc;
     if (!u->stk.empty() && u->stk.back()[0] == layer) u->stk.back()[1] += n;
     else u->stk.push_back({layer, n});
     u->virtual_offset += n;
@@ -230,13 +253,14 @@ static int prefetch_impl(UniMem *u, const char *who, int layer, const void *cons
 
 extern "C" int mole_unimem_prefetch(void *handle, int layer, const void *const host_src[4], int base, int n) {
     UM(handle);
-    return prefetch_impl(u, "mole_unimem_prefetch", layer, host_src, nullptr, base, n);
+    return prefetch_impl(u, "mole_unimem_prefetch", layer, host_src, nullptr, base, n, 0);
 }
 
-extern "C" int mole_unimem_prefetch_ids(void *handle, int layer, const void *const host_src[4], const int32_t *expert_ids, int n) {
+extern "C" int mole_unimem_prefetch_ids(void *handle, int layer, const void *const host_src[4], const int32_t *expert_ids, int n,
+                                        uint64_t tag) {
     UM(handle);
     MOLE_REQUIRE(n == 0 || expert_ids, "mole_unimem_prefetch_ids: null expert list");
-    return prefetch_impl(u, "mole_unimem_prefetch_ids", layer, host_src, expert_ids, 0, n);
+    return prefetch_impl(u, "mole_unimem_prefetch_ids", layer, host_src, expert_ids, 0, n, tag);
 }
 
 extern "C" int mole_unimem_reserve(void *handle, int layer, int n, void **slot_ptrs_out) {
@@ -248,6 +272,7 @@ extern "C" int mole_unimem_reserve(void *handle, int layer, int n, void **slot_p
     }
     for (int p = 0; p < 4; ++p) slot_ptrs_out[p] = u->pool_size > 0 ? u->pool[p] + (size_t)u->virtual_offset * u->slot_bytes[p] : nullptr;
     if (n == 0) return 0;
+    for (int s = u->virtual_offset; s < u->virtual_offset + n; ++s) u->slot_tag[s] = 0;   // the caller fills them
     if (!u->stk.empty() && u->stk.back()[0] == layer) u->stk.back()[1] += n;
     else u->stk.push_back({layer, n});
     u->virtual_offset += n;
@@ -270,7 +295,7 @@ extern "C" int mole_unimem_fetch_top(void *handle, int layer, int *n_out) {
 }
 
 static int fetch_impl(UniMem *u, const char *who, const void *const host_src[4], int view_base, const int32_t *ids, int base, int n,
-                      int prefetched, void **slot_ptrs_out) {
+                      int prefetched, uint64_t tag, void **slot_ptrs_out) {
     const int slot0 = view_base + u->virtual_offset;
     MOLE_REQUIRE(n > 0 && slot0 >= 0 && base >= 0 && prefetched >= 0 && prefetched <= n && host_src && slot_ptrs_out &&
                      (!ids || ids_ok(ids, n)),
@@ -279,7 +304,7 @@ static int fetch_impl(UniMem *u, const char *who, const void *const host_src[4],
         set_error("%s: slots %d..%d exceed the pool of %d", who, slot0, slot0 + n, u->pool_size);
         return MOLE_E_STATE;
     }
-    if (int rc = copy_experts(u, host_src, slot0 + prefetched, ids ? ids + prefetched : nullptr, base + prefetched, n - prefetched)) return rc;
+    if (int rc = copy_experts(u, host_src, slot0 + prefetched, ids ? ids + prefetched : nullptr, base + prefetched, n - prefetched, tag)) return rc;
     for (int p = 0; p < 4; ++p) slot_ptrs_out[p] = u->pool[p] + (size_t)slot0 * u->slot_bytes[p];
     return 0;
 }
@@ -287,14 +312,14 @@ static int fetch_impl(UniMem *u, const char *who, const void *const host_src[4],
 extern "C" int mole_unimem_fetch(void *handle, const void *const host_src[4], int view_base, int base, int n,
                                  int prefetched, void **slot_ptrs_out) {
     UM(handle);
-    return fetch_impl(u, "mole_unimem_fetch", host_src, view_base, nullptr, base, n, prefetched, slot_ptrs_out);
+    return fetch_impl(u, "mole_unimem_fetch", host_src, view_base, nullptr, base, n, prefetched, 0, slot_ptrs_out);
 }
 
 extern "C" int mole_unimem_fetch_ids(void *handle, const void *const host_src[4], int view_base, const int32_t *expert_ids,
-                                     int n, int prefetched, void **slot_ptrs_out) {
+                                     int n, int prefetched, uint64_t tag, void **slot_ptrs_out) {
     UM(handle);
     MOLE_REQUIRE(expert_ids != nullptr, "mole_unimem_fetch_ids: null expert list");
-    return fetch_impl(u, "mole_unimem_fetch_ids", host_src, view_base, expert_ids, 0, n, prefetched, slot_ptrs_out);
+    return fetch_impl(u, "mole_unimem_fetch_ids", host_src, view_base, expert_ids, 0, n, prefetched, tag, slot_ptrs_out);
 }
 
 extern "C" int mole_unimem_wait_params(void *handle, mole_stream_t compute_stream) {
@@ -497,6 +522,13 @@ extern "C" int mole_unimem_writeback_stats(void *handle, uint64_t *bytes, float 
 extern "C" int mole_unimem_tran_stream(void *handle, mole_stream_t *out) {
     UM(handle);
     *out = (mole_stream_t)u->tran;
+    return 0;
+}
+
+extern "C" int mole_unimem_reuse_stats(void *handle, uint64_t *bytes) {
+    UM(handle);
+    if (bytes) *bytes = u->bytes_reused;
+    u->bytes_reused = 0;
     return 0;
 }
 

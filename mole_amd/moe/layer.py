@@ -14,7 +14,9 @@ New, optional keyword arguments (all defaulting to the reference's behaviour): d
 normalize_gate, gelu_bwd ("tanh" = the derivative the reference compiles, MOLE/cpp/define.hpp:6;
 "exact" = erf derivative), gate_logit_bias, reference_layout, activated_only (offloaded experts that
 received no token are neither copied to the pool nor launched; False restores the reference's
-every-expert-in-index-order behaviour).
+every-expert-in-index-order behaviour), resident (experts that a forward pass brought into the pool are
+not fetched again for its backward pass while they are still there; with a pool large enough for all
+offloaded experts of all layers every expert keeps a slot of its own).
 """
 import time
 
@@ -104,7 +106,7 @@ class MOLEModule(torch.nn.Module):
                  acc_step, adv_adam, use_pool, pool_for_extra=[False, False, False], overlap=True,
                  gate_control_by_umoe=True, hybrid_adam=False, device_s_experts=-1, dtype=torch.float32,
                  normalize_gate=True, gelu_bwd="tanh", gate_logit_bias=None, reference_layout=False,
-                 activated_only=True):
+                 activated_only=True, resident=True):
         super().__init__()
         if not torch.cuda.is_available():
             raise RuntimeError("MOLEModule needs an MI355X: the expert path exists only as HIP kernels")
@@ -128,7 +130,7 @@ class MOLEModule(torch.nn.Module):
                                  total_s_experts // self.world_size, total_d_experts // self.world_size, ebatch_size,
                                  dist["world_size"], act, adv_adam, acc_step, 0, dist["local_rank"],
                                  len(MOLEModule._instance), total_d_experts + total_s_experts, gelu_bwd=gelu_bwd,
-                                 activated_only=activated_only)
+                                 activated_only=activated_only, resident=resident)
 
         # only EP = DP; on one GPU every expert is local
         self.d_experts = total_d_experts // self.world_size

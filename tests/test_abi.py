@@ -95,8 +95,8 @@ def test_every_entry_point_rejects_bad_arguments_on_the_host():
         ("mole_adam_step", lambda: lib.mole_adam_step(ok, ok, ok, ok, ok, 64, L.MOLE_F32, 1.0, 0.999, 1, 1e-3, 0.0, 1e-8, 0, None)),
         ("mole_unimem_prefetch", lambda: lib.mole_unimem_prefetch(None, 0, None, 0, 1)),
         ("mole_unimem_fetch", lambda: lib.mole_unimem_fetch(None, None, 0, 0, 1, 0, None)),
-        ("mole_unimem_prefetch_ids", lambda: lib.mole_unimem_prefetch_ids(None, 0, None, None, 1)),
-        ("mole_unimem_fetch_ids", lambda: lib.mole_unimem_fetch_ids(None, None, 0, None, 1, 0, None)),
+        ("mole_unimem_prefetch_ids", lambda: lib.mole_unimem_prefetch_ids(None, 0, None, None, 1, 0)),
+        ("mole_unimem_fetch_ids", lambda: lib.mole_unimem_fetch_ids(None, None, 0, None, 1, 0, 0, None)),
         ("mole_unimem_wait_slots", lambda: lib.mole_unimem_wait_slots(None, 0, 1, None)),
         ("mole_unimem_reserve", lambda: lib.mole_unimem_reserve(None, 0, 1, None)),
         ("mole_unimem_store_grads_ids", lambda: lib.mole_unimem_store_grads_ids(None, None, None, None, 1, None)),

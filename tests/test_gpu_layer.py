@@ -163,10 +163,11 @@ def test_layer_activated_only_skips_experts_without_rows(unified, dtype):
         yb.backward(torch.ones_like(yb) * 1e-2)
         torch.cuda.synchronize(); core.synchronize_tran()
         assert all(float(m.FC1_W_CPU.all_tensors.grad_[e].abs().max()) > 0 for e in range(E))
-        um.copy_stats()
+        um.copy_stats(); um.reuse_stats()
         m.gate[0].linear.weight.grad = None
         res = _run_and_compare(m, x, ref, k, 0.0, dtype)
         nbytes, _ = um.copy_stats()
+        nbytes += um.reuse_stats()          # what a backward pass found still in place from its forward pass
         return m, res, nbytes, _grads(m, E)
 
     m, res, nbytes, grads = run(True)
@@ -430,12 +431,12 @@ def test_layer_state_round_trip():
     assert m2.MOLECore.hybrid_adam_count == 3
 
 
-def _stack(n_layers, S, M, E, k, Fd, dtype, pool, ebatch, seed):
+def _stack(n_layers, S, M, E, k, Fd, dtype, pool, ebatch, seed, **kw):
     from mole_amd.moe.layer import MOLEModule
     MOLEModule.reset_instances()
     torch.manual_seed(seed)
     dist = {"local_rank": 0, "world_size": 1, "rank": 0}
-    return [MOLEModule(E, 0, M, Fd, pool, k, ebatch, dist, "gelu", 1, False, True, dtype=dtype) for _ in range(n_layers)]
+    return [MOLEModule(E, 0, M, Fd, pool, k, ebatch, dist, "gelu", 1, False, True, dtype=dtype, **kw) for _ in range(n_layers)]
 
 
 def _run_stack(layers, x, prefetch):
@@ -479,3 +480,43 @@ def test_stack_with_planned_prefetch_matches_plain_run(global_prefetch):
         assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
         for a, b in zip(got[2], want[2]):
             assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_resident_experts_halve_the_traffic_and_follow_weight_updates(dtype):
+    """Three offloaded layers and a pool with a slot for every expert: each layer keeps its own stretch of slots,
+    the backward pass finds the experts where the forward pass left them (half the host-to-device bytes of a
+    step), and the results equal, bit for bit, those of a stack that fetches for every pass.  Host weights changed
+    between two passes are picked up: a pass never trusts what an earlier pass left behind."""
+    from mole_amd import core
+    S, M, E, k, Fd = 150, 64, 4, 2, 128
+    es = 4 if dtype == torch.float32 else 2
+    expert_bytes = (2 * Fd * M + Fd + M) * es
+    x = torch.randn(S, M, generator=torch.Generator().manual_seed(5)).to(dtype).cuda()
+    print(f"resident experts {dtype}", flush=True)
+    layers = _stack(3, S, M, E, k, Fd, dtype, pool=12, ebatch=3, seed=21, resident=False)
+    want = _run_stack(layers, x, prefetch=False)
+    layers = _stack(3, S, M, E, k, Fd, dtype, pool=12, ebatch=3, seed=21)
+    assert [m.MOLECore._home_base() for m in layers] == [0, 4, 8]
+    for m in layers:
+        m.set_prefetch(E, E)
+    um = core.get_UniMem()
+    for rep in range(2):
+        um.copy_stats(); um.reuse_stats()
+        got = _run_stack(layers, x, prefetch=bool(rep))
+        nbytes, _ = um.copy_stats()
+        active = sum(int((m.last_route.kept_rows > 0).sum()) for m in layers)
+        assert nbytes == active * expert_bytes
+        # every request for an expert that is already in place counts: without prefetch that is the backward pass's
+        # request alone, with prefetch the passes' own requests find what their prefetches brought as well
+        reused = um.reuse_stats()
+        assert reused == active * expert_bytes * (3 if rep else 1)
+        assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+        for a, b in zip(got[2], want[2]):
+            assert torch.equal(a, b)
+    # new host weights between two forward passes without a backward pass in between
+    y_before = layers[0](x, capacity_factor=0.0).detach().clone()
+    layers[0].FC2_W_CPU.all_tensors.mul_(2.0)
+    layers[0].FC2_B_CPU.all_tensors.mul_(2.0)
+    y_after = layers[0](x, capacity_factor=0.0).detach()
+    assert rel_err(y_after, 2.0 * y_before.float()) < (1e-5 if dtype == torch.float32 else 2e-2)

@@ -4,7 +4,9 @@ top-2, no capacity drop.  One layer is built once for the whole file (15 GB of p
 gradients) and checked for
   * parity of y, dx, dWg and of every expert's four host-side gradients with fp32 torch products of the same
     rounded operands (autograd over a dense restatement of the layer on the GPU; the CPU oracle would take minutes),
-  * bit-identical results with and without prefetch, and copies that cover at least 0.8 of the prefetched step,
+  * bit-identical results with and without prefetch and with and without keeping the forward's experts resident
+    for the backward; copies that cover at least 0.8 of the prefetched step when every pass fetches (the
+    reference's traffic), and half the host-to-device bytes when the experts stay resident,
   * pool slots byte-equal to their pinned host source,
   * activated-only traffic: with a handful of tokens the pool's byte counter equals the activated experts' bytes,
     and the results equal those of a run that copies and launches every expert, bit for bit."""
@@ -75,6 +77,7 @@ def _step(m, x, dy, prefetch):
     torch.cuda.synchronize(); core.synchronize_tran()
     wall = time.perf_counter() - t0
     nbytes, busy_ms = um.copy_stats()
+    _step.reused = um.reuse_stats()
     grads = [p.all_tensors.grad_.cuda() for p in (m.FC1_W_CPU, m.FC1_B_CPU, m.FC2_W_CPU, m.FC2_B_CPU)]
     assert um.virtual_offset() == 0 and um.view_pool_size() == POOL
     return y.detach(), xin.grad, m.gate[0].linear.weight.grad.clone(), grads, wall, nbytes, busy_ms
@@ -99,24 +102,41 @@ def test_c4_layer_parity_prefetch_and_overlap(layer):
     from mole_amd import core
     x, dy = _tokens(S, 1)
     print("c4: step without prefetch", flush=True)
+    assert m.MOLECore.resident and m.MOLECore._home_base() == 0    # the pool holds the layer: experts keep their slots
     y0, dx0, dwg0, g0, _, nbytes0, _ = _step(m, x, dy, prefetch=False)
     r = m.last_route
     loads = r.kept_rows.cpu()
     assert int(loads.sum()) == S * K and int(loads.min()) > 0      # no drop; at this token count every expert is hit
-    assert nbytes0 == 2 * E * EXPERT_BYTES                          # weights travel once forward, once backward
+    # the weights travel once, for the forward; the backward finds them where the forward left them
+    assert nbytes0 == E * EXPERT_BYTES and _step.reused == E * EXPERT_BYTES
 
-    print("c4: step with prefetch", flush=True)
+    def same(res):
+        assert torch.equal(res[0], y0) and torch.equal(res[1], dx0) and torch.equal(res[2], dwg0)
+        for a, b in zip(res[3], g0):
+            assert torch.equal(a, b)
+
+    print("c4: step with prefetch, experts resident from forward to backward", flush=True)
     m.set_prefetch(E, E)
-    y1, dx1, dwg1, g1, wall, nbytes1, busy_ms = _step(m, x, dy, prefetch=True)
-    assert nbytes1 == nbytes0
-    assert torch.equal(y1, y0) and torch.equal(dx1, dx0) and torch.equal(dwg1, dwg0)
-    for a, b in zip(g1, g0):
-        assert torch.equal(a, b)
+    res = _step(m, x, dy, prefetch=True)
+    same(res)
+    assert res[5] == E * EXPERT_BYTES
+    print(f"c4: resident step {res[4] * 1e3:.1f} ms, {res[5] / 1e9:.2f} GB host to device", flush=True)
+
+    print("c4: step with prefetch, every pass fetches its experts (the reference's traffic)", flush=True)
+    m.MOLECore.resident = False
+    try:
+        _step(m, x, dy, prefetch=False)          # leaves the activated set as the prediction for the prefetch
+        res = _step(m, x, dy, prefetch=True)
+    finally:
+        m.MOLECore.resident = True
+    same(res)
+    wall, nbytes1, busy_ms = res[4], res[5], res[6]
+    assert nbytes1 == 2 * E * EXPERT_BYTES and _step.reused == 0
     frac = busy_ms * 1e-3 / wall
     print(f"c4: prefetched step {wall * 1e3:.1f} ms, copy stream busy {busy_ms:.1f} ms ({frac:.2f}), "
           f"{nbytes1 / (busy_ms * 1e-3) / 1e9:.1f} GB/s host to device", flush=True)
     assert frac >= 0.8
-    del g1, y1, dx1, dwg1
+    del res
 
     print("c4: fp32 restatement on the GPU", flush=True)
     idx = r.idx.long()
@@ -172,7 +192,7 @@ def test_c4_layer_copies_only_activated_experts(layer):
     n_act = int((loads > 0).sum())
     print(f"c4: {n_act} of {E} experts activated, {nbytes_a / 1e9:.2f} GB copied", flush=True)
     assert 0 < n_act < E - 4
-    assert nbytes_a == 2 * n_act * EXPERT_BYTES
+    assert nbytes_a == n_act * EXPERT_BYTES and _step.reused == n_act * EXPERT_BYTES    # forward copies, backward reuses
     for e in range(E):
         if int(loads[e]) == 0:
             assert all(float(g[e].float().abs().max()) == 0.0 for g in ga)
@@ -182,7 +202,7 @@ def test_c4_layer_copies_only_activated_experts(layer):
         yd, dxd, dwgd, gd, _, nbytes_d, _ = _step(m, x, dy, prefetch=False)
     finally:
         m.MOLECore.activated_only = True
-    assert nbytes_d == 2 * E * EXPERT_BYTES
+    assert nbytes_d + _step.reused == 2 * E * EXPERT_BYTES
     assert torch.equal(ya, yd) and torch.equal(dxa, dxd) and torch.equal(dwga, dwgd)
     for a, b in zip(ga, gd):
         assert torch.equal(a, b)
