@@ -94,35 +94,55 @@ __device__ __forceinline__ uint32_t lds_offset_of(const char *p) {
 // iteration) to erf(x / sqrt 2) and to the odd parts of the two GELU derivatives.  Beyond the clamp the
 // functions are constant to within the stated error.  Absolute errors in fp32 Horner evaluation:
 // erf 5.8e-5, derivatives 1.8e-4 - an order of magnitude below the bf16 rounding of the result.
-template <int N> __device__ __forceinline__ float odd_poly(float x, float inv_c, const float (&c)[N]) {
-    const float v = __builtin_amdgcn_fmed3f(x * inv_c, -1.0f, 1.0f);
-    const float t = v * v;
-    float q = c[N - 1];
-#pragma unroll
-    for (int k = N - 2; k >= 0; --k) q = fmaf(q, t, c[k]);
-    return v * q;
-}
-// gelu(x) = x/2 (1 + erf(x / sqrt 2))
+// gelu(x) = x (1/2 + 1/2 erf(x / sqrt 2)).  The fit of erf(x / sqrt 2) is v q(v^2) in v = clamp(x / 4, -1, 1); with every
+// coefficient scaled by a power of two (c_k / (8 * 16^k): exact in binary floating point, the Horner steps round as
+// before) the same polynomial is evaluated in v = clamp(x, -4, 4) itself and delivers 1/2 erf directly:
+// clamp, square, eight FMAs, one FMA for the 1/2 and the product with x - twelve instructions, no scaling of x, no
+// separate x / 2.  Beyond the clamp erf is +-1 to within the fit's error, so x (1/2 +- 1/2) is x or 0 as it should be.
 __device__ __forceinline__ float fast_gelu_erf(float x) {
-    constexpr float c[9] = {3.19138169f, -8.50055408f, 20.229044f, -37.1561737f, 51.8556824f,
-                            -52.8050575f, 36.4542885f, -15.039053f, 2.77038407f};
-    const float hx = 0.5f * x;
-    return fmaf(hx, odd_poly(x, 0.25f, c), hx);
+    constexpr float c[9] = {3.19138169f / 8.0f,
+                            -8.50055408f / (8.0f * 16.0f),
+                            20.229044f / (8.0f * 256.0f),
+                            -37.1561737f / (8.0f * 4096.0f),
+                            51.8556824f / (8.0f * 65536.0f),
+                            -52.8050575f / (8.0f * 1048576.0f),
+                            36.4542885f / (8.0f * 16777216.0f),
+                            -15.039053f / (8.0f * 268435456.0f),
+                            2.77038407f / (8.0f * 4294967296.0f)};
+    const float v = __builtin_amdgcn_fmed3f(x, -4.0f, 4.0f);
+    const float t = v * v;
+    float q = c[8];
+#pragma unroll
+    for (int k = 7; k >= 0; --k) q = fmaf(q, t, c[k]);
+    return x * fmaf(v, q, 0.5f);
 }
 // The two GELU derivatives share the clamp (4.5) and the degree, so the variant is a choice of coefficients,
 // made once per tile, not a branch per element: tanh form = what the reference's backward multiplies by
-// (MOLE/cpp/gelu.cu:3-14), exact form = Phi(x) + x phi(x).
+// (MOLE/cpp/gelu.cu:3-14), exact form = Phi(x) + x phi(x).  d(x) = 1/2 + v q(v^2), v = clamp(x / 4.5, -1, 1); as above
+// the polynomial is evaluated in v = clamp(x, -4.5, 4.5) with the coefficients divided by 4.5^(2k+1) (in double
+// precision, then rounded once: 4.5 is not a power of two).
 struct DGeluCoef {
     float c[10];
     __device__ __forceinline__ void select(bool tanh_form) {
-        constexpr float ct[10] = {3.58895016f, -24.237009f, 110.279869f, -345.395355f, 772.538513f,
-                                  -1226.4845f, 1338.11902f, -946.521179f, 388.703674f, -70.0920258f};
-        constexpr float ce[10] = {3.58931732f, -24.1413288f, 108.150215f, -329.418243f, 711.674683f,
-                                  -1091.27979f, 1154.8053f, -796.700195f, 320.776367f, -56.9563408f};
+        constexpr double ct[10] = {3.58895016, -24.237009, 110.279869, -345.395355, 772.538513,
+                                   -1226.4845, 1338.11902, -946.521179, 388.703674, -70.0920258};
+        constexpr double ce[10] = {3.58931732, -24.1413288, 108.150215, -329.418243, 711.674683,
+                                   -1091.27979, 1154.8053, -796.700195, 320.776367, -56.9563408};
+        double s = 1.0 / 4.5;
 #pragma unroll
-        for (int i = 0; i < 10; ++i) c[i] = tanh_form ? ct[i] : ce[i];
+        for (int i = 0; i < 10; ++i) {
+            c[i] = (float)((tanh_form ? ct[i] : ce[i]) * s);
+            s *= 1.0 / (4.5 * 4.5);
+        }
     }
-    __device__ __forceinline__ float operator()(float x) const { return 0.5f + odd_poly(x, 1.0f / 4.5f, c); }
+    __device__ __forceinline__ float operator()(float x) const {
+        const float v = __builtin_amdgcn_fmed3f(x, -4.5f, 4.5f);
+        const float t = v * v;
+        float q = c[9];
+#pragma unroll
+        for (int k = 8; k >= 0; --k) q = fmaf(q, t, c[k]);
+        return fmaf(v, q, 0.5f);
+    }
 };
 
 // ---- operand tiles in LDS -------------------------------------------------------------------------
@@ -705,12 +725,23 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
         // contiguous ranges: the (expert, m-tile) units are dealt round-robin over the 8 XCDs, which gives
         // every XCD the same share of every expert; the n-tiles of a unit stay together (they share the
         // m-side operand in that XCD's L2).
+        // With hundreds of experts of similar size that spread is not needed, and it costs traffic: the m-tiles of
+        // an expert on different XCDs each fetch the expert's rows of the n-side operand into their own L2 (3x the
+        // operands' bytes at 256 experts, which made the launch HBM-bound).  Then (wg_expert_major) the experts are
+        // dealt round-robin instead, all blocks of one expert on one XCD.
         const int m_tiles = (g.M + Q_BM - 1) / Q_BM;
         const int slot = blockIdx.x >> 3;
-        const int unit = (slot / n_tiles) * 8 + (blockIdx.x & 7);
-        if (unit >= g.E * m_tiles) return;
-        e = unit / m_tiles;
-        mt = unit % m_tiles;
+        if (g.wg_expert_major) {
+            const int u = slot / n_tiles;
+            e = (u / m_tiles) * 8 + (blockIdx.x & 7);
+            mt = u % m_tiles;
+            if (e >= g.E) return;
+        } else {
+            const int unit = (slot / n_tiles) * 8 + (blockIdx.x & 7);
+            if (unit >= g.E * m_tiles) return;
+            e = unit / m_tiles;
+            mt = unit % m_tiles;
+        }
         nt = slot % n_tiles;
         // Blocks that also sum an operand run an eighth longer.  Consecutive slots of an XCD go to its four
         // shader engines in turn and are handed out in order, so an engine that always gets the long blocks
@@ -825,8 +856,13 @@ static int dispatch256(const GemmArgs &g, bool b_ks, bool wg, int epi, int max_r
     const int n_tiles = ceil_div(g.N, Q_BN);
     if constexpr (TMB != 10) {
         if (wg) {
-            const int tiles = 8 * ceil_div(g.E * ceil_div(g.M, BM), 8) * n_tiles;   // whole (expert, m-tile) units per XCD
-            if (epi == EPI_WGRAD) return launch256<TMB, WM, true, true, EPI_WGRAD>(g, tiles, st, kid);
+            static const int emajor_from = [] { const char *v = getenv("MOLE_WG_EMAJOR"); return v ? atoi(v) : 128; }();
+            GemmArgs gw = g;
+            gw.wg_expert_major = g.E >= emajor_from;
+            // whole (expert, m-tile) units per XCD, or whole experts
+            const int tiles = gw.wg_expert_major ? 8 * ceil_div(g.E, 8) * ceil_div(g.M, BM) * n_tiles
+                                                 : 8 * ceil_div(g.E * ceil_div(g.M, BM), 8) * n_tiles;
+            if (epi == EPI_WGRAD) return launch256<TMB, WM, true, true, EPI_WGRAD>(gw, tiles, st, kid);
             return -100;
         }
     }
