@@ -382,10 +382,24 @@ def run_probes(args):
     kept = torch.full((E,), rows, dtype=torch.int32, device=dev)
     off = torch.arange(E + 1, dtype=torch.int32, device=dev) * rows
     gflop = 2.0 * S * M * F
-    t = timed(lambda: L.check(L.lib().mole_probe_kloop(L.ptr(xd), L.ptr(w1), L.ptr(off), L.ptr(kept), E, S, F, M, L.ptr(sink),
-                                                       L.stream()), "mole_probe_kloop"), 20)
-    cnt, ms = t["probe"]
-    res["k_loop_without_epilogue"] = {"avg_us": round(ms / cnt * 1e3, 1), "tflops": round(gflop / (ms / cnt * 1e-3) / 1e12, 1)}
+    # The K loop of the first product without its epilogue, whole and with one ingredient taken out, on random and on
+    # zero operands.  The variants without the operand loads multiply whatever the launch before them left in LDS,
+    # which is why each follows a whole loop on the same data.  Same instruction stream and (with loads) the same
+    # memory traffic on both kinds of data: what zero operands gain is what the power limit takes on real data.
+    parts = ((0, "whole"), (1, "without_operand_loads"), (2, "without_fragment_reads"), (3, "without_barriers"),
+             (4, "without_loads_reads_and_barriers"))
+    for kind, (xa, wa) in (("random", (xd, w1)), ("zeros", (torch.zeros_like(xd), torch.zeros_like(w1)))):
+        for part, what in parts:
+            try:
+                t = timed(lambda: L.check(L.lib().mole_probe_kloop_part(L.ptr(xa), L.ptr(wa), L.ptr(off), L.ptr(kept), E, S, F, M,
+                                                                        part, L.ptr(sink), L.stream()), "mole_probe_kloop_part"), 20)
+            except RuntimeError:      # only the default tile shape has the variants (MOLE_TMB selects others)
+                L.kernel_timing_enable(False)
+                continue
+            cnt, ms = t["probe"]
+            res[f"k_loop_{what}_{kind}_operands"] = {"avg_us": round(ms / cnt * 1e3, 1),
+                                                     "tflops": round(gflop / (ms / cnt * 1e-3) / 1e12, 1)}
+    del xa, wa
     t = timed(lambda: H.ffn_fwd(xd, off, kept, w1, b1, w2, b2), 20)
     for kname in ("ffn_fwd1", "ffn_fwd2"):
         cnt, ms = t[kname]

@@ -87,11 +87,15 @@ int mole_kernel_timing_read(int n_ids, int *counts, float *ms_total);
  * show the published peak, random bf16 data what the chip sustains); sink: blocks * 512 floats; *flop_out: flop of
  * the launch.  mole_probe_kloop: the product kernel at the shape of h = xd . w1^T (a [rows,K], b [E,N,K], experts
  * by offsets / kept_rows) with its epilogue left out - prologue, K loop and launch only; sink: 512 floats.
- * Both are timed under MOLE_K_PROBE. */
+ * mole_probe_kloop_part: the same with one ingredient of the K loop taken out, to see what the loop waits for
+ * (part 0: nothing, 1: the loads of the operand tiles into LDS, 2: the fragment reads from LDS, 3: the barriers, 4: all three);
+ * what the accumulators then hold is meaningless.  All are timed under MOLE_K_PROBE. */
 size_t mole_probe_mfma_operand_bytes(void);
 int mole_probe_mfma(const void *operands, int blocks, int iters, float *sink, double *flop_out, mole_stream_t stream);
 int mole_probe_kloop(const void *a, const void *b, const int32_t *offsets, const int32_t *kept_rows, int E,
                      int max_rows, int N, int K, float *sink, mole_stream_t stream);
+int mole_probe_kloop_part(const void *a, const void *b, const int32_t *offsets, const int32_t *kept_rows, int E,
+                          int max_rows, int N, int K, int part, float *sink, mole_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
  * Gate.  Replaces MOLETopk.forward (MOLE/utils/Ugate.py:11-14): scores = softmax(logits).

@@ -30,6 +30,7 @@ _SIGNATURES = {
     "mole_probe_mfma_operand_bytes": (c_size_t, []),
     "mole_probe_mfma": (c_int, [_P, c_int, c_int, _P, POINTER(c_double), _P]),
     "mole_probe_kloop": (c_int, [_P, _P, _P, _P, c_int, c_int, c_int, c_int, _P, _P]),
+    "mole_probe_kloop_part": (c_int, [_P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, _P, _P]),
     "mole_softmax_fwd": (c_int, [_P, _P, c_int, c_int, _P, _P]),
     "mole_gate_fwd": (c_int, [_P, c_int, _P, _P, c_int, c_int, c_int, _P, _P]),
     "mole_softmax_bwd": (c_int, [_P, _P, c_int, c_int, _P, _P]),

@@ -33,7 +33,8 @@ __device__ __forceinline__ float d_gelu_exact(float x) {
 }
 
 enum { EPI_STORE = 0, EPI_BIAS = 1, EPI_BIAS_GELU = 2, EPI_DGELU = 3, EPI_WGRAD = 4, EPI_F32 = 5,
-       EPI_NONE = 6 /* measurement only: the K loop runs, nothing is stored */ };
+       EPI_NONE = 6 /* measurement only: the K loop runs, nothing is stored; EPI_NONE + 1..4: the K loop without
+                       its operand loads / its fragment reads / its barriers / all three */ };
 
 struct GemmArgs {
     const void *A, *B;      // operands (see A_KS / B_KS for their layout)

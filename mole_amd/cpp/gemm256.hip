@@ -324,7 +324,9 @@ template <int TMB, int WM, bool M_KS, bool N_KS, bool WG, int TMC> struct Feeder
 // iteration s+1 the rest, into the buffer that stage s-1 has left.  One synchronisation point per
 // iteration, between the halves: wait until this wave's share of stage s+1 has landed (newer stages may
 // still be in flight), then the barrier.
-template <int TMB, int WM, bool M_KS, bool N_KS, bool WG, int TMC, int TMCW, int SUM>
+// PART (measurement only, results are then meaningless): 1 leaves out the operand loads, 2 the fragment reads of the
+// loop (the first stage's fragments are used throughout), 3 the barriers, 4 all three.
+template <int TMB, int WM, bool M_KS, bool N_KS, bool WG, int TMC, int TMCW, int SUM, int PART = 0>
 __device__ __forceinline__ void main_loop(const bf16_t *Mp, long ldm, int m0, int m_ext, const bf16_t *Np, long ldn,
                                           int n0, int n_ext, int k_ext, char *smem, int wave, int wm, int wn,
                                           f32x16 (&acc)[Tile<TMB, WM>::TMW][2], f32x16 &sums) {
@@ -348,14 +350,18 @@ __device__ __forceinline__ void main_loop(const bf16_t *Mp, long ldm, int m0, in
     // SPLIT: with three or more stages in flight a stage's loads are spread over two halves (one iteration
     // of look-ahead is lost for the later half); with two, all of them go into the half after the barrier.
     constexpr bool SPLIT = AHEAD >= 3;
+    constexpr bool NO_LOADS = PART == 1 || PART == 4, NO_READS = PART == 2 || PART == 4, NO_BARRIERS = PART == 3 || PART == 4;
+    if constexpr (!NO_LOADS) {
 #pragma unroll
-    for (int s = 0; s < AHEAD - 1; ++s) fd.template issue<0, L>(s, s);
-    fd.template issue<0, SPLIT ? LH : L>(AHEAD - 1, AHEAD - 1);
+        for (int s = 0; s < AHEAD - 1; ++s) fd.template issue<0, L>(s, s);
+        fd.template issue<0, SPLIT ? LH : L>(AHEAD - 1, AHEAD - 1);
+    }
     __builtin_amdgcn_s_waitcnt(waitcnt_vm((AHEAD - 2) * L + (SPLIT ? LH : L)));
     __builtin_amdgcn_s_barrier();
     fix_tail(0, 0);
     Frags<TMB, WM, M_KS, N_KS, TMC, TMCW> f0, f1;
     f0.read(smem, wm, wn, 0);
+    if constexpr (NO_READS) f1.read(smem, wm, wn, 1);
     int cur_b = 0;                    // ring buffer of stage s
     for (int s = 0; s < nk; ++s) {
         const int nxt_b = cur_b + 1 == SG::NSTAGE ? 0 : cur_b + 1;
@@ -364,8 +370,8 @@ __device__ __forceinline__ void main_loop(const bf16_t *Mp, long ldm, int m0, in
         const char *cur = smem + cur_b * SG::BYTES;
         const char *nxt = smem + nxt_b * SG::BYTES;
 #define MOLE_HALF(P, J0, N, S_LOAD, BUF, FR, STAGE_PTR, KK, FM)                                           \
-        fd.template issue<(J0) + part_lo<P, NP, (N)>(), (J0) + part_lo<P + 1, NP, (N)>()>(S_LOAD, BUF);   \
-        FR.template read_part<P, NP>(STAGE_PTR, wm, wn, KK);                                                \
+        if constexpr (!NO_LOADS) fd.template issue<(J0) + part_lo<P, NP, (N)>(), (J0) + part_lo<P + 1, NP, (N)>()>(S_LOAD, BUF); \
+        if constexpr (!NO_READS) FR.template read_part<P, NP>(STAGE_PTR, wm, wn, KK);                       \
         FM.template mma_part<P, NP, SUM>(acc, sums, wm, wn);                                              \
         __builtin_amdgcn_sched_barrier(0);
         MOLE_HALF(0, SPLIT ? LH : 0, SPLIT ? L - LH : 0, s + AHEAD - 1, fill_b, f1, cur, 1, f0)
@@ -373,7 +379,7 @@ __device__ __forceinline__ void main_loop(const bf16_t *Mp, long ldm, int m0, in
         MOLE_HALF(2, SPLIT ? LH : 0, SPLIT ? L - LH : 0, s + AHEAD - 1, fill_b, f1, cur, 1, f0)
         MOLE_HALF(3, SPLIT ? LH : 0, SPLIT ? L - LH : 0, s + AHEAD - 1, fill_b, f1, cur, 1, f0)
         __builtin_amdgcn_s_waitcnt(waitcnt_vm((AHEAD - 2) * L));
-        __builtin_amdgcn_s_barrier();
+        if constexpr (!NO_BARRIERS) __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
         fix_tail(s + 1, nxt_b);
         MOLE_HALF(0, 0, SPLIT ? LH : L, s + AHEAD, free_b, f0, nxt, 0, f1)
@@ -492,7 +498,7 @@ __device__ __forceinline__ void epilogue(const GemmArgs &g, f32x16 (&acc)[Tile<T
         }
     };
 
-    if constexpr (EPI == EPI_NONE) {
+    if constexpr (EPI >= EPI_NONE) {
         // the K loop alone (mole_probe_kloop): results leave only under a condition that never holds, which is
         // enough to keep the accumulation alive
         if (g.K < 0) {
@@ -799,7 +805,7 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
     for (int q = 0; q < 16; ++q) sums[q] = 0.f;
 #define MOLE_RUN_TILE_SUM(C, SUM)                                                                                         \
     {                                                                                                                     \
-        main_loop<TMB, WM, M_KS, N_KS, WG, WM *(C), (C), SUM>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wu, wm, wn, acc, sums); \
+        main_loop<TMB, WM, M_KS, N_KS, WG, WM *(C), (C), SUM, (EPI > EPI_NONE ? EPI - EPI_NONE : 0)>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wu, wm, wn, acc, sums); \
         if constexpr (SUM != 0) store_sums<SUM, (C)>(g, sums, e, m0, n0, m_ext, wm, wn, lane);                            \
         epilogue<TMB, WM, WG, EPI, (C)>(g, acc, smem, lane, wu, wn, e, row0, m0w, n0, m_ext, live_w, bias_raw);      \
     }
@@ -879,6 +885,12 @@ static int dispatch256(const GemmArgs &g, bool b_ks, bool wg, int epi, int max_r
             if (epi == EPI_BIAS_GELU) return launch256<TMB, WM, false, false, EPI_BIAS_GELU>(gg, tiles, st, kid);
             if (epi == EPI_F32) return launch256<TMB, WM, false, false, EPI_F32>(gg, tiles, st, kid);
             if (epi == EPI_NONE) return launch256<TMB, WM, false, false, EPI_NONE>(gg, tiles, st, kid);
+            if constexpr (TMB == 8 && WM == 2) {     // the loop's parts are probed at the default tile shape only
+                if (epi == EPI_NONE + 1) return launch256<TMB, WM, false, false, EPI_NONE + 1>(gg, tiles, st, kid);
+                if (epi == EPI_NONE + 2) return launch256<TMB, WM, false, false, EPI_NONE + 2>(gg, tiles, st, kid);
+                if (epi == EPI_NONE + 3) return launch256<TMB, WM, false, false, EPI_NONE + 3>(gg, tiles, st, kid);
+                if (epi == EPI_NONE + 4) return launch256<TMB, WM, false, false, EPI_NONE + 4>(gg, tiles, st, kid);
+            }
         }
     } else {
         if (epi == EPI_BIAS) return launch256<TMB, WM, true, false, EPI_BIAS>(gg, tiles, st, kid);

@@ -68,14 +68,20 @@ extern "C" int mole_probe_mfma(const void *operands, int blocks, int iters, floa
     return 0;
 }
 
-extern "C" int mole_probe_kloop(const void *a, const void *b, const int32_t *offsets, const int32_t *kept_rows, int E,
-                                int max_rows, int N, int K, float *sink, mole_stream_t stream) {
+extern "C" int mole_probe_kloop_part(const void *a, const void *b, const int32_t *offsets, const int32_t *kept_rows, int E,
+                                     int max_rows, int N, int K, int part, float *sink, mole_stream_t stream) {
+    MOLE_REQUIRE(part >= 0 && part <= 4, "mole_probe_kloop_part: part %d is not one of 0..4", part);
     MOLE_REQUIRE(a && b && offsets && kept_rows && sink && E >= 1 && max_rows > 0 && N > 0 && K > 0 && N % 8 == 0 && K % 32 == 0,
                  "mole_probe_kloop: bad arguments (E=%d rows=%d N=%d K=%d)", E, max_rows, N, K);
     GemmArgs g{};
     g.offsets = offsets; g.kept = kept_rows; g.E = E;
     g.A = a; g.lda = K; g.B = b; g.ldb = K; g.strideB = (long)N * K; g.N = N; g.K = K; g.C = sink; g.ldc = N;
-    const int rc = launch_gemm256(g, false, false, false, EPI_NONE, max_rows, (hipStream_t)stream, MOLE_K_PROBE);
+    const int rc = launch_gemm256(g, false, false, false, EPI_NONE + part, max_rows, (hipStream_t)stream, MOLE_K_PROBE);
     MOLE_REQUIRE(rc != -100, "mole_probe_kloop: shape not taken by the 256-wide kernel");
     return rc;
+}
+
+extern "C" int mole_probe_kloop(const void *a, const void *b, const int32_t *offsets, const int32_t *kept_rows, int E,
+                                int max_rows, int N, int K, float *sink, mole_stream_t stream) {
+    return mole_probe_kloop_part(a, b, offsets, kept_rows, E, max_rows, N, K, 0, sink, stream);
 }
