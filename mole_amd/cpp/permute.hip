@@ -281,9 +281,10 @@ __global__ __launch_bounds__(256) void dispatch_bwd_gate_kernel(const T *__restr
 // instructions per pair of output elements on it, which is what bounds it; here the VALU work is the
 // unpack / add / pack of a copy.
 // A block of eight waves covers 1024 columns, a wave 128 columns of 16 tokens at a time: its 8 product tiles go
-// through an 8 KB LDS buffer of its own (the MFMA result has a lane hold one column of four tokens; the
-// row-major side wants 16 bytes of one token per lane), then every lane gathers 8 columns of one token's k
-// source rows, adds and stores 16 bytes.  The first-choice gathers of a group of tokens are issued one group ahead.
+// through an 8 KB LDS buffer of its own (the MFMA result has a lane hold four columns of one token; the
+// row-major side wants eight columns of one token per lane), then every lane gathers 8 columns of one token's k
+// source rows, adds and stores 16 bytes.  The first-choice gathers and the gradients of a group of tokens are issued one
+// group ahead (all four groups' up front was slower: 16.1 against 14.2 us, the weights' loads queue behind them).
 constexpr int DM_TOKENS = 64;                 // tokens per block: four groups of 16 (32: +5 %, 16: +20 % at 16384 x 1024)
 constexpr int DM_COLS = 128;                  // columns per wave
 constexpr int DM_ROW = DM_COLS + 4;           // floats per token row of the LDS buffer: 4 rows apart = 16 banks apart
@@ -322,6 +323,21 @@ __global__ __launch_bounds__(512) void dispatch_bwd_gate_mfma_kernel(const bf16_
     uint4 src[4];
     uint32_t src_ok[4];
     gather(src, src_ok, blockIdx.x * DM_TOKENS);
+    // A fragment of a group of 16 tokens: dlogits[tok0 + r16][8 kq .. 8 kq + 7], fetched one group ahead like the rows
+    // (fetched where it is used, the product waited for it in every group: 15.0 -> 14.2 us at 16384 x 1024)
+    auto load_d = [&](float (&d)[8], int tok0) __attribute__((always_inline)) {
+        if constexpr (E8) {
+            const float4 *dp = reinterpret_cast<const float4 *>(dlogits + (size_t)min(tok0 + r16, S - 1) * E + min(8 * kq, E - 8));
+            const float4 d0 = dp[0], d1 = dp[1];
+            d[0] = d0.x; d[1] = d0.y; d[2] = d0.z; d[3] = d0.w;
+            d[4] = d1.x; d[5] = d1.y; d[6] = d1.z; d[7] = d1.w;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) d[i] = dlogits[(size_t)min(tok0 + r16, S - 1) * E + min(8 * kq + i, E - 1)];
+        }
+    };
+    float d[8];
+    load_d(d, blockIdx.x * DM_TOKENS);
     // B fragments: Wg[8 kq + i][col0 + 16 cb + r16], i = 0..7, for the wave's 8 column blocks.  Fetched row by row
     // with 16-byte loads (a lane takes 4 columns of the 8 experts of one group) and turned by way of the LDS
     // buffer, [expert group][column] with a group's 8 experts as one bf16x8 entry: picking them out of global
@@ -366,29 +382,23 @@ __global__ __launch_bounds__(512) void dispatch_bwd_gate_mfma_kernel(const bf16_
         const int tok0 = blockIdx.x * DM_TOKENS + g0;
         uint4 nxt[4];
         uint32_t nxt_ok[4];
-        if (g0 + 16 < DM_TOKENS) gather(nxt, nxt_ok, tok0 + 16);
-        // A fragment: dlogits[tok0 + r16][8 kq .. 8 kq + 7]
-        float d[8];
-        if constexpr (E8) {
-            const float4 *dp = reinterpret_cast<const float4 *>(dlogits + (size_t)min(tok0 + r16, S - 1) * E + min(8 * kq, E - 8));
-            const float4 d0 = dp[0], d1 = dp[1];
-            d[0] = d0.x; d[1] = d0.y; d[2] = d0.z; d[3] = d0.w;
-            d[4] = d1.x; d[5] = d1.y; d[6] = d1.z; d[7] = d1.w;
-        } else {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) d[i] = dlogits[(size_t)min(tok0 + r16, S - 1) * E + min(8 * kq + i, E - 1)];
+        float d_nxt[8];
+        if (g0 + 16 < DM_TOKENS) {
+            gather(nxt, nxt_ok, tok0 + 16);
+            load_d(d_nxt, tok0 + 16);
         }
 #pragma unroll
         for (int i = 0; i < 8; ++i)
             if (tok0 + r16 >= S || 8 * kq + i >= E) d[i] = 0.f;
         const perm_bf16x8 afrag = {(bf16_t)d[0], (bf16_t)d[1], (bf16_t)d[2], (bf16_t)d[3],
                                    (bf16_t)d[4], (bf16_t)d[5], (bf16_t)d[6], (bf16_t)d[7]};
-        // product tiles into LDS: acc[r] = token 4 kq + r, column 16 cb + r16 (conflict-free: see DM_ROW)
+        // product tiles into LDS.  The gate's weights go into the first operand slot, so the four results of a lane
+        // are four consecutive columns of one token (acc[r] = column 16 cb + 4 kq + r of token r16) and leave with
+        // one 16-byte LDS write (a quarter wave's 16 rows are 16 banks-of-four apart: see DM_ROW)
 #pragma unroll
         for (int cb = 0; cb < 8; ++cb) {
-            const perm_f32x4 acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(afrag, bfrag[cb], perm_f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-#pragma unroll
-            for (int r = 0; r < 4; ++r) buf[(4 * kq + r) * DM_ROW + 16 * cb + r16] = acc[r];
+            const perm_f32x4 acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bfrag[cb], afrag, perm_f32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+            *reinterpret_cast<perm_f32x4 *>(buf + r16 * DM_ROW + 16 * cb + 4 * kq) = acc;
         }
         // (a wave's LDS buffer is written and read by that wave only: program order is enough)
 #pragma unroll
@@ -421,6 +431,8 @@ __global__ __launch_bounds__(512) void dispatch_bwd_gate_mfma_kernel(const bf16_
         if (g0 + 16 < DM_TOKENS) {
 #pragma unroll
             for (int u = 0; u < 4; ++u) { src[u] = nxt[u]; src_ok[u] = nxt_ok[u]; }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) d[i] = d_nxt[i];
         }
     }
 }
