@@ -263,8 +263,10 @@ def measure_layer(name, steps, warmup, with_adam=True):
     work = {  # algorithmic work per launch: flop for the GEMMs, bytes for the permutes
         "ffn_fwd1": gemm_flop, "ffn_fwd2": gemm_flop, "ffn_gw2": gemm_flop, "ffn_da": gemm_flop, "ffn_gw1": gemm_flop,
         "ffn_gx": gemm_flop,
-        # the combine backward is one fused kernel (d_o scatter and the gate dot products read dy and o once)
-        "dispatch_fwd": 2.0 * R * M * b, "combine_fwd": (R + S) * M * b, "combine_bwd": (S + 2.0 * R) * M * b,
+        # the combine backward is one fused kernel (d_o scatter and the gate dot products read dy and o once); the
+        # dispatch reads a token's row once and writes it to each of its kept pairs' rows (with one choice per token
+        # that is the 2 R rows of a read and a write per kept row; with more it is S + R, not 2 R)
+        "dispatch_fwd": (min(S, R) + R) * M * b, "combine_fwd": (R + S) * M * b, "combine_bwd": (S + 2.0 * R) * M * b,
         "dispatch_bwd": (R + S) * M * b,
     }
     kernels = {}
