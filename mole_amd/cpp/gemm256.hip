@@ -444,10 +444,7 @@ __device__ __forceinline__ void epilogue(const GemmArgs &g, f32x16 (&acc)[Tile<T
     auto slab_at = [&](int row, int chunk, int half) -> char * {
         return slab + row * 128 + ((chunk ^ ((row >> 1) & 7)) << 4) + ((half ^ (row >> 4)) & 1) * 8;
     };
-    // a 16-byte access sees the two halves of a chunk swapped on rows with bit 4 set
-    auto fix16 = [&](uint4 v, int row) -> uint4 {
-        return (row & 16) ? make_uint4(v.z, v.w, v.x, v.y) : v;
-    };
+    // (a 16-byte access sees the two halves of a chunk swapped on rows with bit 4 set)
     // slab -> global: rows [0, live) of the slab, 128 bytes each
     // The large results - h, a, t and the weight gradients, 134-270 MB a launch, which no block of the same
     // launch reads - leave with non-temporal stores: ordinary stores let them push the operand panels of the
@@ -457,16 +454,48 @@ __device__ __forceinline__ void epilogue(const GemmArgs &g, f32x16 (&acc)[Tile<T
     // and take them from HBM at no loss.  The small results (out, gx: 34 MB) stay ordinary: the row permutes
     // that read them next are memory-bound and lost more than the products gained.
     constexpr bool STREAM_OUT = EPI == EPI_BIAS_GELU || EPI == EPI_DGELU || EPI == EPI_WGRAD;
+    // Addresses of the wide accesses: a wave-uniform 64-bit base (the slab's first row in the result, advanced by
+    // scalar adds from row group to row group) plus a 32-bit per-lane byte offset that is computed once, so a store
+    // costs no address arithmetic on the vector ALU; and the LDS reads of a batch of eight row groups are issued
+    // before the first store, so that one LDS latency is waited for per batch instead of one per store.  (Written
+    // row by row with the row test around the read and the store, each store waited for its own LDS read and
+    // recomputed a 64-bit row * pitch product: two thirds of the epilogue's time apart from the activation.)
+    const uint32_t pitch = (uint32_t)g.ldc * 2;                          // bytes between rows of the result
+    const uint32_t lane_off = (uint32_t)jr * pitch + (uint32_t)jc * 16;  // this lane's 16 bytes of row jr
+    // every row group and every column is stored (the same in all lanes)
+    const bool full = __builtin_amdgcn_readfirstlane(live >= TMC * 32 && nw0 + 64 <= g.N) != 0;
+    // LDS address of this lane's 16 bytes of row group `it` (rows 8 it + jr): with row = 8 it + jr the swizzle term
+    // (row >> 1) & 7 is (jr >> 1) | ((it & 1) << 2), so two per-lane bases and a constant per row group suffice
+    char *const wide0 = slab + jr * 128 + ((jc ^ (jr >> 1)) << 4);
+    char *const wide1 = slab + jr * 128 + ((jc ^ (jr >> 1) ^ 4) << 4);
+    auto wide_cell = [&](int it) -> char * { return ((it & 1) ? wide1 : wide0) + it * 1024; };
+    auto fix_it = [&](uint4 v, int it) -> uint4 {      // rows with bit 4 set (it & 2) hold their halves swapped
+        return (it & 2) ? make_uint4(v.z, v.w, v.x, v.y) : v;
+    };
+    typedef __attribute__((address_space(1))) char gchar;
     auto flush = [&](bf16_t *dst) __attribute__((always_inline)) {
         typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+        gchar *gbase = (gchar *)((char *)dst + ((crow0 + m0) * g.ldc + nw0) * 2);
 #pragma unroll
-        for (int it = 0; it < TMC * 4; ++it) {
-            const int row = it * 8 + jr;
-            const uint4 v = fix16(*reinterpret_cast<const uint4 *>(slab_at(row, jc, (row >> 4) & 1)), row);
-            if (row < live && col_ok) {
-                uint4 *p = reinterpret_cast<uint4 *>(dst + (crow0 + m0 + row) * g.ldc + nw0 + jc * 8);
-                if constexpr (STREAM_OUT) __builtin_nontemporal_store(u32x4{v.x, v.y, v.z, v.w}, reinterpret_cast<u32x4 *>(p));
-                else *p = v;
+        for (int it0 = 0; it0 < TMC * 4; it0 += 8) {
+            uint4 v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (it0 + i < TMC * 4) v[i] = fix_it(*reinterpret_cast<const uint4 *>(wide_cell(it0 + i)), it0 + i);
+            auto put = [&](int i) __attribute__((always_inline)) {
+                gchar *p = gbase + (size_t)(it0 + i) * 8 * pitch + lane_off;
+                typedef __attribute__((address_space(1))) u32x4 g_u32x4;
+                if constexpr (STREAM_OUT) __builtin_nontemporal_store(u32x4{v[i].x, v[i].y, v[i].z, v[i].w}, reinterpret_cast<g_u32x4 *>(p));
+                else *reinterpret_cast<g_u32x4 *>(p) = u32x4{v[i].x, v[i].y, v[i].z, v[i].w};
+            };
+            if (full) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    if (it0 + i < TMC * 4) put(i);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    if (it0 + i < TMC * 4 && (it0 + i) * 8 + jr < live && col_ok) put(i);
             }
         }
     };
@@ -474,27 +503,29 @@ __device__ __forceinline__ void epilogue(const GemmArgs &g, f32x16 (&acc)[Tile<T
     // into the operand (rows past the end read its last row, columns past the end its first column): what lands
     // in cells outside the live part is never written back, and a load under a condition would make the
     // compiler wait for all loads in flight at each one, so the eight would run one after the other.
-    const long row_last = crow0 + m_ext - 1;
-    const int col_c = col_ok ? nw0 + jc * 8 : 0;
     auto fill = [&](const bf16_t *src) __attribute__((always_inline)) {
+        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+        // rows are counted from the slab's first row, or from the operand's last row when the slab starts past it
+        const long first = min(crow0 + m0, crow0 + m_ext - 1);
+        const uint32_t last_off = (uint32_t)(crow0 + m_ext - 1 - first) * pitch;      // byte offset of the last valid row
+        const gchar *gbase = (const gchar *)((const char *)src + first * g.ldc * 2);
+        const uint32_t col_off = col_ok ? (uint32_t)(nw0 + jc * 8) * 2 : 0u;
+        const uint32_t row_off = (uint32_t)jr * pitch;
 #pragma unroll
         for (int it0 = 0; it0 < TMC * 4; it0 += 8) {
             uint4 v[8];
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 if (it0 + i >= TMC * 4) continue;
-                const long row = crow0 + m0 + (it0 + i) * 8 + jr;
-                {   // read once, here: a non-temporal load keeps it from displacing the K loop's operands (-4 us)
-                    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-                    const u32x4 w = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + (row < row_last ? row : row_last) * g.ldc + col_c));
-                    v[i] = make_uint4(w[0], w[1], w[2], w[3]);
-                }
+                const uint32_t ro = min(row_off + (uint32_t)(it0 + i) * 8 * pitch, last_off);
+                // read once, here: a non-temporal load keeps it from displacing the K loop's operands (-4 us)
+                typedef __attribute__((address_space(1))) u32x4 g_u32x4;
+                const u32x4 w = __builtin_nontemporal_load(reinterpret_cast<const g_u32x4 *>(gbase + ro + col_off));
+                v[i] = make_uint4(w[0], w[1], w[2], w[3]);
             }
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const int row = (it0 + i) * 8 + jr;
-                if (it0 + i < TMC * 4) *reinterpret_cast<uint4 *>(slab_at(row, jc, (row >> 4) & 1)) = fix16(v[i], row);
-            }
+            for (int i = 0; i < 8; ++i)
+                if (it0 + i < TMC * 4) *reinterpret_cast<uint4 *>(wide_cell(it0 + i)) = fix_it(v[i], it0 + i);
         }
     };
 
