@@ -40,7 +40,7 @@ MEASURED_TRAFFIC_BYTES = {
            "ffn_gx": 383.2e6},
     "c3": {"ffn_fwd1": 3816.1e6, "ffn_fwd2": 2214.7e6, "ffn_gw2": 3085.4e6, "ffn_da": 3824.1e6, "ffn_gw1": 3085.4e6,
            "ffn_gx": 2219.6e6},
-    "c5": {"ffn_fwd1": 4371.8e6, "ffn_fwd2": 3329.5e6, "ffn_gw2": 5971.4e6, "ffn_da": 4378.7e6, "ffn_gw1": 5971.4e6,
+    "c5": {"ffn_fwd1": 4371.8e6, "ffn_fwd2": 3329.5e6, "ffn_gw2": 3032.0e6, "ffn_da": 4378.7e6, "ffn_gw1": 3032.0e6,
            "ffn_gx": 3306.4e6},
 }
 PEAK_HBM_BYTES = PEAK_HBM_GBS * 1e9
