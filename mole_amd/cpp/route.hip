@@ -730,6 +730,7 @@ __global__ __launch_bounds__(256) void gate_fwd_kernel(const bf16_t *__restrict_
     constexpr int LPR = RB / 16, RPI = 64 / LPR;                // lanes per row, rows per load instruction
     constexpr int PART_BYTES = 4 * 16 * TG * (EG * 16 + 1) * 4;
     constexpr int STAGE_BYTES = STAGE ? 4 * 16 * TG * RS : 0;
+    static_assert(!STAGE || STAGE_BYTES >= PART_BYTES, "the launch sizes the dynamic LDS for the staged rows");
     __shared__ __align__(16) char s_static[STAGE ? 16 : PART_BYTES];
     extern __shared__ __align__(16) char s_dyn[];               // STAGE: max(PART_BYTES, STAGE_BYTES), given at launch
     char *s_all = STAGE ? s_dyn : s_static;
