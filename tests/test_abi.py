@@ -28,6 +28,33 @@ def test_library_exports_every_declared_symbol():
     assert lib.mole_version() >= 100
 
 
+def test_header_is_plain_c_and_a_c_program_links(tmp_path):
+    """The boundary is a C ABI: the header compiles as strict C99 (no C++ types, no torch types), and a C program
+    that calls an entry point links against the shared library and runs without a GPU."""
+    import shutil
+    import subprocess
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc here")
+    inc = os.path.join(ROOT, "include")
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", "-x", "c",
+                    os.path.join(inc, "mole_hip.h")], check=True)
+    src = tmp_path / "caller.c"
+    src.write_text('#include <stdio.h>\n#include "mole_hip.h"\n'
+                   'int main(void) {\n'
+                   '    /* bad arguments are refused on the host, with a message, before anything touches a GPU */\n'
+                   '    int rc = mole_dispatch_fwd(NULL, MOLE_BF16, NULL, 8, 12, 2, NULL, NULL);\n'
+                   '    printf("%d %d %s\\n", mole_version(), rc, mole_last_error_string());\n'
+                   '    return rc == -1 ? 0 : 1;\n}\n')
+    from mole_amd import _lib as L
+    libdir = os.path.dirname(L.LIB_PATH)
+    exe = tmp_path / "caller"
+    subprocess.run([gcc, "-std=c99", "-I", inc, str(src), "-o", str(exe), "-L", libdir, "-l:" + os.path.basename(L.LIB_PATH),
+                    "-Wl,-rpath," + libdir], check=True)
+    out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split(None, 2)
+    assert int(out[0]) >= 100 and int(out[1]) == -1 and "M" in out[2]
+
+
 def test_argument_validation_needs_no_gpu():
     from mole_amd import _lib as L
     lib = L.lib()
