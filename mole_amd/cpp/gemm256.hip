@@ -748,9 +748,16 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
         m_ext = found < WAVE ? __shfl(rows_lane, found, WAVE) : rows_of(e);
         int mt_class = target - before;
         if (mf) {
+            // groups of G n-tiles, an expert's m-tiles of the class inside a group, the group's n-tiles innermost
+            // (G = 1: m-tile first; the last group may be short)
             const int c_e = cnt_found / n_tiles;      // the expert's m-tiles of this class
-            nt = mt_class / c_e;
-            mt_class = mt_class % c_e;
+            const int G = g.m_fastest;
+            const int n_groups = (n_tiles + G - 1) / G;
+            const int grp = min(mt_class / (c_e * G), n_groups - 1);
+            const int j = mt_class - grp * c_e * G;
+            const int gsz = min(G, n_tiles - grp * G);
+            nt = grp * G + j % gsz;
+            mt_class = j / gsz;
         }
         mt = mt_class + (heavy ? 0 : heavy_of(m_ext));   // an expert's light tiles follow its heavy ones
         const int t_e = (m_ext + Q_BM - 1) / Q_BM;
@@ -906,7 +913,8 @@ static int dispatch256(const GemmArgs &g, bool b_ks, bool wg, int epi, int max_r
     // block slots: the worst-case number of m-tiles (an expert with r rows has ceil(r / BM) of them)
     const int rows_bound = g.offsets ? max_rows : g.single_rows;
     GemmArgs gg = g;
-    gg.m_fastest = (m_fastest_mask() >> kid) & 1;
+    static const int mfast_group = [] { const char *v = getenv("MOLE_MFAST_G"); return v && atoi(v) > 0 ? atoi(v) : 1; }();
+    gg.m_fastest = ((m_fastest_mask() >> kid) & 1) ? mfast_group : 0;
     // (+ 16: the heavy and the light tiles of an XCD are rounded up to whole slots separately)
     const int tiles = (((rows_bound / BM + (g.offsets ? g.E : 1)) * n_tiles + 7) & ~7) + 16;
     if (wg) return -100;
