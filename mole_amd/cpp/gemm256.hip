@@ -507,7 +507,9 @@ __device__ __forceinline__ void epilogue(const GemmArgs &g, f32x16 (&acc)[Tile<T
         typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
         // rows are counted from the slab's first row, or from the operand's last row when the slab starts past it
         const long first = min(crow0 + m0, crow0 + m_ext - 1);
-        const uint32_t last_off = (uint32_t)(crow0 + m_ext - 1 - first) * pitch;      // byte offset of the last valid row
+        // byte offset of the last valid row, as far as the slab reaches (the row count is bounded before it meets the
+        // pitch: an expert of 10^5 rows times a pitch of tens of KB does not fit 32 bits)
+        const uint32_t last_off = (uint32_t)min(crow0 + m_ext - 1 - first, (long)(TMC * 32 - 1)) * pitch;
         const gchar *gbase = (const gchar *)((const char *)src + first * g.ldc * 2);
         const uint32_t col_off = col_ok ? (uint32_t)(nw0 + jc * 8) * 2 : 0u;
         const uint32_t row_off = (uint32_t)jr * pitch;
