@@ -1,5 +1,6 @@
 """Where the reference keeps its native extension.  The C ABI of the MI355X implementation is declared in
-mole_hip.h in this directory and built into mole_amd/cpp/libmole_hip.so; LIB_PATH names the built library."""
+mole_hip.h in this directory (it forwards to include/mole_hip.h), implemented by the HIP sources beside it and built
+into libmole_hip.so in this directory by `python -m mole_amd.build`; LIB_PATH names the built library."""
 import os
 
 from mole_amd._lib import LIB_PATH  # noqa: F401

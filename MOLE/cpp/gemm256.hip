@@ -1,9 +1,9 @@
 // bf16 grouped GEMM for gfx950: the fast path of the six expert-FFN products.
 //
-// A block of 4 waves owns a BM (m) x 256 (n) output tile, BM = 256 or 128; every wave covers all BM
-// rows and 64 columns (BM/32 x 2 MFMA 32x32x16 blocks, fp32 accumulators in AGPRs).  BM = 256 runs
-// one block per CU (256 accumulator registers per lane); BM = 128 runs two, so that one block's
-// epilogue overlaps the other's K loop and ragged experts quantise into finer tiles.
+// A block of 8 waves (2 wave rows x 4 wave columns, two waves per SIMD) owns a BM (m) x 256 (n) output tile, BM =
+// 256 or up to 320; a wave covers BM/2 rows and 64 columns (BM/64 x 2 MFMA 32x32x16 blocks, fp32 accumulators).
+// One block per CU.  (A build with -DMOLE_TUNING also carries the four-wave shapes and launch orders that were
+// measured against this one and lost.)
 // Operand tiles go from HBM/L2 straight into LDS (global_load_lds_dwordx4, no staging registers)
 // through a ring of stages of 32 of K, several stages of loads in flight while one is consumed: with
 // a single stage of look-ahead the loop ran at the memory latency, not at the MFMA rate.  One
@@ -886,15 +886,25 @@ static int launch256(GemmArgs g, int tiles, hipStream_t st, int kid) {
     return 0;
 }
 
-// Which products number their tiles m-tile first (bit = MOLE_K_* id).  MOLE_MFAST in the environment overrides
-// the default (tuning aid).
-static int m_fastest_mask() {
-    static const int mask = [] {
-        const char *v = getenv("MOLE_MFAST");
-        return v ? atoi(v) : 0;
-    }();
-    return mask;
-}
+// Launch options that were measured and are off by default; a -DMOLE_TUNING build reads them from the environment
+// (MOLE_MFAST: bit mask of the products that number an XCD's tiles m-tile first, MOLE_MFAST_G: n-tiles per group of
+// that order, MOLE_WG_EMAJOR: expert count from which a weight gradient keeps an expert's blocks on one XCD,
+// MOLE_TMB: 4 | 8 = four-wave tiles of 128 | 256 rows, 16 = the 256-row eight-wave tile for every product,
+// MOLE_NO_SUMS: bias gradients from their own kernel).
+#ifdef MOLE_TUNING
+static int env_int(const char *name, int dflt) { const char *v = getenv(name); return v ? atoi(v) : dflt; }
+static int m_fastest_mask() { static const int v = env_int("MOLE_MFAST", 0); return v; }
+static int m_fastest_group() { static const int v = env_int("MOLE_MFAST_G", 1); return v > 0 ? v : 1; }
+static int wg_emajor_from() { static const int v = env_int("MOLE_WG_EMAJOR", 128); return v; }
+static int forced_tile() { static const int v = env_int("MOLE_TMB", 0); return v; }
+static bool sums_off() { static const bool v = getenv("MOLE_NO_SUMS") != nullptr; return v; }
+#else
+static int m_fastest_mask() { return 0; }
+static int m_fastest_group() { return 1; }
+static int wg_emajor_from() { return 128; }
+static int forced_tile() { return 0; }
+static bool sums_off() { return false; }
+#endif
 
 template <int TMB, int WM>
 static int dispatch256(const GemmArgs &g, bool b_ks, bool wg, int epi, int max_rows, hipStream_t st, int kid) {
@@ -902,9 +912,8 @@ static int dispatch256(const GemmArgs &g, bool b_ks, bool wg, int epi, int max_r
     const int n_tiles = ceil_div(g.N, Q_BN);
     if constexpr (TMB != 10) {
         if (wg) {
-            static const int emajor_from = [] { const char *v = getenv("MOLE_WG_EMAJOR"); return v ? atoi(v) : 128; }();
             GemmArgs gw = g;
-            gw.wg_expert_major = g.E >= emajor_from;
+            gw.wg_expert_major = g.E >= wg_emajor_from();
             // whole (expert, m-tile) units per XCD, or whole experts
             const int tiles = gw.wg_expert_major ? 8 * ceil_div(g.E, 8) * ceil_div(g.M, BM) * n_tiles
                                                  : 8 * ceil_div(g.E * ceil_div(g.M, BM), 8) * n_tiles;
@@ -915,8 +924,7 @@ static int dispatch256(const GemmArgs &g, bool b_ks, bool wg, int epi, int max_r
     // block slots: the worst-case number of m-tiles (an expert with r rows has ceil(r / BM) of them)
     const int rows_bound = g.offsets ? max_rows : g.single_rows;
     GemmArgs gg = g;
-    static const int mfast_group = [] { const char *v = getenv("MOLE_MFAST_G"); return v && atoi(v) > 0 ? atoi(v) : 1; }();
-    gg.m_fastest = ((m_fastest_mask() >> kid) & 1) ? mfast_group : 0;
+    gg.m_fastest = ((m_fastest_mask() >> kid) & 1) ? m_fastest_group() : 0;
     // (+ 16: the heavy and the light tiles of an XCD are rounded up to whole slots separately)
     const int tiles = (((rows_bound / BM + (g.offsets ? g.E : 1)) * n_tiles + 7) & ~7) + 16;
     if (wg) return -100;
@@ -926,12 +934,14 @@ static int dispatch256(const GemmArgs &g, bool b_ks, bool wg, int epi, int max_r
             if (epi == EPI_BIAS_GELU) return launch256<TMB, WM, false, false, EPI_BIAS_GELU>(gg, tiles, st, kid);
             if (epi == EPI_F32) return launch256<TMB, WM, false, false, EPI_F32>(gg, tiles, st, kid);
             if (epi == EPI_NONE) return launch256<TMB, WM, false, false, EPI_NONE>(gg, tiles, st, kid);
+#ifdef MOLE_TUNING
             if constexpr (TMB == 8 && WM == 2) {     // the loop's parts are probed at the default tile shape only
                 if (epi == EPI_NONE + 1) return launch256<TMB, WM, false, false, EPI_NONE + 1>(gg, tiles, st, kid);
                 if (epi == EPI_NONE + 2) return launch256<TMB, WM, false, false, EPI_NONE + 2>(gg, tiles, st, kid);
                 if (epi == EPI_NONE + 3) return launch256<TMB, WM, false, false, EPI_NONE + 3>(gg, tiles, st, kid);
                 if (epi == EPI_NONE + 4) return launch256<TMB, WM, false, false, EPI_NONE + 4>(gg, tiles, st, kid);
             }
+#endif
         }
     } else {
         if (epi == EPI_BIAS) return launch256<TMB, WM, true, false, EPI_BIAS>(gg, tiles, st, kid);
@@ -947,13 +957,9 @@ static int dispatch256(const GemmArgs &g, bool b_ks, bool wg, int epi, int max_r
 // average one, so the launch stays one round.  The K = M products run four rounds anyway; their short
 // remainder tiles, numbered last, fill the final round, which measured better than the even split
 // (t = (go.w2^T) gelu'(h): 213 against 219 us) - and h = xd.w1^T + b1 with the GELU epilogue would spill at
-// the 160 accumulators of the larger tile.  MOLE_TMB=4|8 in the environment selects the four-wave variants
-// with 128 or 256 rows, 16 the 256-row eight-wave tile for everything (tuning aid).
+// the 160 accumulators of the larger tile.
 static int tile_blocks_for(int kid) {
-    static const int forced = [] {
-        const char *v = getenv("MOLE_TMB");
-        return v ? atoi(v) : 0;
-    }();
+    const int forced = forced_tile();
     if (forced == 4 || forced == 8 || forced == 16) return forced;
     return (kid == MOLE_K_FFN_FWD2 || kid == MOLE_K_FFN_GX) ? 20 : 16;
 }
@@ -963,8 +969,7 @@ static int tile_blocks_for(int kid) {
 bool gemm256_sums_operand(const GemmArgs &g, int kid) {
     if (g.lda % 8 || g.ldb % 8 || g.ldc % 8 || g.N % 8 || g.M % 8) return false;
     const int tmb = tile_blocks_for(kid);
-    static const bool off = getenv("MOLE_NO_SUMS") != nullptr;   // tuning aid: bias gradients from their own kernel
-    if (off) return false;
+    if (sums_off()) return false;
     return tmb == 16 || tmb == 20;
 }
 
@@ -974,11 +979,12 @@ int launch_gemm256(const GemmArgs &g, bool a_ks, bool b_ks, bool wg, int epi, in
     if (!wg && (a_ks || g.K % Q_BK)) return -100;
     if (wg && (!a_ks || !b_ks || g.M % 8)) return -100;
     const int tmb = tile_blocks_for(kid);
+#ifdef MOLE_TUNING
     if (tmb == 4) return dispatch256<4, 1>(g, b_ks, wg, epi, max_rows, st, kid);
-    if (tmb == 16) return dispatch256<8, 2>(g, b_ks, wg, epi, max_rows, st, kid);   // 256 rows, eight waves
+    if (tmb == 8) return dispatch256<8, 1>(g, b_ks, wg, epi, max_rows, st, kid);
+#endif
     if (tmb == 20 && !wg && b_ks) return dispatch256<10, 2>(g, b_ks, wg, epi, max_rows, st, kid);   // up to 320 rows, eight waves
-    if (tmb == 20) return dispatch256<8, 2>(g, b_ks, wg, epi, max_rows, st, kid);
-    return dispatch256<8, 1>(g, b_ks, wg, epi, max_rows, st, kid);
+    return dispatch256<8, 2>(g, b_ks, wg, epi, max_rows, st, kid);                                  // 256 rows, eight waves
 }
 
 }  // namespace mole

@@ -10,6 +10,7 @@
 //                     h = xd . w1^T) with the epilogue left out: prologue + K loop (LDS-DMA feed, fragment reads,
 //                     MFMAs) + launch.
 #include "gemm.h"
+#include "mole_hip_probe.h"
 
 namespace mole {
 

@@ -32,17 +32,97 @@ WORKLOADS = {
 }
 PEAK_MFMA_TFLOPS = {"bf16": 2500.0, "f32": 157.3}   # MI355X dense peaks
 PEAK_HBM_GBS = 8000.0
-# HBM bytes per launch (read + write) of the grouped GEMMs at workload c2, from rocprofv3 FETCH_SIZE and
-# WRITE_SIZE runs of this script scaled by the same counters' readings for a copy of known size
-# (profiles/bench_c2_hbm_traffic.txt, profiles/bench_c3_c5_hbm_traffic.txt); c1 has no counter run and reports null
-MEASURED_TRAFFIC_BYTES = {
-    "c2": {"ffn_fwd1": 758.2e6, "ffn_fwd2": 373.2e6, "ffn_gw2": 547.0e6, "ffn_da": 748.5e6, "ffn_gw1": 547.0e6,
-           "ffn_gx": 383.2e6},
-    "c3": {"ffn_fwd1": 3816.1e6, "ffn_fwd2": 2214.7e6, "ffn_gw2": 3085.4e6, "ffn_da": 3824.1e6, "ffn_gw1": 3085.4e6,
-           "ffn_gx": 2219.6e6},
-    "c5": {"ffn_fwd1": 4371.8e6, "ffn_fwd2": 3329.5e6, "ffn_gw2": 3032.0e6, "ffn_da": 4378.7e6, "ffn_gw1": 3032.0e6,
-           "ffn_gx": 3306.4e6},
-}
+# HBM bytes per launch (read + write) of the grouped products come from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of
+# this script (`--ingest-counters` turns the two counter CSVs into profiles/hbm_traffic.json, which also records the
+# hashes of the kernel sources the counters were read from).  A workload whose kernel sources have changed since
+# reports "traffic": null rather than a stale figure.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+KERNEL_SOURCES = ("MOLE/cpp/gemm256.hip", "MOLE/cpp/ffn_gemm.hip", "MOLE/cpp/gemm.h")
+# read bytes = FETCH_SIZE x 2 KiB, written bytes = WRITE_SIZE x 1 KiB on this chip (calibrated against a copy of
+# known size in the same runs, see profiles/bench_c2_hbm_traffic.txt)
+FETCH_UNIT_BYTES, WRITE_UNIT_BYTES = 2048.0, 1024.0
+# a product counts as HBM-bound when the bytes it really moves, over its duration, reach the rate a large copy
+# sustains on this chip (4.9-5.4 TB/s of the 8 TB/s peak); below that its duration follows the matrix pipe
+HBM_BOUND_FROM = 0.55
+
+
+def kernel_source_hashes():
+    import hashlib
+    return {f: hashlib.sha256(open(os.path.join(ROOT, f), "rb").read()).hexdigest()[:16] for f in KERNEL_SOURCES}
+
+
+def measured_traffic(name):
+    """{kernel: bytes per launch} for workload `name`, or {} when no counter run exists for the current kernel sources."""
+    try:
+        with open(TRAFFIC_FILE) as fh:
+            data = json.load(fh)
+    except (OSError, ValueError):
+        return {}
+    entry = data.get("workloads", {}).get(name)
+    if not entry or entry.get("kernel_sources") != kernel_source_hashes():
+        return {}
+    return entry["bytes_per_launch"]
+
+
+def ingest_counters(args):
+    """Reads the counter_collection CSVs of a FETCH_SIZE run and a WRITE_SIZE run of `bench.py --workload W --no-c1
+    --no-c35 --no-cpu-baseline` and stores the grouped products' HBM bytes per launch for W in profiles/hbm_traffic.json."""
+    import csv
+    import re
+    import subprocess
+
+    def launches(path, counter):
+        """{product: [counter value of every launch, in dispatch order]} of the grouped kernels in one counter CSV"""
+        rows = []
+        with open(path, newline="") as fh:
+            for r in csv.DictReader(fh):
+                mt = re.search(r"mole::gemm(?:256)?_kernel<(.*)>\(", r["Kernel_Name"])
+                if r.get("Counter_Name") == counter and mt:
+                    targs = [a.strip() for a in mt.group(1).split(",")]
+                    rows.append((int(r["Dispatch_Id"]), targs, int(r["Grid_Size"]), float(r["Counter_Value"])))
+        rows.sort(key=lambda t: t[0])
+        # template arguments end in <..., WG, [BM, BN,] EPI>: EPI 2 = h and a, 1 = out, 3 = t, 4 = a weight gradient (g_w2
+        # and g_w1 alternate), 0 = gx - or a product of the gate, which has another grid than the launch of `out`
+        out = {n: [] for n in ("ffn_fwd1", "ffn_fwd2", "ffn_gw2", "ffn_da", "ffn_gw1", "ffn_gx")}
+        grid_fwd2, n_wg = None, 0
+        for _, targs, grid, val in rows:
+            epi = int(targs[-1])
+            if epi == 2: out["ffn_fwd1"].append(val)
+            elif epi == 1: out["ffn_fwd2"].append(val); grid_fwd2 = grid
+            elif epi == 3: out["ffn_da"].append(val)
+            elif epi == 4 and "true" in targs[:4]:
+                out["ffn_gw2" if n_wg % 2 == 0 else "ffn_gw1"].append(val); n_wg += 1
+            elif epi == 0 and grid == grid_fwd2: out["ffn_gx"].append(val)
+        return out
+    fetch, write = launches(args.ingest_counters[0], "FETCH_SIZE"), launches(args.ingest_counters[1], "WRITE_SIZE")
+    steps = len(fetch["ffn_fwd1"])
+    assert steps > 0 and all(len(v) == steps for v in fetch.values()) and all(len(v) == steps for v in write.values()), \
+        ({n: len(v) for n, v in fetch.items()}, {n: len(v) for n, v in write.items()})
+    first = steps // 3                      # the first third of the launches is warm-up
+    out = {}
+    for n in fetch:
+        rd = sum(fetch[n][first:]) / (steps - first) * FETCH_UNIT_BYTES
+        wr = sum(write[n][first:]) / (steps - first) * WRITE_UNIT_BYTES
+        out[n] = round(rd + wr)
+        out[n + "_read"], out[n + "_written"] = round(rd), round(wr)
+    try:
+        with open(TRAFFIC_FILE) as fh:
+            data = json.load(fh)
+    except (OSError, ValueError):
+        data = {"what": "HBM bytes per launch of the grouped products, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of "
+                        "bench.py (bench.py --ingest-counters); FETCH_SIZE x 2 KiB + WRITE_SIZE x 1 KiB", "workloads": {}}
+    try:
+        commit = subprocess.run(["git", "-C", ROOT, "rev-parse", "--short", "HEAD"], capture_output=True, text=True).stdout.strip()
+    except OSError:
+        commit = ""
+    data["workloads"][args.workload] = {"kernel_sources": kernel_source_hashes(), "measured_after_commit": commit,
+                                        "steps_averaged": steps - first, "bytes_per_launch": out}
+    with open(TRAFFIC_FILE, "w") as fh:
+        json.dump(data, fh, indent=1, sort_keys=True)
+        fh.write("\n")
+    print(json.dumps({args.workload: out}))
+
+
 PEAK_HBM_BYTES = PEAK_HBM_GBS * 1e9
 
 
@@ -286,13 +366,14 @@ def measure_layer(name, steps, warmup, with_adam=True):
     peak = PEAK_MFMA_TFLOPS[w["dtype"]]
     dom_s = kernels[dom]["avg_us"] * 1e-6
     gemm_total_us = sum(kernels[n]["avg_us"] for n in gemms)
-    traffic = MEASURED_TRAFFIC_BYTES.get(name, {}).get(dom)
+    traffic = measured_traffic(name).get(dom)
     mfma_frac = kernels[dom]["tflops"] / peak
     hbm_alg_frac = gemm_bytes[dom] / dom_s / PEAK_HBM_BYTES
     hbm_meas_frac = traffic / dom_s / PEAK_HBM_BYTES if traffic else None
-    # the roof the kernel is nearer to, judged by the bytes it really moves when a counter run gave them
-    hbm_side = hbm_meas_frac if hbm_meas_frac is not None else hbm_alg_frac
-    if hbm_side > mfma_frac:
+    # HBM-bound when the bytes the kernel really moves go at the rate of a large copy; without a counter run for the
+    # current kernel sources, when its algorithmic bytes are nearer their roof than its flop are to theirs
+    hbm_bound = hbm_meas_frac >= HBM_BOUND_FROM if hbm_meas_frac is not None else hbm_alg_frac > mfma_frac
+    if hbm_bound:
         roofline = {"bound": "hbm", "kernel": dom, "achieved": round(gemm_bytes[dom] / dom_s / 1e9, 1), "peak": PEAK_HBM_GBS,
                     "unit": "GB/s", "frac": round(hbm_alg_frac, 4)}
     else:
@@ -436,6 +517,10 @@ def main():
                     help="c4 only: fetch the experts again for every backward pass, as the reference does")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-c1", action="store_true", help="skip the configuration-1 (fp32) figures beside the headline")
+    ap.add_argument("--no-c35", action="store_true", help="skip the configuration-3 and -5 figures beside the headline")
+    ap.add_argument("--ingest-counters", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
+                    help="no GPU work: read the counter_collection CSVs of a FETCH_SIZE and a WRITE_SIZE rocprofv3 run of "
+                         "--workload W and store the products' HBM bytes per launch in profiles/hbm_traffic.json")
     ap.add_argument("--probe", action="store_true", help="run the matrix-core and K-loop probes instead of the layer")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -443,6 +528,8 @@ def main():
               file=sys.stderr)
         sys.exit(2)
 
+    if args.ingest_counters:
+        return ingest_counters(args)
     import torch
     assert torch.cuda.is_available(), "bench.py needs an MI355X"
     if args.probe:
@@ -461,6 +548,13 @@ def main():
         c1 = measure_layer("c1", args.steps, args.warmup, with_adam=False)
         out["c1"] = {"tokens_per_s": c1["value"], "ms_per_step": c1["ms_per_step"], "dtype": c1["dtype"],
                      "workload": c1["config"]["workload"], "roofline": c1["roofline"], "hbm_permutes": c1["hbm_permutes"]}
+    if args.workload == "c2" and not args.no_c35:
+        # configurations 3 (Zipf loads, 64 experts) and 5 (256 experts, top-8) beside the headline, a few steps each
+        for name in ("c3", "c5"):
+            r = measure_layer(name, min(args.steps, 10), min(args.warmup, 3), with_adam=False)
+            out[name] = {"tokens_per_s": r["value"], "ms_per_step": r["ms_per_step"], "dtype": r["dtype"],
+                         "workload": r["config"]["workload"], "roofline": r["roofline"], "hbm_permutes": r["hbm_permutes"],
+                         "kernels_us": {n: v["avg_us"] for n, v in r["kernels"].items()}}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))

@@ -75,27 +75,11 @@ enum {
     MOLE_K_GATE_FWD = 14,   /* gate logits + softmax in one kernel, or the softmax kernel alone */
     MOLE_K_GATE_BWD = 15,   /* dgates -> dlogits */
     MOLE_K_GATE_WGRAD = 16, /* dWg: partial sums + their reduction */
-    MOLE_K_PROBE = 17,      /* mole_probe_* */
+    MOLE_K_RESERVED_17 = 17, /* timing slot of the measurement aids declared in mole_hip_probe.h */
     MOLE_K_COUNT = 18
 };
 int mole_kernel_timing_enable(int on);
 int mole_kernel_timing_read(int n_ids, int *counts, float *ms_total);
-
-/* Measurement aids for the roofline of the grouped products (no counterpart in the reference; used by the
- * benchmark script only).  mole_probe_mfma: `blocks` blocks of eight waves issue v_mfma_f32_32x32x16_bf16 back to
- * back for `iters` rounds of 8 on operands taken once from `operands` (mole_probe_mfma_operand_bytes() bytes: zeros
- * show the published peak, random bf16 data what the chip sustains); sink: blocks * 512 floats; *flop_out: flop of
- * the launch.  mole_probe_kloop: the product kernel at the shape of h = xd . w1^T (a [rows,K], b [E,N,K], experts
- * by offsets / kept_rows) with its epilogue left out - prologue, K loop and launch only; sink: 512 floats.
- * mole_probe_kloop_part: the same with one ingredient of the K loop taken out, to see what the loop waits for
- * (part 0: nothing, 1: the loads of the operand tiles into LDS, 2: the fragment reads from LDS, 3: the barriers, 4: all three);
- * what the accumulators then hold is meaningless.  All are timed under MOLE_K_PROBE. */
-size_t mole_probe_mfma_operand_bytes(void);
-int mole_probe_mfma(const void *operands, int blocks, int iters, float *sink, double *flop_out, mole_stream_t stream);
-int mole_probe_kloop(const void *a, const void *b, const int32_t *offsets, const int32_t *kept_rows, int E,
-                     int max_rows, int N, int K, float *sink, mole_stream_t stream);
-int mole_probe_kloop_part(const void *a, const void *b, const int32_t *offsets, const int32_t *kept_rows, int E,
-                          int max_rows, int N, int K, int part, float *sink, mole_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
  * Gate.  Replaces MOLETopk.forward (MOLE/utils/Ugate.py:11-14): scores = softmax(logits).

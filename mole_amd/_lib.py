@@ -12,7 +12,7 @@ from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_int32, c_int64
 
 import torch  # noqa: F401  (must precede the dlopen below)
 
-LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpp", "libmole_hip.so")
+LIB_PATH = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "MOLE", "cpp", "libmole_hip.so")
 
 MOLE_F32, MOLE_BF16 = 0, 1
 LAYOUT_PADDED, LAYOUT_RAGGED = 0, 1

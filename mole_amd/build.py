@@ -1,4 +1,5 @@
-"""Builds mole_amd/cpp/libmole_hip.so (gfx950 only) with hipcc.  `python -m mole_amd.build`."""
+"""Builds MOLE/cpp/libmole_hip.so (gfx950 only) with hipcc, from the sources beside it: the native extension sits
+where the reference keeps its own (MOLE/cpp).  `python -m mole_amd.build`."""
 from __future__ import annotations
 
 import os
@@ -8,7 +9,7 @@ from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
-CPP = os.path.join(HERE, "cpp")
+CPP = os.path.join(ROOT, "MOLE", "cpp")
 LIB = os.path.join(CPP, "libmole_hip.so")
 SOURCES = ["error.cpp", "route.hip", "permute.hip", "ffn_gemm.hip", "gemm256.hip", "adam.hip", "unimem.hip", "probe.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -17,6 +18,10 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-x", "hip",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wno-unused-command-line-argument",
          "-I" + os.path.join(ROOT, "include"), "-I" + CPP]
+# MOLE_TUNING=1 in the environment of the build adds the tile shapes, launch orders and K-loop ablations that were
+# measured against the defaults (selected at run time by MOLE_TMB, MOLE_MFAST, ...: see MOLE/cpp/gemm256.hip)
+if os.environ.get("MOLE_TUNING"):
+    FLAGS.append("-DMOLE_TUNING")
 
 
 def _compile(src: str) -> str:
