@@ -91,9 +91,55 @@ __global__ __launch_bounds__(ADAM_THREADS) void adam_bf16_kernel(const bf16_t *_
     }
 }
 
+// acc[i] = acc[i] + add[i], rounded once to the parameter dtype (the reference's host-side `+=` of two tensors of that
+// dtype, data_transfer.cpp:9-12): 16 bytes per lane in, 16 out.
+template <typename T>
+__global__ __launch_bounds__(ADAM_THREADS) void grad_add_kernel(T *__restrict__ acc, const T *__restrict__ add, size_t n) {
+    constexpr int V = 16 / sizeof(T);
+    const size_t i = ((size_t)blockIdx.x * ADAM_THREADS + threadIdx.x) * V;
+    if (i + V <= n) {
+        if constexpr (sizeof(T) == 4) {
+            float4 a = *reinterpret_cast<const float4 *>(acc + i);
+            const float4 b = *reinterpret_cast<const float4 *>(add + i);
+            a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+            *reinterpret_cast<float4 *>(acc + i) = a;
+        } else {
+            const uint4 a = *reinterpret_cast<const uint4 *>(acc + i), b = *reinterpret_cast<const uint4 *>(add + i);
+            const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, bw[4] = {b.x, b.y, b.z, b.w};
+            uint32_t ow[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const bf16_t lo = (bf16_t)(__uint_as_float(aw[q] << 16) + __uint_as_float(bw[q] << 16));
+                const bf16_t hi = (bf16_t)(__uint_as_float(aw[q] & 0xffff0000u) + __uint_as_float(bw[q] & 0xffff0000u));
+                ow[q] = (uint32_t)__builtin_bit_cast(uint16_t, lo) | ((uint32_t)__builtin_bit_cast(uint16_t, hi) << 16);
+            }
+            *reinterpret_cast<uint4 *>(acc + i) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+        }
+    } else {
+        for (size_t j = i; j < n; ++j) acc[j] = from_f32<T>(to_f32(acc[j]) + to_f32(add[j]));
+    }
+}
+
 }  // namespace mole
 
 using namespace mole;
+
+extern "C" int mole_grad_add(void *acc, const void *add, size_t n, int dtype, mole_stream_t stream) {
+    MOLE_REQUIRE(dtype == MOLE_F32 || dtype == MOLE_BF16, "mole_grad_add: bad dtype %d", dtype);
+    if (n == 0) return 0;
+    MOLE_REQUIRE(acc && add, "mole_grad_add: null pointer");
+    MOLE_REQUIRE((((uintptr_t)acc | (uintptr_t)add) & 15) == 0, "mole_grad_add: buffers must be 16-byte aligned");
+    const size_t per_block = (size_t)ADAM_THREADS * (dtype == MOLE_BF16 ? 8 : 4);
+    const size_t blocks = (n + per_block - 1) / per_block;
+    MOLE_REQUIRE(blocks <= 0x7fffffffull, "mole_grad_add: n=%zu too large for one launch", n);
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == MOLE_BF16)
+        hipLaunchKernelGGL(grad_add_kernel<bf16_t>, dim3((unsigned)blocks), dim3(ADAM_THREADS), 0, st, (bf16_t *)acc, (const bf16_t *)add, n);
+    else
+        hipLaunchKernelGGL(grad_add_kernel<float>, dim3((unsigned)blocks), dim3(ADAM_THREADS), 0, st, (float *)acc, (const float *)add, n);
+    MOLE_LAUNCH_CHECK();
+    return 0;
+}
 
 extern "C" int mole_adam_step(const void *p, const void *g, float *m, float *v, void *p_out, size_t n, int dtype,
                               float beta1, float beta2, int t, float lr, float lam, float eps, int adamw,

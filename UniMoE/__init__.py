@@ -13,6 +13,7 @@ import MOLE.utils.Ugate
 import MOLE.utils.Uparam
 import MOLE.utils.Uscheduler
 import MOLE.utils.Ustream
+import MOLE.utils.Utimer
 
 for _name, _mod in list(sys.modules.items()):
     if _name == "MOLE" or _name.startswith("MOLE."):

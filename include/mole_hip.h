@@ -257,7 +257,9 @@ int mole_gemm_tn(const void *a, const void *b, int dtype, int rows, int Mo, int 
  *   release(view_base, n, stream) records that compute on `stream` has finished with the slots.
  *
  * prefetch_ids / fetch_ids are the same two calls for an explicit list of experts instead of a range:
- * expert expert_ids[i] (an index into the pinned host arrays) lands in the i-th slot of the call, so the
+ * expert expert_ids[i] (an index into the pinned host arrays; the library checks ids for >= 0 only - it is handed
+ * base pointers, not extents, so the caller guarantees that every id, like every base + n of the range forms,
+ * lies inside its host arrays, as the reference's callers do for their tensor slices) lands in the i-th slot of the call, so the
  * host side can bring in only the experts that routing activated (kept_rows[e] > 0) and hand the grouped
  * FFN a compacted offsets / kept_rows pair in the same order.  The reference always copies whole index
  * ranges (MOLE/cpp/core.cpp:41-57, 1025-1047); these two have no counterpart there.  Consecutive ids that
@@ -347,6 +349,11 @@ int mole_unimem_store_state(void *handle, void *const host_dst[], const void *co
 int mole_adam_step(const void *p, const void *g, float *m, float *v, void *p_out, size_t n, int dtype,
                    float beta1, float beta2, int t, float lr, float lam, float eps, int adamw,
                    mole_stream_t stream);
+
+/* acc[i] += add[i] over n elements of dtype, rounded once per element: the sum of a micro-step's gradients and the
+ * running sum fetched from the host; replaces the host-side addition of grad_accumulate
+ * (MOLE/cpp/data_transfer.cpp:9-12, called from store_grad, MOLE/cpp/core.cpp:77-103).  16-byte aligned. */
+int mole_grad_add(void *acc, const void *add, size_t n, int dtype, mole_stream_t stream);
 
 /* Greedy cross-layer prefetch assignment; replaces fast_assign_prefetch
  * (MOLE/cpp/core.cpp:1302-1345).  lp_out [n]; gp_out holds up to gp_cap triples

@@ -83,6 +83,7 @@ _SIGNATURES = {
     "mole_unimem_store_state": (c_int, [_P, POINTER(_P), POINTER(_P), POINTER(c_size_t), c_int, _P]),
     "mole_adam_step": (c_int, [_P, _P, _P, _P, _P, c_size_t, c_int, c_float, c_float, c_int, c_float, c_float, c_float,
                                c_int, _P]),
+    "mole_grad_add": (c_int, [_P, _P, c_size_t, c_int, _P]),
     "mole_fast_assign_prefetch": (c_int, [c_int, POINTER(c_int), POINTER(c_int), c_int, POINTER(c_int),
                                           POINTER(c_int), c_int, POINTER(c_int)]),
 }

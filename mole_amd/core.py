@@ -19,6 +19,7 @@ handed to the compute stream through events (core.cpp:110-143, 212-249).
 from __future__ import annotations
 
 import ctypes
+import itertools
 from ctypes import c_float, c_int, c_uint64, c_void_p
 from typing import List, Optional
 
@@ -375,6 +376,12 @@ def plan_chunks(n_total: int, prefetched: int, view_pool_size: int, ebatch_size:
     return out
 
 
+# Tags under which forward passes fill pool slots come from one counter for the whole process: a tag is never handed
+# out twice while the pool lives, whatever layers are destroyed and rebuilt around it (a rebuilt layer can get the same
+# pinned host addresses back from the allocator, and a repeated tag would then match a stale slot).
+_PASS_TAGS = itertools.count(1)
+
+
 class MOLECore:
     """Per-layer state and the expert-batch pipeline (define.hpp:338-607, core.cpp:991-1300).
 
@@ -424,6 +431,10 @@ class MOLECore:
         self._passes = 0            # forward passes so far: part of the tag under which a pass fills pool slots
         self._tag = 0               # tag of the pass in preparation or in flight (0: none yet)
         self._tag_used = True       # a forward pass has run under _tag: the next prefetch_fwd / forward takes a new one
+        # Where a pass keeps its experts - a fixed stretch of slots (first slot) or the prefetch stack (None) - is
+        # decided once per pass, by the first prefetch for it or by the forward itself, and carried to its backward.
+        self._home_fwd = None       # decision for the coming forward pass (valid while experts are prefetched for it)
+        self._home_pass = None      # decision of the last forward pass: its backward and the prefetches for it use it
 
     # the reference's counters of experts prefetched so far (define.hpp:352-353)
     @property
@@ -477,7 +488,7 @@ class MOLECore:
             return 0
         if self._tag_used:
             self._passes += 1
-            self._tag = ((self.moe_id + 1) << 40) | self._passes
+            self._tag = next(_PASS_TAGS)
             self._tag_used = False
         return self._tag
 
@@ -494,6 +505,15 @@ class MOLECore:
         if sum(c.d_experts for c in layers) > um.pool_size or um.virtual_offset() != 0:
             return None
         return sum(c.d_experts for c in layers[:layers.index(self)])
+
+    def _home_for(self, which: str):
+        """The slot placement of the pass `which` is being prepared for: decided when nothing has been prefetched for
+        the coming forward pass yet, then kept until its backward pass is done."""
+        if which == "fwd":
+            if not self._pref["fwd"]:
+                self._home_fwd = self._home_base()
+            return self._home_fwd
+        return self._home_pass
 
     def _home_fetch(self, home: int, ids, tag: int):
         """Bring the experts `ids` into their own slots (home + e); runs of consecutive experts in one call."""
@@ -514,7 +534,7 @@ class MOLECore:
             todo = [e for e in known if e not in seen][:batch_size]
         if not todo:
             return
-        home = self._home_base()
+        home = self._home_for(which)
         if home is not None:
             self._home_fetch(home, todo, tag)
         elif not self.activated_only:
@@ -611,7 +631,8 @@ class MOLECore:
         host_meta, tag = None, 0
         if self.d_experts:
             um = get_UniMem()
-            home = self._home_base()
+            home = self._home_for("fwd")
+            self._home_pass = home
             resident = self._take_prefetched("fwd", home)
             tag = self._forward_tag()
             self._tag_used = True
@@ -640,7 +661,7 @@ class MOLECore:
                     um.wait_slots(view_base, size)
                     H.ffn_fwd_into(x2, off_c[lo:], kept_c[lo:], size, rows, M, F, p[0], p[1], p[2], p[3], h, a, out)
                     um.release(view_base, size)
-        saved = (x2, h, a, offsets, kept_rows, requires_grad, shape, host_meta, tag)
+        saved = (x2, h, a, offsets, kept_rows, requires_grad, shape, host_meta, tag, self._home_pass)
         if return_saved:          # the caller (an autograd node) keeps the activations itself
             return out.view(shape), saved
         self._saved = saved       # reference behaviour: the core holds them until backward (define.hpp:594-606)
@@ -651,7 +672,7 @@ class MOLECore:
             saved, self._saved = self._saved, None
         if saved is None:
             raise RuntimeError("MOLECore.backward without a preceding forward")
-        x2, h, a, offsets, kept_rows, need_gx, shape, host_meta, tag = saved
+        x2, h, a, offsets, kept_rows, need_gx, shape, host_meta, tag, home = saved
         M = shape[-1]
         go = all_output_grad.reshape(-1, M)
         if not go.is_contiguous():
@@ -668,7 +689,6 @@ class MOLECore:
                            gx, acc, self.gelu_bwd)
         if self.d_experts:
             um = get_UniMem()
-            home = self._home_base()
             resident = self._take_prefetched("bwd", home)
             d, e0 = self.d_experts, self.s_experts
             host_grads = [c[1] for c in self.cpu]
@@ -768,7 +788,7 @@ class MOLECore:
         prev = [torch.empty_like(gg) for gg in g]
         um.load_state(prev, host_slices, after_writeback=True)
         for gg, pp in zip(g, prev):
-            gg += pp
+            H.grad_add(gg, pp)
         um.store_state(host_slices, g)
 
     def _instant_adam(self, p_slots, g, ids, adding):
@@ -811,7 +831,7 @@ class MOLECore:
             for k in range(4):
                 gk = g[k][at:at + n]
                 if adding:
-                    gk += g_prev[k]
+                    H.grad_add(gk, g_prev[k])
                 out = torch.empty_like(gk)
                 per_expert = gk[0].numel() * es
                 H.adam_step(p_slots[k] + at * per_expert, gk, m[k], v[k], beta1, beta2, t + 1, lr, lam, eps, adamw, p_out=out)
@@ -829,11 +849,17 @@ class BatchFusedFWD(torch.autograd.Function):
     def forward(ctx, dispatched_input, module, dummy_param, time_it=False, prefetch=False, offsets=None, kept_rows=None):
         ctx.module = module
         ctx.prefetch = prefetch
+        ctx.time_it = bool(time_it)
         out = module.MOLECore.forward(dispatched_input, dispatched_input.requires_grad, offsets, kept_rows)
         return out
 
     @staticmethod
     def backward(ctx, grad_out):
+        if ctx.time_it:       # the expert node's share of the layer's backward (the reference times the same span)
+            from .utils.Utimer import UATimer
+            UATimer.track_bwd_start(ctx.module.moe_id)
         gx = ctx.module.MOLECore.backward(grad_out)
+        if ctx.time_it:
+            UATimer.track_bwd_end(ctx.module.moe_id)
         dummy = torch.zeros_like(ctx.module.dummy_param) if ctx.module.dummy_param is not None else None
         return gx, None, dummy, None, None, None, None

@@ -318,6 +318,14 @@ def ffn_bwd(go, xd, h, a, offsets, kept_rows, w1, w2, g_w1, g_b1, g_w2, g_b2, ne
     return gx
 
 
+def grad_add(acc: torch.Tensor, add: torch.Tensor) -> None:
+    """acc += add, element by element in the tensors' dtype (one rounding): gradient sums over micro-steps."""
+    _dev(acc); _dev(add)
+    if acc.dtype != add.dtype or acc.numel() != add.numel() or not (acc.is_contiguous() and add.is_contiguous()):
+        raise RuntimeError("mole_amd.grad_add: acc and add must be contiguous and agree in dtype and size")
+    L.check(L.lib().mole_grad_add(L.ptr(acc), L.ptr(add), acc.numel(), L.dtype_code(acc.dtype), L.stream()), "mole_grad_add")
+
+
 def adam_step(p, g, m, v, beta1: float, beta2: float, t: int, lr: float, lam: float, eps: float, adamw: bool,
               p_out=None) -> None:
     """One fused Adam / AdamW step (define.hpp:543-579) over all elements of p: m and v (fp32) are updated in

@@ -27,6 +27,7 @@ from .. import core
 from .. import hip_ops as H
 from ..core import BatchFusedFWD, MOLECore
 from ..utils import Ugate
+from ..utils.Utimer import UATimer
 from ..utils.Uparam import CPUHostBatchedParameter, GPUHostBatchedParameter, UnifiedCPUTensor
 from . import fast_dispatch as tutel_fast_dispatcher
 
@@ -56,8 +57,9 @@ class _FusedMoE(torch.autograd.Function):
     """x [S,M] -> y [S,M] on the ragged layout; the whole of layer.py:442-458 in one node."""
 
     @staticmethod
-    def forward(ctx, x, wg, dummy_param, module, capacity_factor):
+    def forward(ctx, x, wg, dummy_param, module, capacity_factor, time_it=False):
         m = module
+        ctx.time_it = time_it
         S, M = x.shape
         k = min(m.topk, m.total_experts)
         scores = Ugate.gate_scores(x, wg, m.gate[0].logit_bias)
@@ -78,6 +80,8 @@ class _FusedMoE(torch.autograd.Function):
     def backward(ctx, dy, d_l_aux):
         m, r = ctx.m, ctx.r
         x, wg, scores, out = ctx.saved_tensors
+        if ctx.time_it:
+            UATimer.track_bwd_start(m.moe_id)
         d_o, dgates = H.combine_bwd(dy.contiguous(), out, r.row, r.gates)
         gxd = m.MOLECore.backward(d_o, saved=ctx.saved)
         ctx.saved = None
@@ -88,7 +92,9 @@ class _FusedMoE(torch.autograd.Function):
         wg32 = wg.detach().float().contiguous()
         dx = H.dispatch_bwd(gxd, r.row, dlogits, wg32)
         dwg = H.gate_wgrad(dlogits, x).to(wg.dtype)
-        return dx, dwg, torch.zeros_like(m.dummy_param), None, None
+        if ctx.time_it:
+            UATimer.track_bwd_end(m.moe_id)
+        return dx, dwg, torch.zeros_like(m.dummy_param), None, None, None
 
 
 class MOLEModule(torch.nn.Module):
@@ -236,6 +242,8 @@ class MOLEModule(torch.nn.Module):
                 capacity_factor=1.0, time_it=False, prefetch=False):
         original_shape = input_.shape
         original_dtype = input_.dtype
+        if time_it:      # the profiling window of the scheduler: this layer's forward and backward spans are recorded
+            UATimer.track_fwd_start(self.moe_id)
         if prefetch:
             input_ = pfetchbwd.apply(input_, self)
         resized_input = input_.reshape(-1, self.embed_dim)
@@ -253,10 +261,12 @@ class MOLEModule(torch.nn.Module):
             expert_output = tutel_fast_dispatcher.fast_decode(data=experts_output, critial_data=crit)
         else:
             expert_output, self.l_aux = _FusedMoE.apply(resized_input, self.gate[0].linear.weight, self.dummy_param,
-                                                        self, float(capacity_factor))
+                                                        self, float(capacity_factor), bool(time_it))
 
         expert_output = expert_output.reshape(original_shape)
         out = expert_output.to(original_dtype)
+        if time_it:
+            UATimer.track_fwd_end(self.moe_id)
 
         if prefetch:
             if self.moe_id < len(MOLEModule._instance) - 1:

@@ -5,17 +5,27 @@ measured times into per-layer prefetch counts (MOLE/utils/Uscheduler.py:228-349)
     UniScheduler.set_prefetch_scheme   applies a plan to the MOLEModule instances (Uscheduler.py:259-343)
     UniScheduler.measure_fetch_time    seconds to fetch one expert, from MOLEModule.dummy_fetch (Uscheduler.py:231-238)
     UniScheduler.prefetch_fwd          what a training loop calls before the first layer (Uscheduler.py:345-349)
+    UniScheduler.schedule_policy / set_step / time_it / prefetch_it / profile_prefetch
+                                       the profiling window (Uscheduler.py:56-63, 163-184, 228-258): during the first
+                                       profile_step steps the layers run with time_it=True and record their forward
+                                       and backward spans (utils/Utimer.py); profile_prefetch folds them and the
+                                       measured fetch time into running means and plans the prefetch from them
+    UniScheduler.save_states / load_states
+                                       the checkpoint file (Uscheduler.py:67-92): torch.save([model_state,
+                                       optim_state]) with one get_layer_state() dict per layer
 
-The rest of the reference's scheduler (argument parsing, optimizer set-up, checkpoint files, the timers that
-produce the per-layer statistics) is not part of this package: the caller passes the per-layer forward and
-backward times it measured.
+The rest of the reference's scheduler (argument parsing, construction of the CPU optimizer) is not part of this
+package; the optimizer state saved here is that of the in-pipeline Adam (the fp32 moments of the offloaded experts).
 """
 from __future__ import annotations
 
 import math
 from typing import List, Optional, Sequence
 
+import torch
+
 from .. import core
+from .Utimer import UATimer
 
 
 def plan_prefetch(pool_size: int, fwd_stat: Sequence[float], bwd_stat: Sequence[float], ftime: float,
@@ -65,6 +75,134 @@ def plan_prefetch(pool_size: int, fwd_stat: Sequence[float], bwd_stat: Sequence[
 class UniScheduler:
     """The prefetch-related static methods of the reference's UniScheduler, over MOLEModule._instance."""
     ftime: Optional[float] = None
+    fwd_stat: Optional[List[float]] = None
+    bwd_stat: Optional[List[float]] = None
+    cur_step = -1
+    profile_step = -1
+    prefetch_on = False
+    deactivate_first_prefetch = True
+    prefetch_floor = False
+    global_prefetch = False
+    last_plan: Optional[List[dict]] = None
+
+    @staticmethod
+    def reset():
+        """Forget policy, step counter and every measured time (a new run in the same process)."""
+        UniScheduler.ftime = UniScheduler.fwd_stat = UniScheduler.bwd_stat = UniScheduler.last_plan = None
+        UniScheduler.cur_step, UniScheduler.profile_step, UniScheduler.prefetch_on = -1, -1, False
+        UniScheduler.deactivate_first_prefetch, UniScheduler.prefetch_floor, UniScheduler.global_prefetch = True, False, False
+        UATimer.clear()
+
+    # ---- the profiling window (Uscheduler.py:56-63, 163-184, 228-258) ------------------------------------
+    @staticmethod
+    def schedule_policy(profile_step, prefetch_on, deactivate_first_prefetch=True, prefetch_floor=False,
+                        global_prefetch=False):
+        UniScheduler.profile_step = profile_step
+        UniScheduler.prefetch_on = prefetch_on
+        UniScheduler.deactivate_first_prefetch = deactivate_first_prefetch
+        UniScheduler.prefetch_floor = prefetch_floor
+        UniScheduler.global_prefetch = global_prefetch
+
+    @staticmethod
+    def set_step(cur_step):
+        """At the beginning of every step (Uscheduler.py:163-169): inside the profiling window the timers start
+        afresh; the prefetch stack is emptied."""
+        UniScheduler.cur_step = cur_step
+        if UniScheduler.time_it():
+            UATimer.clear()
+        core.clear_virtual_mem()
+
+    @staticmethod
+    def time_it() -> bool:
+        """Pass this as MOLEModule.forward(..., time_it=...): true during the profiling window (Uscheduler.py:171-177)."""
+        return UniScheduler.cur_step < UniScheduler.profile_step
+
+    @staticmethod
+    def prefetch_it() -> bool:
+        """Pass this as MOLEModule.forward(..., prefetch=...): true after the window when prefetch is on (Uscheduler.py:179-184)."""
+        return UniScheduler.cur_step > UniScheduler.profile_step and UniScheduler.prefetch_on
+
+    @staticmethod
+    def profile_prefetch(force_prefetch_scheme=None):
+        """At the end of a step inside the profiling window (Uscheduler.py:228-258): measure the time to fetch one
+        expert, read the layers' forward and backward spans of this step, fold all three into running means
+        (mean of the old value and the new one, as the reference does) and, with prefetch on, plan the prefetch
+        from them.  The first two steps are skipped like the reference's (start-up costs would distort the means).
+        Returns the plan, or None when nothing was planned."""
+        if not UniScheduler.time_it() or UniScheduler.cur_step < 2:
+            return None
+        UniScheduler.measure_fetch_time(1)
+        fwd, bwd = UATimer.stats()
+        mean = lambda old, new: list(new) if old is None else [(a + b) / 2 for a, b in zip(old, new)]
+        if fwd:
+            UniScheduler.fwd_stat = mean(UniScheduler.fwd_stat, fwd)
+        if bwd:
+            UniScheduler.bwd_stat = mean(UniScheduler.bwd_stat, bwd)
+        if not UniScheduler.prefetch_on or UniScheduler.fwd_stat is None or UniScheduler.bwd_stat is None:
+            return None
+        return UniScheduler.set_prefetch_scheme(UniScheduler.fwd_stat, UniScheduler.bwd_stat, None,
+                                                UniScheduler.prefetch_floor, force_prefetch_scheme,
+                                                UniScheduler.deactivate_first_prefetch, UniScheduler.global_prefetch)
+
+    # ---- checkpoint files (Uscheduler.py:67-92) ----------------------------------------------------------
+    @staticmethod
+    def get_optim_state():
+        """State of the in-pipeline Adam in the layout of the reference's MOLEMixedAdam.get_optim_state
+        (MOLE/optim/mixed_optim.py:245-277): [expert_state, gate_state]; expert_state[4 l + p] = {"step",
+        "exp_avg", "exp_avg_sq"} for parameter kind p of layer l (the order of the optimizer's parameter list,
+        Uscheduler.py:104-112), the moments being the fp32 arrays of the layer's offloaded experts.  The gate is
+        the caller's own optimizer's business here (gate_state None), and so are GPU-resident experts."""
+        core.synchronize_tran()
+        state = {}
+        for l, m in enumerate(UniScheduler._layers()):
+            if m.d_experts == 0 or not m.adv_adam:
+                continue
+            # set_adam hands over the counter before a step (the reference's optimizer does so every step), so after
+            # that step the number of steps done is one more
+            t = m.MOLECore.adam[2] + 1 if m.MOLECore.adam is not None else 0
+            for p, c in enumerate(m.MOLECore.cpu):
+                state[4 * l + p] = {"step": int(t), "exp_avg": c[2].clone(), "exp_avg_sq": c[3].clone()}
+        return [state or None, None]
+
+    @staticmethod
+    def set_optim_state(states):
+        core.synchronize_tran()
+        expert_state = states[0] if states else None
+        if not expert_state:
+            return
+        for l, m in enumerate(UniScheduler._layers()):
+            if m.d_experts == 0 or not m.adv_adam:
+                continue
+            for p, c in enumerate(m.MOLECore.cpu):
+                st = expert_state[4 * l + p]
+                # the reference's state holds GPU-resident experts first: the offloaded ones are the last rows
+                c[2].copy_(st["exp_avg"][-c[2].shape[0]:])
+                c[3].copy_(st["exp_avg_sq"][-c[3].shape[0]:])
+            if m.MOLECore.adam is not None:
+                a = list(m.MOLECore.adam)
+                a[2] = int(expert_state[4 * l]["step"])      # steps done = the counter before the next step
+                m.MOLECore.adam = tuple(a)
+
+    @staticmethod
+    def save_states(state_file="MOLE_states", grad=False):
+        """torch.save([model_state, optim_state], state_file + ".pt") (Uscheduler.py:67-75): model_state holds one
+        MOLEModule.get_layer_state(grad) per layer, in layer order."""
+        model_state = [m.get_layer_state(grad) for m in UniScheduler._layers()]
+        torch.save([model_state, UniScheduler.get_optim_state()], state_file + ".pt")
+
+    @staticmethod
+    def load_states(state_file="MOLE_states", grad=False):
+        """Inverse of save_states (Uscheduler.py:78-92).  The file is read with a loader that executes nothing
+        from it (tensors, lists, dicts, numbers and None are all a state file holds)."""
+        all_state = torch.load(state_file + ".pt", map_location="cpu", weights_only=True)
+        model_state, optim_state = all_state[0], all_state[1]
+        layers = UniScheduler._layers()
+        if len(model_state) != len(layers):
+            raise RuntimeError(f"load_states: the file holds {len(model_state)} layers, the model has {len(layers)}")
+        for m, st in zip(layers, model_state):
+            m.set_layer_state(st, grad)
+        UniScheduler.set_optim_state(optim_state)
+        return all_state
 
     @staticmethod
     def _layers():
@@ -99,6 +237,7 @@ class UniScheduler:
             m.global_prefetch = use_global
             m.global_prefetch_fwd_count = p["global_fwd"]
             m.global_prefetch_bwd_count = p["global_bwd"]
+        UniScheduler.last_plan = plan
         return plan
 
     @staticmethod
@@ -106,6 +245,8 @@ class UniScheduler:
         layers = UniScheduler._layers()
         if not layers:
             return
+        if UniScheduler.profile_step >= 0 and not UniScheduler.prefetch_it():
+            return            # a policy is set (schedule_policy) and this step does not prefetch (Uscheduler.py:345-349)
         if layers[0].global_prefetch:
             layers[0].global_prefetch_fwd()
         layers[0].local_prefetch_fwd()

@@ -12,6 +12,10 @@ that changes a routing decision or a gradient shows up against data that does no
                       for hand-made tie / overflow / degenerate cases and seeded Zipf-skewed cases
   layer_small.npz     one fp32 layer (S 96, M 32, E 4, top-2, F 64, capacity factor 1.0, both GELU backward
                       variants): inputs, y, dx, dwg and the four expert gradients
+  MOLE_states_tiny.pt a checkpoint file in the layout UniScheduler.save_states writes in the reference
+                      (MOLE/utils/Uscheduler.py:67-75, MOLE/moe/layer.py:397-427): [model_state, optim_state],
+                      model_state = one {"gate", "experts", "grad"} dict per layer, here the one layer of
+                      layer_small.npz with the oracle's gradients, laid out by hand from those arrays
 """
 import os
 import sys
@@ -83,8 +87,21 @@ def layer_small():
     np.savez_compressed(os.path.join(HERE, "layer_small.npz"), **out)
 
 
+def states_tiny():
+    z = np.load(os.path.join(HERE, "layer_small.npz"))
+    t = lambda name: torch.from_numpy(z[name]).clone()
+    E = z["w1"].shape[0]
+    experts = [[t("w1")[e], t("b1")[e], t("w2")[e], t("b2")[e]] for e in range(E)]
+    grads = [[t("tanh/g_w1")[e], t("tanh/g_b1")[e], t("tanh/g_w2")[e], t("tanh/g_b2")[e]] for e in range(E)]
+    grads += [t("tanh/dwg"), None]                  # the gate's weight gradient, then its (absent) bias gradient
+    layer = {"gate": [t("wg"), None], "experts": experts, "grad": grads}
+    optim_state = [None, None]                      # [expert_state, gate_state] of an optimizer that has not stepped
+    torch.save([[layer], optim_state], os.path.join(HERE, "MOLE_states_tiny.pt"))
+
+
 if __name__ == "__main__":
     routing_cases()
     layer_small()
-    for f in ("routing_cases.npz", "layer_small.npz"):
+    states_tiny()
+    for f in ("routing_cases.npz", "layer_small.npz", "MOLE_states_tiny.pt"):
         print(f, os.path.getsize(os.path.join(HERE, f)), "bytes")

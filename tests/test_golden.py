@@ -124,3 +124,25 @@ def test_hip_layer_reproduces_layer_fixture(variant):
     assert rel_err(m.gate[0].linear.weight.grad, torch.from_numpy(z[f"{variant}/dwg"])) < 1e-5
     for p, n in ((m.FC1_W_GPU, "g_w1"), (m.FC1_B_GPU, "g_b1"), (m.FC2_W_GPU, "g_w2"), (m.FC2_B_GPU, "g_b2")):
         assert rel_err(p.grad_tensors, torch.from_numpy(z[f"{variant}/{n}"])) < 1e-5, n
+
+
+def test_checkpoint_fixture_has_the_reference_file_layout():
+    """tests/golden/MOLE_states_tiny.pt: [model_state, optim_state] as UniScheduler.save_states writes it
+    (MOLE/utils/Uscheduler.py:67-75), one {"gate", "experts", "grad"} dict per layer (MOLE/moe/layer.py:397-427),
+    readable by a loader that executes nothing from the file, and holding the arrays of layer_small.npz."""
+    all_state = torch.load(os.path.join(GOLD, "MOLE_states_tiny.pt"), map_location="cpu", weights_only=True)
+    z = np.load(os.path.join(GOLD, "layer_small.npz"))
+    assert isinstance(all_state, list) and len(all_state) == 2
+    model_state, optim_state = all_state
+    assert optim_state == [None, None] and len(model_state) == 1
+    st = model_state[0]
+    assert sorted(st) == ["experts", "gate", "grad"]
+    E = z["w1"].shape[0]
+    assert len(st["gate"]) == 2 and st["gate"][1] is None and np.array_equal(st["gate"][0].numpy(), z["wg"])
+    assert len(st["experts"]) == E and len(st["grad"]) == E + 2 and st["grad"][E + 1] is None
+    for e in range(E):
+        for t, name in zip(st["experts"][e], ("w1", "b1", "w2", "b2")):
+            assert np.array_equal(t.numpy(), z[name][e])
+        for t, name in zip(st["grad"][e], ("g_w1", "g_b1", "g_w2", "g_b2")):
+            assert np.array_equal(t.numpy(), z[f"tanh/{name}"][e])
+    assert np.array_equal(st["grad"][E].numpy(), z["tanh/dwg"])

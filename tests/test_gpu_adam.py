@@ -125,3 +125,69 @@ def test_pipeline_adam_offloaded_experts(adamW, hybrid, acc_step, dtype):
         assert torch.equal(t.momentum[n_gpu:], m_start[i][n_gpu:])
         if n_gpu < d:
             assert rel_err(t.grad_[n_gpu:].float(), g_total[n_gpu:]) < (1e-5 if dtype == torch.float32 else 2e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("S", [400, 5])
+@pytest.mark.parametrize("adamW,hybrid,acc_step", [(False, -1, 1), (False, 3, 1), (True, -1, 2), (False, 4, 2)])
+def test_pipeline_adam_with_home_slots_equals_the_stack_run(adamW, hybrid, acc_step, S, dtype):
+    """A pool with a slot for every offloaded expert (each expert keeps a slot of its own from the forward to the
+    backward pass, the update reads the parameters there) against a pool of 3 slots recycled through the prefetch
+    stack: host parameters, moments and gradients are equal bit for bit.  hybrid = 3 cuts a chunk of two experts in
+    the middle; with 5 tokens most experts get no row (their gradient is zero, the optimizer still moves them)."""
+    print(f"pipeline adam home slots adamW={adamW} hybrid={hybrid} acc_step={acc_step} S={S} {dtype}", flush=True)
+    from mole_amd import core
+    M, E, k, Fd, d = 64, 8, 2, 128, 6
+
+    def run(pool):
+        m, x, _ = _build(S, M, E, k, Fd, dtype, d_experts=d, pool=pool, ebatch=2, acc_step=acc_step, adv_adam=True)
+        assert (m.MOLECore._home_base() is not None) == (pool >= d)
+        g_ = torch.Generator().manual_seed(11)
+        for t in _cpu_params(m):
+            t.momentum.copy_(torch.randn(t.shape, generator=g_) * 1e-3)
+            t.variance.copy_(torch.rand(t.shape, generator=g_) * 1e-5)
+            t.grad_.fill_(3.0)               # stale contents: the first micro-step overwrites them
+        m.MOLECore.set_adam(0.9, 0.999, 3, 1e-2, 0.1, 1e-8, adamW, hybrid)
+        for _ in range(acc_step):
+            _step(m, x, dtype)
+        core.synchronize_tran()
+        out = []
+        if S == 5:
+            # experts without rows: their gradient is exactly zero, so the update is the Adam step of a zero
+            # gradient from the moments set above (the weight-gradient kernel writes zeros for an expert without rows)
+            idle = [e for e in range(d) if int(m.last_route.kept_rows[E - d + e]) == 0 and (hybrid == -1 or e < hybrid)]
+            assert idle
+            p0 = _cpu_params_initial(S, M, E, k, Fd, dtype, d, keep=m)
+            g_ = torch.Generator().manual_seed(11)
+            for t, p_init in zip(_cpu_params(m), p0):
+                m_init = torch.randn(t.shape, generator=g_) * 1e-3
+                v_init = torch.rand(t.shape, generator=g_) * 1e-5
+                pe, me, ve = O.adam_step(p_init.float()[idle], m_init[idle], v_init[idle], torch.zeros_like(m_init[idle]),
+                                         0.9, 0.999, 3, 1e-2, 0.1, 1e-8, adamW)
+                assert torch.allclose(t.momentum[idle], me, rtol=1e-5, atol=1e-9)
+                assert torch.allclose(t.variance[idle], ve, rtol=1e-5, atol=1e-12)
+                assert rel_err(t[idle].float(), pe) < (1e-5 if dtype == torch.float32 else 4e-3)
+        for t in _cpu_params(m):
+            out += [t.clone(), t.momentum.clone(), t.variance.clone(), t.grad_.clone()]
+        return out
+
+    want = run(3)
+    got = run(d)
+    names = [f"{p} {w}" for p in ("w1", "b1", "w2", "b2") for w in ("parameter", "momentum", "variance", "gradient")]
+    n_gpu = d if hybrid == -1 else hybrid
+    for name, a, b in zip(names, got, want):
+        if name.endswith("gradient"):
+            # experts updated on the GPU keep whatever their host gradient array held (the update consumed the
+            # gradient on the device); those past the prefix hold the step's gradient
+            a, b = a[n_gpu:], b[n_gpu:]
+        assert torch.equal(a, b), name
+
+
+def _cpu_params_initial(S, M, E, k, Fd, dtype, d, keep):
+    """the offloaded parameters as _build sets them for this seed (drawn again on the host; `keep` is the live
+    layer, whose pool must not be torn down)"""
+    g = torch.Generator().manual_seed(0)
+    torch.randn(S, M, generator=g); torch.randn(E, M, generator=g)
+    w1, b1 = torch.randn(E, Fd, M, generator=g) * 0.02, torch.randn(E, Fd, generator=g) * 0.02
+    w2, b2 = torch.randn(E, Fd, M, generator=g) * 0.02, torch.randn(E, M, generator=g) * 0.02
+    return [t[E - d:].to(dtype) for t in (w1, b1, w2, b2)]

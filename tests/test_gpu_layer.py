@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from oracle import moe_oracle as O
-from tests.util import rel_err, tol
+from tests.util import expert_rel_err, rel_err, row_rel_err, tol
 
 pytestmark = pytest.mark.gpu
 
@@ -74,11 +74,13 @@ def _run_and_compare(m, x, ref, k, cf, dtype, gelu_bwd="tanh", normalize=True, a
     assert rel_err(y, res.y) < t
     assert rel_err(x.grad, res.dx) < t
     assert rel_err(m.gate[0].linear.weight.grad, res.dwg) < t
-    g_w1, g_b1, g_w2, g_b2 = _grads(m, ref["w1"].shape[0])
-    assert rel_err(g_w1, res.g_w1) < t
-    assert rel_err(g_b1, res.g_b1) < t
-    assert rel_err(g_w2, res.g_w2) < t
-    assert rel_err(g_b2, res.g_b2) < t
+    # the four expert gradients, every expert against its own largest element (an expert with few rows has small
+    # gradients: one maximum over all experts would let it be wrong by any factor)
+    for name, got, want in zip(("g_w1", "g_b1", "g_w2", "g_b2"), _grads(m, ref["w1"].shape[0]),
+                               (res.g_w1, res.g_b1, res.g_w2, res.g_b2)):
+        err = expert_rel_err(got, want)
+        assert err < t, f"{name}: worst expert off by {err:.2e}"
+        res.extras[name + "_gpu"] = got
     assert abs(float(m.l_aux.detach()) - res.crit.l_aux) < 1e-4 * max(1.0, res.crit.l_aux)
     res.extras["y_gpu"], res.extras["dx_gpu"] = y.detach(), x.grad
     return res
@@ -221,7 +223,6 @@ def test_layer_config1_exact():
     """BASELINE config 1 as specified: 4096 x 512 fp32, 8 experts, top-2, F = 2048, N(0, 0.02) weights,
     MSE against zero, seed 0; with the reference's default capacity factor and without dropping.  Besides the
     max-norm tolerance, every row of y and dx is held to it relative to the row's own largest element."""
-    from tests.util import row_rel_err
     for cf in (1.0, 0.0):
         print(f"layer config1 cf={cf}", flush=True)
         m, x, ref = _build(4096, 512, 8, 2, 2048, torch.float32, seed=0)
@@ -229,6 +230,11 @@ def test_layer_config1_exact():
         ry, rdx = row_rel_err(res.extras["y_gpu"], res.y), row_rel_err(res.extras["dx_gpu"], res.dx)
         print(f"layer config1 cf={cf}: per-row relative error y {ry:.2e}, dx {rdx:.2e}", flush=True)
         assert ry < 1e-5 and rdx < 1e-5
+        # the two weight gradients row by row: row (e, f) of g_w1 and of g_w2 against its own largest element
+        rw1 = row_rel_err(res.extras["g_w1_gpu"], res.g_w1)
+        rw2 = row_rel_err(res.extras["g_w2_gpu"], res.g_w2)
+        print(f"layer config1 cf={cf}: per-row relative error g_w1 {rw1:.2e}, g_w2 {rw2:.2e}", flush=True)
+        assert rw1 < 1e-5 and rw2 < 1e-5
 
 
 def _near_tie_report(scores64, idx_gpu, idx_cpu, k, bound):
@@ -237,7 +243,9 @@ def _near_tie_report(scores64, idx_gpu, idx_cpu, k, bound):
     diff = (idx_gpu != idx_cpu).any(axis=0).nonzero()[0]
     for i in diff:
         a, b = idx_gpu[:, i], idx_cpu[:, i]
-        involved = sorted(set(a.tolist()) ^ set(b.tolist())) or sorted(set(a.tolist()))   # same set, other order
+        # the experts at the choice positions where the two sides differ: another expert chosen, or the same experts
+        # in another order
+        involved = sorted(set(a[a != b].tolist()) | set(b[a != b].tolist()))
         vals = scores64[i, involved]
         assert float(vals.max() - vals.min()) <= bound * float(vals.max()), \
             f"token {i}: GPU chose {a.tolist()}, oracle {b.tolist()}, scores {scores64[i, sorted(set(a.tolist()) | set(b.tolist()))]}"
@@ -245,7 +253,9 @@ def _near_tie_report(scores64, idx_gpu, idx_cpu, k, bound):
 
 
 @pytest.mark.parametrize("name,S,M,E,k,cf,dtype", [("c1", 4096, 512, 8, 2, 1.0, torch.float32),
-                                                   ("c2", 16384, 1024, 16, 1, 1.25, torch.bfloat16)])
+                                                   ("c2", 16384, 1024, 16, 1, 1.25, torch.bfloat16),
+                                                   ("c3", 8192, 2048, 64, 2, 0.0, torch.bfloat16),
+                                                   ("c5", 32768, 2048, 256, 8, 0.0, torch.bfloat16)])
 def test_routing_from_tokens_matches_oracle(name, S, M, E, k, cf, dtype):
     """Routing end to end from x (gate product, softmax, top-k, locations, capacity, permutation) against the
     oracle run on the same seeded x and Wg with no help from the GPU's scores.  The two gates sum their products
@@ -257,27 +267,42 @@ def test_routing_from_tokens_matches_oracle(name, S, M, E, k, cf, dtype):
     print(f"routing from tokens {name}", flush=True)
     g = torch.Generator().manual_seed(0)
     x = torch.randn(S, M, generator=g)
-    wg = torch.randn(E, M, generator=g) * 0.02
+    # c5 is specified with N(0,1) gate logits (the two-kernel gate of 256 experts, top-8: near ties are likeliest
+    # there), c3 with a Zipf(1.2) per-expert logit bias over a random ranking of the experts
+    wg = torch.randn(E, M, generator=g) * (1.0 / M ** 0.5 if name == "c5" else 0.02)
+    bias = torch.log((torch.randperm(E, generator=g).float() + 1.0) ** -1.2) if name == "c3" else None
     xr = x.to(dtype)
     wr = wg if dtype == torch.float32 else wg.bfloat16().float()      # the bf16 gate kernel rounds Wg
-    scores_gpu = Ugate.gate_scores(xr.cuda(), wg.cuda())
+    scores_gpu = Ugate.gate_scores(xr.cuda(), wg.cuda(), None if bias is None else bias.cuda())
     r = H.route(scores_gpu, k, cf)
-    scores_cpu = O.gate_scores(xr.float(), wr)
+    scores_cpu = O.gate_scores(xr.float(), wr, bias)
     c = O.extract_critical(scores_cpu.numpy(), k, cf)
     idx_gpu, idx_cpu = r.idx.cpu().numpy(), np.stack(c.indices_s)
-    scores64 = torch.softmax(xr.double() @ wr.double().t(), dim=-1).numpy()
-    # a few ulp of fp32 relative to the score
-    flips = _near_tie_report(scores64, idx_gpu, idx_cpu, k, bound=8 * 1.2e-7)
+    logits64 = xr.double() @ wr.double().t()
+    scores64 = torch.softmax(logits64 if bias is None else logits64 + bias.double(), dim=-1).numpy()
+    # a few ulp of fp32 relative to the score.  An absolute difference d between two sums for the same logit is a
+    # relative difference d of the score; c5's logits have unit variance and 2048 terms, so its two summation
+    # orders differ by a few 1e-7 absolute where the other configurations' (logits of variance 0.02^2 M) stay below 1e-7
+    flips = _near_tie_report(scores64, idx_gpu, idx_cpu, k, bound=(32 if name == "c5" else 8) * 1.2e-7)
     print(f"routing from tokens {name}: {flips} of {S} tokens routed differently (near ties)", flush=True)
-    assert flips <= 2
-    if flips == 0:
-        np.testing.assert_array_equal(idx_gpu, idx_cpu)
-        np.testing.assert_array_equal(r.counts.cpu().numpy(), c.counts)
-        np.testing.assert_array_equal(r.loc.cpu().numpy(), np.stack(c.locations_s))
-        np.testing.assert_array_equal(r.row.cpu().numpy(), c.rows(True))
-        np.testing.assert_array_equal(r.kept_rows.cpu().numpy(), c.kept_rows)
-        assert int(r.capacity.cpu()) == c.capacity
-        assert rel_err(r.gates.cpu(), torch.from_numpy(np.stack(c.gates_s))) < 1e-5
+    # with k choices out of E there are k orderings per token that a last-bit difference can turn: at top-8 of 256
+    # a handful of the 32768 tokens is expected, at top-1 and top-2 none or one
+    assert flips <= (2 if k <= 2 else 24)
+    if flips:
+        # the oracle once more, with the GPU's scores for exactly the near-tie tokens and its own for all others:
+        # everything downstream of those few decisions must then agree as well
+        diff = (idx_gpu != idx_cpu).any(axis=0).nonzero()[0]
+        mixed = scores_cpu.numpy().copy()
+        mixed[diff] = scores_gpu.cpu().numpy()[diff]
+        c = O.extract_critical(mixed, k, cf)
+        idx_cpu = np.stack(c.indices_s)
+    np.testing.assert_array_equal(idx_gpu, idx_cpu)
+    np.testing.assert_array_equal(r.counts.cpu().numpy(), c.counts)
+    np.testing.assert_array_equal(r.loc.cpu().numpy(), np.stack(c.locations_s))
+    np.testing.assert_array_equal(r.row.cpu().numpy(), c.rows(True))
+    np.testing.assert_array_equal(r.kept_rows.cpu().numpy(), c.kept_rows)
+    assert int(r.capacity.cpu()) == c.capacity
+    assert rel_err(r.gates.cpu(), torch.from_numpy(np.stack(c.gates_s))) < 1e-5
 
 
 def test_layer_gelu_exact_switch_and_gate_bias():

@@ -36,6 +36,21 @@ def row_rel_err(got: torch.Tensor, want: torch.Tensor) -> float:
     return float(torch.where(mag > 0, diff / mag.clamp_min(1e-300), diff).max())
 
 
+def expert_rel_err(got: torch.Tensor, want: torch.Tensor) -> float:
+    """max over experts e of max |got[e] - want[e]| / max |want[e]| for [E, ...] parameter gradients: every expert
+    is held to the tolerance relative to its own largest gradient, so that an expert with few rows and small
+    gradients cannot hide behind a loaded one.  An expert whose reference gradient is all zero (no rows) counts
+    with its absolute error."""
+    E = want.shape[0]
+    got = got.detach().double().cpu().reshape(E, -1)
+    want = want.detach().double().cpu().reshape(E, -1)
+    if want.numel() == 0:
+        return 0.0
+    diff = (got - want).abs().amax(dim=1)
+    mag = want.abs().amax(dim=1)
+    return float(torch.where(mag > 0, diff / mag.clamp_min(1e-300), diff).max())
+
+
 FP32_TOL = 1e-5
 BF16_TOL = 2e-2
 
