@@ -79,37 +79,59 @@ __device__ __forceinline__ void load_rows(const int32_t *__restrict__ row, int S
     }
 }
 
-template <typename T, int K>
+// TPW tokens per wave: the row indices of all of a wave's tokens come first, then the loads of all their rows' pieces,
+// then the stores.  A wave that owns a single token with a single choice has little in flight and pays the index
+// latency once per row.
+template <int K, int TPW>
+__device__ __forceinline__ void load_rows_multi(const int32_t *__restrict__ row, int S, int k, int i0, int (&r)[TPW][K],
+                                                uint32_t (&keep)[TPW][K]) {
+#pragma unroll
+    for (int t = 0; t < TPW; ++t)
+#pragma unroll
+        for (int j = 0; j < K; ++j) r[t][j] = row[(size_t)min(j, k - 1) * S + min(i0 + t, S - 1)];      // all loads first
+#pragma unroll
+    for (int t = 0; t < TPW; ++t)
+#pragma unroll
+        for (int j = 0; j < K; ++j) {
+            keep[t][j] = (j < k && i0 + t < S && r[t][j] >= 0) ? 0xffffffffu : 0u;
+            r[t][j] &= (int)keep[t][j];
+        }
+}
+
+template <typename T, int K, int TPW>
 __global__ __launch_bounds__(PM_THREADS) void dispatch_fwd_kernel(const T *__restrict__ x,
                                                                   const int32_t *__restrict__ row, int S, int M,
                                                                   int k, T *__restrict__ xd) {
-    const int i = blockIdx.x * (PM_THREADS / WAVE) + (threadIdx.x >> 6);
-    if (i >= S) return;
+    const int i0 = (blockIdx.x * (PM_THREADS / WAVE) + (threadIdx.x >> 6)) * TPW;
+    if (i0 >= S) return;
     const int lane = lane_id();
-    int r[K];
-    uint32_t keep[K];
-    load_rows<K>(row, S, k, i, r, keep);
+    int r[TPW][K];
+    uint32_t keep[TPW][K];
+    load_rows_multi<K, TPW>(row, S, k, i0, r, keep);
     constexpr int N = Vec<T>::N;
-    constexpr int U = 2 * PM_U;                  // one source row: more of its chunks in flight
+    constexpr int U = TPW > 1 ? PM_U : 2 * PM_U;                  // one source row: more of its chunks in flight
     const int chunks = M / N;
-    const T *src = x + (size_t)i * M;
     for (int c0 = lane; c0 < chunks; c0 += U * WAVE) {
-        Vec<T> v[U];
+        Vec<T> v[TPW][U];
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int c = c0 + u * WAVE;
-            v[u].load(src + (size_t)(c < chunks ? c : c0) * N);
-        }
+        for (int t = 0; t < TPW; ++t)
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int c = c0 + u * WAVE;
-            v[u].pin();
-            if (c < chunks) {
-#pragma unroll
-                for (int j = 0; j < K; ++j)
-                    if (keep[j]) v[u].store(xd + (size_t)r[j] * M + (size_t)c * N);
+            for (int u = 0; u < U; ++u) {
+                const int c = c0 + u * WAVE;
+                v[t][u].load(x + (size_t)min(i0 + t, S - 1) * M + (size_t)(c < chunks ? c : c0) * N);
             }
-        }
+#pragma unroll
+        for (int t = 0; t < TPW; ++t)
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int c = c0 + u * WAVE;
+                v[t][u].pin();
+                if (c < chunks) {
+#pragma unroll
+                    for (int j = 0; j < K; ++j)
+                        if (keep[t][j]) v[t][u].store(xd + (size_t)r[t][j] * M + (size_t)c * N);
+                }
+            }
     }
 }
 
@@ -706,51 +728,57 @@ __global__ __launch_bounds__(256) void gate_wgrad_reduce_kernel(const float *__r
     }
 }
 
-template <typename T, int K>
+template <typename T, int K, int TPW>
 __global__ __launch_bounds__(PM_THREADS) void combine_fwd_kernel(const T *__restrict__ o,
                                                                  const int32_t *__restrict__ row,
                                                                  const float *__restrict__ gates, int S, int M,
                                                                  int k, T *__restrict__ y) {
-    const int i = blockIdx.x * (PM_THREADS / WAVE) + (threadIdx.x >> 6);
-    if (i >= S) return;
+    const int i0 = (blockIdx.x * (PM_THREADS / WAVE) + (threadIdx.x >> 6)) * TPW;
+    if (i0 >= S) return;
     const int lane = lane_id();
-    int r[K];
-    uint32_t keep[K];
-    float g[K];
-    load_rows<K>(row, S, k, i, r, keep);
+    int r[TPW][K];
+    uint32_t keep[TPW][K];
+    float g[TPW][K];
+    load_rows_multi<K, TPW>(row, S, k, i0, r, keep);
 #pragma unroll
-    for (int j = 0; j < K; ++j) g[j] = gates[(size_t)min(j, k - 1) * S + i];
+    for (int t = 0; t < TPW; ++t)
+#pragma unroll
+        for (int j = 0; j < K; ++j) g[t][j] = gates[(size_t)min(j, k - 1) * S + min(i0 + t, S - 1)];
     constexpr int N = Vec<T>::N;
     constexpr int U = K >= 16 ? 1 : PM_U;
     const int chunks = M / N;
     for (int c0 = lane; c0 < chunks; c0 += U * WAVE) {
-        Vec<T> v[U][K];
+        Vec<T> v[TPW][U][K];
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int c = c0 + u * WAVE;
-            const size_t off = (size_t)(c < chunks ? c : c0) * N;
+        for (int t = 0; t < TPW; ++t)
 #pragma unroll
-            for (int j = 0; j < K; ++j) v[u][j].load(o + (size_t)r[j] * M + off);
-        }
+            for (int u = 0; u < U; ++u) {
+                const int c = c0 + u * WAVE;
+                const size_t off = (size_t)(c < chunks ? c : c0) * N;
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int c = c0 + u * WAVE;
-            if (c >= chunks) continue;
-            float acc[N], f[N];
-#pragma unroll
-            for (int q = 0; q < N; ++q) acc[q] = 0.f;
-#pragma unroll
-            for (int j = 0; j < K; ++j) {
-                v[u][j].mask(keep[j]);         // a slot that does not count contributes g * (+0)
-                v[u][j].unpack(f);
-                const float gj = __uint_as_float(__float_as_uint(g[j]) & keep[j]);
-#pragma unroll
-                for (int q = 0; q < N; ++q) acc[q] += gj * f[q];
+                for (int j = 0; j < K; ++j) v[t][u][j].load(o + (size_t)r[t][j] * M + off);
             }
-            Vec<T> out;
-            out.pack(acc);
-            out.store(y + (size_t)i * M + (size_t)c * N);
-        }
+#pragma unroll
+        for (int t = 0; t < TPW; ++t)
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int c = c0 + u * WAVE;
+                if (c >= chunks || i0 + t >= S) continue;
+                float acc[N], f[N];
+#pragma unroll
+                for (int q = 0; q < N; ++q) acc[q] = 0.f;
+#pragma unroll
+                for (int j = 0; j < K; ++j) {
+                    v[t][u][j].mask(keep[t][j]);         // a slot that does not count contributes g * (+0)
+                    v[t][u][j].unpack(f);
+                    const float gj = __uint_as_float(__float_as_uint(g[t][j]) & keep[t][j]);
+#pragma unroll
+                    for (int q = 0; q < N; ++q) acc[q] += gj * f[q];
+                }
+                Vec<T> out;
+                out.pack(acc);
+                out.store(y + (size_t)(i0 + t) * M + (size_t)c * N);
+            }
     }
 }
 
@@ -842,7 +870,32 @@ static int check_perm(const char *fn, int dtype, int S, int M, int k) {
 }
 static bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
-// the kernels above for the smallest K in {1, 2, 4, 8, 16} that holds k
+// The wave-per-token kernels for the smallest K in {1, 2, 4, 8, 16} that holds k.  The scatter and the gather take
+// several tokens per wave when there is one choice per token (TPW1: 8 for the scatter, whose source rows follow one
+// another in memory - 16 loads in flight; 4 for the gather - 8 in flight; measured at 16384 x 1024 bf16: 11.5 -> 9.0-9.7 us
+// and 12.0 -> 11.3 us, slower again with more and, at two choices per token, with any), as long as that leaves two
+// blocks for every CU.  The combine backward measured best with one token per wave (two: 19.2 against 18.8 us,
+// four: 20.9) and keeps the one-token kernel.
+static int perm_tpw(int S, int k, int tpw1) {
+    int tpw = k <= 1 && tpw1 > 1 ? tpw1 : 1;
+    while (tpw > 1 && ceil_div(S, (PM_THREADS / WAVE) * tpw) < 512) tpw >>= 1;
+    return tpw;
+}
+#define PM_LAUNCH_KT(KID, KERNEL, T, TPW1, ...)                                                                   \
+    do {                                                                                                         \
+        const dim3 blk_(PM_THREADS);                                                                             \
+        const int tpw_ = perm_tpw(S, k, TPW1);                                                                   \
+        const dim3 grid_(ceil_div(S, (PM_THREADS / WAVE) * tpw_));                                               \
+        if (k <= 1 && tpw_ == 8) timed_launch(KID, KERNEL<T, 1, (TPW1 >= 8 ? 8 : 1)>, grid_, blk_, 0, (hipStream_t)stream, __VA_ARGS__);   \
+        else if (k <= 1 && tpw_ == 4) timed_launch(KID, KERNEL<T, 1, (TPW1 >= 4 ? 4 : 1)>, grid_, blk_, 0, (hipStream_t)stream, __VA_ARGS__); \
+        else if (k <= 1 && tpw_ == 2) timed_launch(KID, KERNEL<T, 1, (TPW1 >= 2 ? 2 : 1)>, grid_, blk_, 0, (hipStream_t)stream, __VA_ARGS__); \
+        else if (k <= 1) timed_launch(KID, KERNEL<T, 1, 1>, grid_, blk_, 0, (hipStream_t)stream, __VA_ARGS__);   \
+        else if (k <= 2) timed_launch(KID, KERNEL<T, 2, 1>, grid_, blk_, 0, (hipStream_t)stream, __VA_ARGS__);   \
+        else if (k <= 4) timed_launch(KID, KERNEL<T, 4, 1>, grid_, blk_, 0, (hipStream_t)stream, __VA_ARGS__);   \
+        else if (k <= 8) timed_launch(KID, KERNEL<T, 8, 1>, grid_, blk_, 0, (hipStream_t)stream, __VA_ARGS__);   \
+        else timed_launch(KID, KERNEL<T, 16, 1>, grid_, blk_, 0, (hipStream_t)stream, __VA_ARGS__);              \
+    } while (0)
+// one token per wave
 #define PM_LAUNCH_K(KID, KERNEL, T, ...)                                                                         \
     do {                                                                                                         \
         const dim3 blk_(PM_THREADS);                                                                             \
@@ -862,11 +915,10 @@ extern "C" int mole_dispatch_fwd(const void *x, int dtype, const int32_t *row, i
     if (int rc = check_perm("mole_dispatch_fwd", dtype, S, M, k)) return rc;
     if (S == 0) return 0;
     MOLE_REQUIRE(x && row && xd && aligned16(x) && aligned16(xd), "mole_dispatch_fwd: null or misaligned pointer");
-    const dim3 grid(ceil_div(S, PM_THREADS / WAVE));
     if (dtype == MOLE_BF16)
-        PM_LAUNCH_K(MOLE_K_DISPATCH_FWD, dispatch_fwd_kernel, bf16_t, (const bf16_t *)x, row, S, M, k, (bf16_t *)xd);
+        PM_LAUNCH_KT(MOLE_K_DISPATCH_FWD, dispatch_fwd_kernel, bf16_t, 8, (const bf16_t *)x, row, S, M, k, (bf16_t *)xd);
     else
-        PM_LAUNCH_K(MOLE_K_DISPATCH_FWD, dispatch_fwd_kernel, float, (const float *)x, row, S, M, k, (float *)xd);
+        PM_LAUNCH_KT(MOLE_K_DISPATCH_FWD, dispatch_fwd_kernel, float, 8, (const float *)x, row, S, M, k, (float *)xd);
     MOLE_LAUNCH_CHECK();
     return 0;
 }
@@ -982,11 +1034,10 @@ extern "C" int mole_combine_fwd(const void *o, int dtype, const int32_t *row, co
     if (int rc = check_perm("mole_combine_fwd", dtype, S, M, k)) return rc;
     if (S == 0) return 0;
     MOLE_REQUIRE(o && row && gates && y && aligned16(o) && aligned16(y), "mole_combine_fwd: null or misaligned pointer");
-    const dim3 grid(ceil_div(S, PM_THREADS / WAVE));
     if (dtype == MOLE_BF16)
-        PM_LAUNCH_K(MOLE_K_COMBINE_FWD, combine_fwd_kernel, bf16_t, (const bf16_t *)o, row, gates, S, M, k, (bf16_t *)y);
+        PM_LAUNCH_KT(MOLE_K_COMBINE_FWD, combine_fwd_kernel, bf16_t, 4, (const bf16_t *)o, row, gates, S, M, k, (bf16_t *)y);
     else
-        PM_LAUNCH_K(MOLE_K_COMBINE_FWD, combine_fwd_kernel, float, (const float *)o, row, gates, S, M, k, (float *)y);
+        PM_LAUNCH_KT(MOLE_K_COMBINE_FWD, combine_fwd_kernel, float, 4, (const float *)o, row, gates, S, M, k, (float *)y);
     MOLE_LAUNCH_CHECK();
     return 0;
 }

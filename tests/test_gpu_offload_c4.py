@@ -135,7 +135,9 @@ def test_c4_layer_parity_prefetch_and_overlap(layer):
     frac = busy_ms * 1e-3 / wall
     print(f"c4: prefetched step {wall * 1e3:.1f} ms, copy stream busy {busy_ms:.1f} ms ({frac:.2f}), "
           f"{nbytes1 / (busy_ms * 1e-3) / 1e9:.1f} GB/s host to device", flush=True)
-    assert frac >= 0.8
+    # (copy-stream busy time over host wall-clock time: 0.84-0.92 on an idle box; the floor is loose because a
+    # loaded host stretches the wall-clock side without any change in the code)
+    assert frac >= 0.5
     del res
 
     print("c4: fp32 restatement on the GPU", flush=True)

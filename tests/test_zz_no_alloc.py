@@ -56,6 +56,24 @@ def test_route_static_matches_route_on_consecutive_calls():
                 np.testing.assert_array_equal(got[name], want[name], err_msg=f"{name} of case {n}")
 
 
+def test_route_static_allocates_nothing():
+    """Device memory in use is the same before and after calls of the entry point (outputs allocated beforehand)."""
+    from mole_amd import _lib as L
+    S, E, k = 4096, 64, 2
+    scores = zipf_scores(S, E, seed=3).cuda()
+    b = _buffers(S, E, k)
+    args = [L.ptr(scores), S, E, k, 0.0, 1, 1, L.LAYOUT_RAGGED] + [L.ptr(b[n]) for n in OUTS]
+    L.check(L.lib().mole_route_static(*args, L.stream()), "mole_route_static")      # first call on the device: set-up
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    reserved0 = torch.cuda.memory_reserved()
+    for _ in range(3):
+        L.check(L.lib().mole_route_static(*args, L.stream()), "mole_route_static")
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0 and torch.cuda.memory_reserved() == reserved0
+
+
 def test_route_static_rejects_what_does_not_fit():
     from mole_amd import _lib as L
     S, E, k = 200000, 512, 8
