@@ -146,23 +146,26 @@ __device__ __forceinline__ void mma_step(const char *ldsA, const char *ldsB, int
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn)
             b[tn] = *reinterpret_cast<const uint4 *>(ldsB + lds_off(rowB0 + tn * 32 + lr, 2 * kk + h));
+        if constexpr (sizeof(T) == 2) {
 #pragma unroll
-        for (int tm = 0; tm < TM; ++tm)
+            for (int tm = 0; tm < TM; ++tm)
 #pragma unroll
-            for (int tn = 0; tn < TN; ++tn) {
-                if constexpr (sizeof(T) == 2) {
+                for (int tn = 0; tn < TN; ++tn)
                     acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
                         __builtin_bit_cast(bf16x8, a[tm]), __builtin_bit_cast(bf16x8, b[tn]), acc[tm][tn], 0, 0, 0);
-                } else {
-                    const float af[4] = {__uint_as_float(a[tm].x), __uint_as_float(a[tm].y),
-                                         __uint_as_float(a[tm].z), __uint_as_float(a[tm].w)};
-                    const float bf[4] = {__uint_as_float(b[tn].x), __uint_as_float(b[tn].y),
-                                         __uint_as_float(b[tn].z), __uint_as_float(b[tn].w)};
+        } else {
+            // the four k of a 16-byte fragment, the cells of the wave tile innermost: consecutive MFMAs write
+            // different accumulators
 #pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[j], bf[j], acc[tm][tn], 0, 0, 0);
-                }
-            }
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+                    for (int tn = 0; tn < TN; ++tn) {
+                        const uint32_t aw[4] = {a[tm].x, a[tm].y, a[tm].z, a[tm].w}, bw[4] = {b[tn].x, b[tn].y, b[tn].z, b[tn].w};
+                        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(aw[j]), __uint_as_float(bw[j]), acc[tm][tn], 0, 0, 0);
+                    }
+        }
     }
 }
 
