@@ -316,6 +316,17 @@ template <int TMB, int WM, bool M_KS, bool N_KS, bool WG, int TMC> struct Feeder
     }
 };
 
+__device__ __forceinline__ uint2 pack4(float a, float b, float c, float d) {
+    const bf16x4 v = {(bf16_t)a, (bf16_t)b, (bf16_t)c, (bf16_t)d};
+    return __builtin_bit_cast(uint2, v);
+}
+__device__ __forceinline__ void unpack4(uint2 u, float *f) {
+    f[0] = __uint_as_float(u.x << 16);
+    f[1] = __uint_as_float(u.x & 0xffff0000u);
+    f[2] = __uint_as_float(u.y << 16);
+    f[3] = __uint_as_float(u.y & 0xffff0000u);
+}
+
 // The K loop.  Stage s (32 of K) lives in ring buffer s mod NSTAGE and is fetched NSTAGE-1 stages ahead.
 // A wave cannot issue MFMAs while one of its loads waits for the memory pipeline to take it, so the loads
 // of a stage are not issued in one burst: each half of an iteration is cut into parts, and a part issues
@@ -326,10 +337,13 @@ template <int TMB, int WM, bool M_KS, bool N_KS, bool WG, int TMC> struct Feeder
 // still be in flight), then the barrier.
 // PART (measurement only, results are then meaningless): 1 leaves out the operand loads, 2 the fragment reads of the
 // loop (the first stage's fragments are used throughout), 3 the barriers, 4 all three.
-template <int TMB, int WM, bool M_KS, bool N_KS, bool WG, int TMC, int TMCW, int SUM, int PART = 0>
+// BIAS: the accumulators start from the bias of their columns instead of zero (bias_raw: the 8 x 4 columns a lane
+// holds, fetched before the operand loads and therefore landed when the first stage has), so that the epilogue adds
+// nothing.
+template <int TMB, int WM, bool M_KS, bool N_KS, bool WG, int TMC, int TMCW, int SUM, int PART = 0, bool BIAS = false>
 __device__ __forceinline__ void main_loop(const bf16_t *Mp, long ldm, int m0, int m_ext, const bf16_t *Np, long ldn,
                                           int n0, int n_ext, int k_ext, char *smem, int wave, int wm, int wn,
-                                          f32x16 (&acc)[Tile<TMB, WM>::TMW][2], f32x16 &sums) {
+                                          f32x16 (&acc)[Tile<TMB, WM>::TMW][2], f32x16 &sums, const uint2 (&bias_raw)[8]) {
     typedef Tile<TMB, WM> TL;
     typedef Stage<TMB, WM, M_KS, TMC> SG;
     constexpr int AHEAD = SG::NSTAGE - 1, NP = 4;
@@ -358,6 +372,17 @@ __device__ __forceinline__ void main_loop(const bf16_t *Mp, long ldm, int m0, in
     }
     __builtin_amdgcn_s_waitcnt(waitcnt_vm((AHEAD - 2) * L + (SPLIT ? LH : L)));
     __builtin_amdgcn_s_barrier();
+    if constexpr (BIAS) {
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            float b4[4];
+            unpack4(bias_raw[c], b4);
+#pragma unroll
+            for (int tm = 0; tm < TMCW; ++tm)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[tm][c >> 2][4 * (c & 3) + j] = b4[j];
+        }
+    }
     fix_tail(0, 0);
     Frags<TMB, WM, M_KS, N_KS, TMC, TMCW> f0, f1;
     f0.read(smem, wm, wn, 0);
@@ -390,17 +415,6 @@ __device__ __forceinline__ void main_loop(const bf16_t *Mp, long ldm, int m0, in
         cur_b = nxt_b;
     }
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));   // nothing may still be writing LDS when the block retires
-}
-
-__device__ __forceinline__ uint2 pack4(float a, float b, float c, float d) {
-    const bf16x4 v = {(bf16_t)a, (bf16_t)b, (bf16_t)c, (bf16_t)d};
-    return __builtin_bit_cast(uint2, v);
-}
-__device__ __forceinline__ void unpack4(uint2 u, float *f) {
-    f[0] = __uint_as_float(u.x << 16);
-    f[1] = __uint_as_float(u.x & 0xffff0000u);
-    f[2] = __uint_as_float(u.y << 16);
-    f[3] = __uint_as_float(u.y & 0xffff0000u);
 }
 
 // The bias of the 8 x 4 columns a lane holds results for, as raw bf16 quadruples; fetched before the K loop
@@ -577,21 +591,14 @@ __device__ __forceinline__ void epilogue(const GemmArgs &g, f32x16 (&acc)[Tile<T
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const int n = nw0 + tn * 32 + 8 * q + 4 * h;
-                float bias[4] = {0.f, 0.f, 0.f, 0.f};
-                if constexpr (EPI == EPI_BIAS || EPI == EPI_BIAS_GELU) unpack4(bias_raw[tn * 4 + q], bias);
-                (void)n;
+                (void)n;          // (the bias is in the accumulators already: the K loop started from it)
 #pragma unroll
                 for (int tm = 0; tm < TMC; ++tm) {
                     char *cell = slab_at(tm * 32 + lm, tn * 4 + q, h);
                     float v[4];
 #pragma unroll
                     for (int j = 0; j < 4; ++j) v[j] = acc[tm][tn][4 * q + j];
-                    if constexpr (EPI == EPI_BIAS) {
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) v[j] += bias[j];
-                    } else if constexpr (EPI == EPI_BIAS_GELU) {
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) v[j] += bias[j];
+                    if constexpr (EPI == EPI_BIAS_GELU) {
                         if (pass == 1) {
 #pragma unroll
                             for (int j = 0; j < 4; ++j) v[j] = fast_gelu_erf(v[j]);
@@ -845,7 +852,7 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
     for (int q = 0; q < 16; ++q) sums[q] = 0.f;
 #define MOLE_RUN_TILE_SUM(C, SUM)                                                                                         \
     {                                                                                                                     \
-        main_loop<TMB, WM, M_KS, N_KS, WG, WM *(C), (C), SUM, (EPI > EPI_NONE ? EPI - EPI_NONE : 0)>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wu, wm, wn, acc, sums); \
+        main_loop<TMB, WM, M_KS, N_KS, WG, WM *(C), (C), SUM, (EPI > EPI_NONE ? EPI - EPI_NONE : 0), (EPI == EPI_BIAS || EPI == EPI_BIAS_GELU)>(Mp, g.lda, m0, m_ext, Np, g.ldb, n0, g.N, k_ext, smem, wu, wm, wn, acc, sums, bias_raw); \
         if constexpr (SUM != 0) store_sums<SUM, (C)>(g, sums, e, m0, n0, m_ext, wm, wn, lane);                            \
         epilogue<TMB, WM, WG, EPI, (C)>(g, acc, smem, lane, wu, wn, e, row0, m0w, n0, m_ext, live_w, bias_raw);      \
     }
