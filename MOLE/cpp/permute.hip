@@ -792,18 +792,16 @@ __global__ __launch_bounds__(PM_THREADS) void combine_fwd_kernel(const T *__rest
     }
 }
 
+// The row streaming of the combine backward for token i: d_o[row_j] = g_j dy[i], and the k dot products <dy[i], o[row_j]>
+// summed over the wave (every lane ends up with all of them).
 template <typename T, int K>
-__global__ __launch_bounds__(PM_THREADS) void combine_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ o,
-                                                                 const int32_t *__restrict__ row,
-                                                                 const float *__restrict__ gates, int S, int M,
-                                                                 int k, T *__restrict__ d_o,
-                                                                 float *__restrict__ dgates) {
-    const int i = blockIdx.x * (PM_THREADS / WAVE) + (threadIdx.x >> 6);
-    if (i >= S) return;
+__device__ __forceinline__ void combine_bwd_rows(const T *__restrict__ dy, const T *__restrict__ o,
+                                                 const int32_t *__restrict__ row, const float *__restrict__ gates, int S,
+                                                 int M, int k, int i, T *__restrict__ d_o, float (&dot)[K]) {
     const int lane = lane_id();
     int r[K];
     uint32_t keep[K];
-    float g[K], dot[K];
+    float g[K];
     load_rows<K>(row, S, k, i, r, keep);
 #pragma unroll
     for (int j = 0; j < K; ++j) {
@@ -851,9 +849,105 @@ __global__ __launch_bounds__(PM_THREADS) void combine_bwd_kernel(const T *__rest
         }
     }
 #pragma unroll
-    for (int j = 0; j < K; ++j) {
-        const float d = wave_sum(dot[j]);
-        if (lane == 0 && j < k) dgates[(size_t)j * S + i] = d;
+    for (int j = 0; j < K; ++j) dot[j] = wave_sum(dot[j]);
+}
+
+template <typename T, int K>
+__global__ __launch_bounds__(PM_THREADS) void combine_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ o,
+                                                                 const int32_t *__restrict__ row,
+                                                                 const float *__restrict__ gates, int S, int M,
+                                                                 int k, T *__restrict__ d_o,
+                                                                 float *__restrict__ dgates) {
+    const int i = blockIdx.x * (PM_THREADS / WAVE) + (threadIdx.x >> 6);
+    if (i >= S) return;
+    float dot[K];
+    combine_bwd_rows<T, K>(dy, o, row, gates, S, M, k, i, d_o, dot);
+#pragma unroll
+    for (int j = 0; j < K; ++j)
+        if (lane_id() == 0 && j < k) dgates[(size_t)j * S + i] = dot[j];
+}
+
+// The combine backward with the gate's backward in its tail: the k gate gradients of a token never leave the wave
+// that formed them.  From them: the gradient of the raw gate values through the normalisation gate_j = graw_j /
+// max(sum graw, eps), scattered to the chosen experts' scores, plus the load-balancing loss's term when counts0 and
+// d_l_aux are given, then through the softmax.  Lane l holds experts l, l + 64, ... (VPL of them); the token's score
+// row and indices are requested before the rows are streamed, so the tail waits for no memory.
+struct GateBwdArgs {
+    const float *scores;      // [S,E]
+    const int32_t *idx;       // [k,S]
+    int E, normalize, through_softmax;
+    const int32_t *counts0;   // [E] or null
+    const float *d_l_aux;     // [1] or null
+    float *dlogits;           // [S,E]
+};
+template <typename T, int K, int VPL>
+__global__ __launch_bounds__(PM_THREADS) void combine_bwd_gate_kernel(const T *__restrict__ dy, const T *__restrict__ o,
+                                                                      const int32_t *__restrict__ row,
+                                                                      const float *__restrict__ gates, int S, int M,
+                                                                      int k, T *__restrict__ d_o, const GateBwdArgs ga) {
+    const int i = blockIdx.x * (PM_THREADS / WAVE) + (threadIdx.x >> 6);
+    if (i >= S) return;
+    const int lane = lane_id(), E = ga.E;
+    // the token's scores, the choice this lane looks after (lanes below k), and that choice's raw gate value
+    float s[VPL], ds[VPL];
+#pragma unroll
+    for (int r = 0; r < VPL; ++r) {
+        const int e = lane + 64 * r;
+        s[r] = ga.scores[(size_t)i * E + min(e, E - 1)];
+    }
+    const int my_e = ga.idx[(size_t)min(lane, k - 1) * S + i];
+    float dot[K];
+    combine_bwd_rows<T, K>(dy, o, row, gates, S, M, k, i, d_o, dot);
+    // the raw gate value of this lane's choice is the score of expert my_e, which lane my_e % 64 holds: handed over
+    // between lanes (a load of it would have to wait for my_e first, one more memory latency per wave)
+    float my_gr = 0.f;
+    const int e_c = min(max(my_e, 0), E - 1);
+#pragma unroll
+    for (int r = 0; r < VPL; ++r) {
+        const float v = __shfl(s[r], e_c & 63, WAVE);
+        if ((e_c >> 6) == r) my_gr = v;
+    }
+    float my_dg = 0.f;
+#pragma unroll
+    for (int j = 0; j < K; ++j)
+        if (lane == j) my_dg = dot[j];
+    if (lane >= k) { my_dg = 0.f; my_gr = 0.f; }
+#pragma unroll
+    for (int r = 0; r < VPL; ++r) {
+        if (lane + 64 * r >= E) s[r] = 0.f;
+        ds[r] = 0.f;
+    }
+    if (ga.counts0 != nullptr) {
+        const float scale = ga.d_l_aux[0] * ((float)E / ((float)S * (float)S));
+#pragma unroll
+        for (int r = 0; r < VPL; ++r) ds[r] = scale * (float)ga.counts0[min(lane + 64 * r, E - 1)];
+    }
+    constexpr float EPS = 1.1920928955078125e-07f;
+    const float denom = wave_sum(my_gr);
+    const float dotg = wave_sum(my_dg * my_gr);
+    const bool norm = k > 1 && ga.normalize;
+    const bool clamped = denom < EPS;
+    const float den = clamped ? EPS : denom;
+    const float sub = (norm && !clamped) ? dotg / (den * den) : 0.f;
+    const float my_dgraw = norm ? my_dg / den - sub : my_dg;
+    for (int j = 0; j < k; ++j) {
+        const int e = __builtin_amdgcn_readlane(my_e, j);
+        const float dgraw = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, my_dgraw), j));
+        if ((e & 63) == lane) {
+            const int rr = e >> 6;
+#pragma unroll
+            for (int r = 0; r < VPL; ++r)
+                if (r == rr) ds[r] += dgraw;
+        }
+    }
+    float dsum = 0.f;
+#pragma unroll
+    for (int r = 0; r < VPL; ++r) dsum += ds[r] * s[r];
+    dsum = wave_sum(dsum);
+#pragma unroll
+    for (int r = 0; r < VPL; ++r) {
+        const int e = lane + 64 * r;
+        if (e < E) ga.dlogits[(size_t)i * E + e] = ga.through_softmax ? s[r] * (ds[r] - dsum) : ds[r];
     }
 }
 
@@ -1066,6 +1160,38 @@ extern "C" int mole_combine_bwd(const void *dy, const void *o, int dtype, const 
         PM_LAUNCH_K(MOLE_K_COMBINE_BWD, combine_bwd_kernel, bf16_t, (const bf16_t *)dy, (const bf16_t *)o, row, gates, S, M, k, (bf16_t *)d_o, dgates);
     else
         PM_LAUNCH_K(MOLE_K_COMBINE_BWD, combine_bwd_kernel, float, (const float *)dy, (const float *)o, row, gates, S, M, k, (float *)d_o, dgates);
+    MOLE_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int mole_combine_bwd_gate(const void *dy, const void *o, int dtype, const int32_t *row, const float *gates,
+                                     int S, int M, int k, void *d_o, const float *scores, const int32_t *idx, int E,
+                                     int normalize_gate, int through_softmax, const int32_t *counts0,
+                                     const float *d_l_aux, float *dlogits, mole_stream_t stream) {
+    if (int rc = check_perm("mole_combine_bwd_gate", dtype, S, M, k)) return rc;
+    MOLE_REQUIRE(E >= 1 && E <= 256 && k <= E, "mole_combine_bwd_gate: E=%d must be 1..256 and at least k=%d (larger gates: mole_combine_bwd + mole_gate_bwd)", E, k);
+    if (S == 0) return 0;
+    MOLE_REQUIRE(dy && o && row && gates && d_o && scores && idx && dlogits && aligned16(dy) && aligned16(o) && aligned16(d_o),
+                 "mole_combine_bwd_gate: null or misaligned pointer");
+    MOLE_REQUIRE((counts0 == nullptr) == (d_l_aux == nullptr), "mole_combine_bwd_gate: counts0 and d_l_aux go together");
+    const GateBwdArgs ga{scores, idx, E, normalize_gate, through_softmax, counts0, d_l_aux, dlogits};
+    const dim3 grid(ceil_div(S, PM_THREADS / WAVE)), blk(PM_THREADS);
+    hipStream_t st = (hipStream_t)stream;
+    const int vpl = E <= 64 ? 1 : (E <= 128 ? 2 : 4);
+#define MOLE_CBG(T, KK)                                                                                              \
+    do {                                                                                                             \
+        if (vpl == 1) timed_launch(MOLE_K_COMBINE_BWD, combine_bwd_gate_kernel<T, KK, 1>, grid, blk, 0, st, (const T *)dy, (const T *)o, row, gates, S, M, k, (T *)d_o, ga); \
+        else if (vpl == 2) timed_launch(MOLE_K_COMBINE_BWD, combine_bwd_gate_kernel<T, KK, 2>, grid, blk, 0, st, (const T *)dy, (const T *)o, row, gates, S, M, k, (T *)d_o, ga); \
+        else timed_launch(MOLE_K_COMBINE_BWD, combine_bwd_gate_kernel<T, KK, 4>, grid, blk, 0, st, (const T *)dy, (const T *)o, row, gates, S, M, k, (T *)d_o, ga); \
+    } while (0)
+#define MOLE_CBG_K(T)                                                                                                \
+    do {                                                                                                             \
+        if (k <= 1) MOLE_CBG(T, 1); else if (k <= 2) MOLE_CBG(T, 2); else if (k <= 4) MOLE_CBG(T, 4);                \
+        else if (k <= 8) MOLE_CBG(T, 8); else MOLE_CBG(T, 16);                                                       \
+    } while (0)
+    if (dtype == MOLE_BF16) MOLE_CBG_K(bf16_t); else MOLE_CBG_K(float);
+#undef MOLE_CBG_K
+#undef MOLE_CBG
     MOLE_LAUNCH_CHECK();
     return 0;
 }

@@ -191,6 +191,14 @@ int mole_combine_fwd(const void *o, int dtype, const int32_t *row, const float *
 int mole_combine_bwd(const void *dy, const void *o, int dtype, const int32_t *row,
                      const float *gates, int S, int M, int k, void *d_o, float *dgates,
                      mole_stream_t stream);
+/* mole_combine_bwd followed by mole_gate_bwd (below) in one kernel, for gates of up to 256 experts: the backward of
+ * tutel's fast_decode (MOLE/moe/layer.py:457-458) and the autograd of the gate values inside extract_critical
+ * (layer.py:445-446) and of the softmax (MOLE/utils/Ugate.py:11-14).  The k gate gradients of a token stay in the
+ * wave that formed them; the arguments after d_o are those of mole_gate_bwd, dlogits [S,E] its result. */
+int mole_combine_bwd_gate(const void *dy, const void *o, int dtype, const int32_t *row, const float *gates,
+                          int S, int M, int k, void *d_o, const float *scores, const int32_t *idx, int E,
+                          int normalize_gate, int through_softmax, const int32_t *counts0,
+                          const float *d_l_aux, float *dlogits, mole_stream_t stream);
 int mole_zero_pad_rows(void *buf, int dtype, const int32_t *kept_rows, const int32_t *offsets,
                        int E, int M, mole_stream_t stream);
 

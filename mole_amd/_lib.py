@@ -47,6 +47,7 @@ _SIGNATURES = {
     "mole_dispatch_bwd": (c_int, [_P, c_int, _P, c_int, c_int, c_int, _P, _P, c_int, _P, _P, _P]),
     "mole_combine_fwd": (c_int, [_P, c_int, _P, _P, c_int, c_int, c_int, _P, _P]),
     "mole_combine_bwd": (c_int, [_P, _P, c_int, _P, _P, c_int, c_int, c_int, _P, _P, _P]),
+    "mole_combine_bwd_gate": (c_int, [_P, _P, c_int, _P, _P, c_int, c_int, c_int, _P, _P, _P, c_int, c_int, c_int, _P, _P, _P, _P]),
     "mole_zero_pad_rows": (c_int, [_P, c_int, _P, _P, c_int, c_int, _P]),
     "mole_ffn_fwd": (c_int, [_P, c_int, _P, _P, c_int, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P]),
     "mole_ffn_bwd": (c_int, [_P, _P, _P, _P, c_int, _P, _P, c_int, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P,

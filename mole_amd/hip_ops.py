@@ -265,6 +265,31 @@ def combine_bwd(dy: torch.Tensor, o: torch.Tensor, row: torch.Tensor, gates: tor
     return d_o, dgates
 
 
+def combine_bwd_gate(dy: torch.Tensor, o: torch.Tensor, row: torch.Tensor, gates: torch.Tensor, scores: torch.Tensor,
+                     idx: torch.Tensor, normalize_gate: bool, through_softmax: bool = True,
+                     counts0: Optional[torch.Tensor] = None, d_l_aux: Optional[torch.Tensor] = None):
+    """combine_bwd and gate_bwd in one kernel (gates of up to 256 experts): returns d_o and d(logits) (or d(scores)
+    when not through_softmax).  Larger gates, and the case where every pair was dropped, take the two calls."""
+    S, E = scores.shape
+    if E > 256 or o.numel() == 0:
+        d_o, dgates = combine_bwd(dy, o, row, gates)
+        return d_o, gate_bwd(dgates, scores, idx, normalize_gate, through_softmax, counts0, d_l_aux)
+    _dev(dy), _dev(o), _dev(row), _dev(gates), _dev(scores), _dev(idx)
+    k = row.shape[0]
+    M = o.shape[-1]
+    if (counts0 is None) != (d_l_aux is None):
+        raise RuntimeError("combine_bwd_gate: counts0 and d_l_aux go together")
+    if d_l_aux is not None:
+        _dev(counts0)
+        d_l_aux = _dev(d_l_aux.reshape(1).float())
+    d_o = torch.empty_like(o)
+    dlogits = torch.empty_like(scores)
+    L.check(L.lib().mole_combine_bwd_gate(L.ptr(dy), L.ptr(o), L.dtype_code(o.dtype), L.ptr(row), L.ptr(gates), S, M, k,
+                                          L.ptr(d_o), L.ptr(scores), L.ptr(idx), E, int(normalize_gate), int(through_softmax),
+                                          L.ptr(counts0), L.ptr(d_l_aux), L.ptr(dlogits), L.stream()), "mole_combine_bwd_gate")
+    return d_o, dlogits
+
+
 def zero_pad_rows(buf: torch.Tensor, kept_rows: torch.Tensor, offsets: torch.Tensor) -> None:
     _dev(buf)
     E = kept_rows.shape[0]

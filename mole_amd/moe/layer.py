@@ -82,13 +82,13 @@ class _FusedMoE(torch.autograd.Function):
         x, wg, scores, out = ctx.saved_tensors
         if ctx.time_it:
             UATimer.track_bwd_start(m.moe_id)
-        d_o, dgates = H.combine_bwd(dy.contiguous(), out, r.row, r.gates)
-        gxd = m.MOLECore.backward(d_o, saved=ctx.saved)
-        ctx.saved = None
         # l_aux reaches the gate only when the caller added it to the loss (an unused output arrives as zeros,
         # which costs nothing: the term rides along in the same kernel)
         aux = {} if d_l_aux is None else dict(counts0=r.counts[0], d_l_aux=d_l_aux)
-        dlogits = H.gate_bwd(dgates, scores, r.idx, m.normalize_gate, through_softmax=True, **aux)
+        d_o, dlogits = H.combine_bwd_gate(dy.contiguous(), out, r.row, r.gates, scores, r.idx, m.normalize_gate,
+                                          through_softmax=True, **aux)
+        gxd = m.MOLECore.backward(d_o, saved=ctx.saved)
+        ctx.saved = None
         wg32 = wg.detach().float().contiguous()
         dx = H.dispatch_bwd(gxd, r.row, dlogits, wg32)
         dwg = H.gate_wgrad(dlogits, x).to(wg.dtype)

@@ -134,3 +134,35 @@ def test_kernel_timing_counts_launches_and_leaves_results_alone():
     for rep in timed:
         assert all(torch.equal(a, b) for a, b in zip(rep, plain))
     assert all(c == 0 for c, _ in L.kernel_timing_read().values())      # a read forgets what it returned
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("S,M,E,k,cf,normalize,aux", [(300, 64, 8, 2, 1.0, True, True), (1000, 128, 16, 1, 1.25, True, False),
+                                                      (513, 64, 100, 4, 0.0, False, True), (257, 256, 256, 8, 0.0, True, True),
+                                                      (64, 64, 3, 3, 0.5, True, False)])
+def test_combine_bwd_with_the_gate_backward_in_its_tail(S, M, E, k, cf, normalize, aux, dtype):
+    """mole_combine_bwd_gate against mole_combine_bwd followed by mole_gate_bwd on the same inputs: the same d_o bit
+    for bit, the same d(logits) to rounding (the two sum a token's k terms over lanes in different patterns)."""
+    from mole_amd import hip_ops as H
+    from tests.util import zipf_scores
+    print(f"combine_bwd_gate S={S} M={M} E={E} k={k} cf={cf} {dtype}", flush=True)
+    g = torch.Generator().manual_seed(S + E)
+    scores = zipf_scores(S, E, seed=S).cuda()
+    r = H.route(scores, k, cf, normalize)
+    rows = max(int(r.offsets[-1]), 1)
+    o = torch.randn(rows, M, generator=g).to(dtype).cuda()
+    dy = torch.randn(S, M, generator=g).to(dtype).cuda()
+    kw = dict(counts0=r.counts[0], d_l_aux=torch.tensor([0.7], device="cuda")) if aux else {}
+    d_o1, dgates = H.combine_bwd(dy, o, r.row, r.gates)
+    want = H.gate_bwd(dgates, scores, r.idx, normalize, True, **kw)
+    d_o2, got = H.combine_bwd_gate(dy, o, r.row, r.gates, scores, r.idx, normalize, True, **kw)
+    torch.cuda.synchronize()
+    kept = (r.row >= 0).any(dim=0)
+    assert bool(kept.any())
+    written = torch.zeros(rows, dtype=torch.bool, device="cuda")
+    written[r.row[r.row >= 0].long()] = True
+    assert torch.equal(d_o1[written], d_o2[written])
+    assert rel_err(got, want) < 1e-5
+    want_s = H.gate_bwd(dgates, scores, r.idx, normalize, False, **kw)
+    _, got_s = H.combine_bwd_gate(dy, o, r.row, r.gates, scores, r.idx, normalize, False, **kw)
+    assert rel_err(got_s, want_s) < 1e-5
