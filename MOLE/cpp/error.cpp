@@ -23,16 +23,12 @@ struct TimedLaunch { int id; hipEvent_t a, b; };
 static bool g_timing = false;
 static std::mutex g_tmu;
 static std::vector<TimedLaunch> g_launches;
-static std::vector<hipEvent_t> g_free_events;
+// Events are created for every timed launch and destroyed when their times have been read: an event that is used again
+// keeps its old time stamp when a launch does not record it, and the launch is then charged with whatever ran since.
 
 bool timing_enabled() { return g_timing; }
 
 static hipEvent_t get_event() {
-    if (!g_free_events.empty()) {
-        hipEvent_t e = g_free_events.back();
-        g_free_events.pop_back();
-        return e;
-    }
     hipEvent_t e = nullptr;
     (void)hipEventCreate(&e);
     return e;
@@ -73,12 +69,13 @@ extern "C" int mole_kernel_timing_read(int n_ids, int *counts, float *ms_total) 
     std::lock_guard<std::mutex> lk(g_tmu);
     for (int i = 0; i < n_ids; ++i) { counts[i] = 0; ms_total[i] = 0.f; }
     for (auto &t : g_launches) {
-        MOLE_HIP(hipEventSynchronize(t.b));
         float ms = 0.f;
-        MOLE_HIP(hipEventElapsedTime(&ms, t.a, t.b));
-        if (t.id >= 0 && t.id < n_ids) { counts[t.id] += 1; ms_total[t.id] += ms; }
-        g_free_events.push_back(t.a);
-        g_free_events.push_back(t.b);
+        // a launch whose events were not both recorded is left out of the count rather than guessed at
+        const bool ok = hipEventSynchronize(t.b) == hipSuccess && hipEventElapsedTime(&ms, t.a, t.b) == hipSuccess;
+        if (!ok) (void)hipGetLastError();
+        if (ok && t.id >= 0 && t.id < n_ids) { counts[t.id] += 1; ms_total[t.id] += ms; }
+        (void)hipEventDestroy(t.a);
+        (void)hipEventDestroy(t.b);
     }
     g_launches.clear();
     return 0;
