@@ -36,7 +36,9 @@ Parity status.
     algorithm: brute-force top-k with the (score desc, index asc) order, stable-sort closed form
     for locations, integer closed form for capacity, permutation invariants, adjointness of
     encode/decode backward, torch autograd on a dense one-hot formulation.
-  * UniMemModel / fast_assign_prefetch are integer state machines restated from the C++.
+  * UniMemModel / fast_assign_prefetch are integer state machines restated from the C++; fast_assign_prefetch is
+    also checked against the reference's own function, compiled from where it lies by oracle/build_ref.py into
+    oracle/_ref/libmole_ref.so (tests/test_oracle_ref.py: every small input and thousands of random ones).
   * adam_step is pinned against torch.optim.Adam and torch.optim.AdamW over several steps in fp64
     and against hand-computed first-step values (tests/test_oracle_adam.py).
 
