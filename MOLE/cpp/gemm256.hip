@@ -819,6 +819,35 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
     k_ext = __builtin_amdgcn_readfirstlane(k_ext);
     row0 = ((long)__builtin_amdgcn_readfirstlane((int)(row0 >> 32)) << 32) | (unsigned)__builtin_amdgcn_readfirstlane((int)row0);
     const int m0 = mt * tile_h, n0 = nt * Q_BN;
+    if constexpr (WG && EPI == EPI_WGRAD) {
+        if (k_ext == 0) {
+            // An expert without rows: its gradient tile is zero (and adds nothing when sums are being built up).  The
+            // zeros leave straight from registers, two 512-byte row pieces per wave and store - no operand ring, no
+            // LDS slab, no barrier (with skewed loads most experts of a launch are such: 28 of 64 at 8192 tokens,
+            // top-2, Zipf(1.2)).
+            if (g.accumulate) return;
+            typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+            bf16_t *Cz = (bf16_t *)g.C + (long)e * g.strideC;
+            const int col = n0 + (lane & 31) * 8;
+            for (int r = wave * 2 + (lane >> 5); r < Q_BM; r += 2 * TL::NW) {
+                const int m = m0 + r;
+                if (m < m_ext && col < g.N)
+                    __builtin_nontemporal_store(u32x4{0u, 0u, 0u, 0u}, reinterpret_cast<u32x4 *>(Cz + (long)m * g.ldc + col));
+            }
+            if (g.colsum != nullptr) {
+                bf16_t *out = (bf16_t *)g.colsum;
+                const bf16_t z = (bf16_t)0.0f;
+                if (g.colsum_side == 1 && nt == sum_nt) {
+                    for (int r = threadIdx.x; r < Q_BM; r += TL::THREADS)
+                        if (m0 + r < m_ext) out[(long)e * g.M + m0 + r] = z;
+                } else if (g.colsum_side == 2 && mt == sum_mt) {
+                    for (int c = threadIdx.x; c < Q_BN; c += TL::THREADS)
+                        if (n0 + c < g.N) out[(long)e * g.N + n0 + c] = z;
+                }
+            }
+            return;
+        }
+    }
     const bf16_t *Mp = (const bf16_t *)g.A + row0 * g.lda;
     const bf16_t *Np = WG ? (const bf16_t *)g.B + row0 * g.ldb : (const bf16_t *)g.B + (long)e * g.strideB;
 

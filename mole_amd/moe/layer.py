@@ -60,6 +60,9 @@ class _FusedMoE(torch.autograd.Function):
     def forward(ctx, x, wg, dummy_param, module, capacity_factor, time_it=False):
         m = module
         ctx.time_it = time_it
+        # an output the loss does not use (l_aux, mostly) arrives as None in backward instead of as a tensor of zeros
+        # that autograd would have to fill first: one small kernel and its place in the queue less per step
+        ctx.set_materialize_grads(False)
         S, M = x.shape
         k = min(m.topk, m.total_experts)
         scores = Ugate.gate_scores(x, wg, m.gate[0].logit_bias)
@@ -80,6 +83,8 @@ class _FusedMoE(torch.autograd.Function):
     def backward(ctx, dy, d_l_aux):
         m, r = ctx.m, ctx.r
         x, wg, scores, out = ctx.saved_tensors
+        if dy is None:            # only l_aux was used
+            dy = torch.zeros_like(x)
         if ctx.time_it:
             UATimer.track_bwd_start(m.moe_id)
         # l_aux reaches the gate only when the caller added it to the loss (an unused output arrives as zeros,
