@@ -436,12 +436,17 @@ static bool fast_path_enabled() {
     return on;
 }
 
-// bf16 products go to the 256x256 direct-to-LDS kernel when their shape allows it
+// products go to the direct-to-LDS kernel of their element type when their shape allows it
 template <typename T, bool A_KS, bool B_KS, bool WG, int EPI>
 static int run_gemm(const GemmArgs &g, int max_rows, int tiles_generic, hipStream_t st, int kid) {
     if constexpr (sizeof(T) == 2) {
         if (fast_path_enabled()) {
             const int rc = launch_gemm256(g, A_KS, B_KS, WG, EPI, max_rows, st, kid);
+            if (rc != -100) return rc;
+        }
+    } else {
+        if (fast_path_enabled()) {
+            const int rc = launch_gemm_f32(g, A_KS, B_KS, WG, EPI, max_rows, st, kid);
             if (rc != -100) return rc;
         }
     }

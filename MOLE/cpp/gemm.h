@@ -93,5 +93,7 @@ struct GemmArgs {
 // meet its alignment requirements; the caller then uses the generic kernel.
 int launch_gemm256(const GemmArgs &g, bool a_ks, bool b_ks, bool wg, int epi, int max_rows, hipStream_t st, int kid);
 bool gemm256_sums_operand(const GemmArgs &g, int kid);
+// fp32 tiles with direct-to-LDS loads (gemm_f32.hip); -100 as above.
+int launch_gemm_f32(const GemmArgs &g, bool a_ks, bool b_ks, bool wg, int epi, int max_rows, hipStream_t st, int kid);
 
 }  // namespace mole

@@ -11,7 +11,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CPP = os.path.join(ROOT, "MOLE", "cpp")
 LIB = os.path.join(CPP, "libmole_hip.so")
-SOURCES = ["error.cpp", "route.hip", "permute.hip", "ffn_gemm.hip", "gemm256.hip", "adam.hip", "unimem.hip", "probe.hip"]
+SOURCES = ["error.cpp", "route.hip", "permute.hip", "ffn_gemm.hip", "gemm256.hip", "gemm_f32.hip", "adam.hip", "unimem.hip", "probe.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-x", "hip",
          # keep the compiler from forming packed-fp32 VALU ops
