@@ -450,7 +450,7 @@ static int run_gemm(const GemmArgs &g, int max_rows, int tiles_generic, hipStrea
             if (rc != -100) return rc;
         }
     }
-    // only the 256-wide kernel sums an operand on the side: the caller asks gemm256_sums_operand() first
+    // only the direct-to-LDS kernels sum an operand on the side: the caller asks gemm*_sums_operand() first
     MOLE_REQUIRE(g.colsum == nullptr, "grouped GEMM: operand sums requested from a kernel that does not produce them");
     return launch_gemm<T, A_KS, B_KS, WG, TBM, TBN, EPI>(g, tiles_generic, st, kid);
 }
@@ -484,14 +484,17 @@ static int ffn_bwd_t(const void *go, const void *xd, const void *h, const void *
     g.accumulate = accumulate; g.gelu_bwd = gelu_bwd;
     const int wg_tiles = E * ceil_div(F, TBM) * ceil_div(M, TBN);
     // The bias gradients are sums of go and of t over every expert's rows: go and t are operands of the two
-    // weight-gradient products, whose 256-wide kernel sums an operand on the side (one more MFMA against a
-    // block of ones in the blocks that see the whole operand).  Other kernels leave them to bias_grad_kernel.
+    // weight-gradient products, whose direct-to-LDS kernels sum an operand on the side in the blocks that see the
+    // whole operand (bf16: one more MFMA against a block of ones; fp32: the fragments are added up as they pass).
+    // The generic kernel leaves them to bias_grad_kernel.
     GemmArgs gw2{};
     gw2 = g;
     gw2.A = a; gw2.lda = F; gw2.B = go; gw2.ldb = M; gw2.M = F; gw2.N = M; gw2.C = g_w2; gw2.ldc = M; gw2.strideC = (long)F * M;
     bool fused_sums = false;
     if constexpr (sizeof(T) == 2)
         fused_sums = fast_path_enabled() && gemm256_sums_operand(gw2, MOLE_K_FFN_GW2) && gemm256_sums_operand(gw2, MOLE_K_FFN_GW1);
+    else
+        fused_sums = fast_path_enabled() && gemm_f32_sums_operand(gw2);
     // g_w2[e] = a^T . go          (contract over the expert's rows); g_b2 = sum go
     if (fused_sums) { gw2.colsum = g_b2; gw2.colsum_side = 2; }
     if (int rc = run_gemm<T, true, true, true, EPI_WGRAD>(gw2, max_rows, wg_tiles, st, MOLE_K_FFN_GW2)) return rc;

@@ -82,7 +82,7 @@ struct GemmArgs {
     int accumulate;         // EPI_WGRAD: add into C
     int gelu_bwd;           // EPI_DGELU: MOLE_GELU_BWD_*
     int n_blocks;           // real number of tiles in the launch (grid is rounded up to 8)
-    void *colsum;           // weight gradients, 256-wide kernel: [E][M] (side 1) or [E][N] (side 2) sums of an operand
+    void *colsum;           // weight gradients, direct-to-LDS kernels: [E][M] (side 1) or [E][N] (side 2) sums of an operand
     int colsum_side;        //   over the expert's rows: 1 = the m-side operand (A), 2 = the n-side operand (B)
     int wg_expert_major;    // weight gradients, 256-wide kernel: all (m-tile, n-tile) blocks of an expert on one XCD
     int m_fastest;          // row-ragged products, 256-wide kernel: number an expert's tiles m-tile first (see gemm256.hip)
@@ -95,5 +95,6 @@ int launch_gemm256(const GemmArgs &g, bool a_ks, bool b_ks, bool wg, int epi, in
 bool gemm256_sums_operand(const GemmArgs &g, int kid);
 // fp32 tiles with direct-to-LDS loads (gemm_f32.hip); -100 as above.
 int launch_gemm_f32(const GemmArgs &g, bool a_ks, bool b_ks, bool wg, int epi, int max_rows, hipStream_t st, int kid);
+bool gemm_f32_sums_operand(const GemmArgs &g);
 
 }  // namespace mole

@@ -5,10 +5,10 @@
 // v_mfma_f32_32x32x2_f32 keeps a SIMD's matrix pipe busy for 64 cycles and consumes one register of each operand,
 // so the arithmetic leaves room for everything else - as long as something else is ready to issue.  The kernel is
 // therefore built for several independent blocks per CU rather than one large one: a block of 4 waves (2 x 2) owns a
-// BM x BN tile (128 x 128, or 64 x 128 where that gives the chip two blocks per CU instead of one), its operand
-// stages of 16 of K come from HBM/L2 straight into a four-stage LDS ring (global_load_lds_dwordx4, three stages in
-// flight, one barrier per stage), and the fragments of stage s+1 are read into registers while the MFMAs of stage s
-// run.  Two blocks share a CU: one block's prologue, barriers and epilogue run under the other's MFMAs.
+// BM x BN tile (64 x 128 for the row-ragged products, 128 x 128 for the weight gradients), its operand stages of 16
+// of K come from HBM/L2 straight into a ring of three or four LDS stages (global_load_lds_dwordx4, one barrier per
+// stage), and the fragments of stage s+1 are read into registers while the MFMAs of stage s run, the loads and reads
+// dealt out between the MFMAs.  Two to four blocks share a CU.
 //
 // LDS images (the 16-byte piece a lane's load fills is fixed by the hardware; which global address it fetches
 // is ours to choose, so any permutation of pieces is free):
@@ -29,13 +29,12 @@ namespace {
 
 constexpr int F_BK = 16;          // k per stage: 64 bytes of a K-contiguous row
 constexpr int F_THREADS = 256;    // 4 waves, 2 x 2
-constexpr int F_NSTAGE = 4;
 
-template <int BM, int BN> struct FTile {
+template <int BM, int BN, int NSTAGE> struct FTile {
     static constexpr int TMW = BM / 64, TNW = BN / 64;        // 32-row blocks per wave on either side
     static constexpr int M_BYTES = BM * F_BK * 4, N_BYTES = BN * F_BK * 4, STAGE = M_BYTES + N_BYTES;
     static constexpr int LM = BM / 64, LN = BN / 64, L = LM + LN;   // 1-KiB loads per wave and stage
-    static constexpr int LDS_BYTES = F_NSTAGE * STAGE;
+    static constexpr int LDS_BYTES = NSTAGE * STAGE;
 };
 
 // Per-lane byte offsets of the loads a wave issues for one stage of an operand tile, relative to the tile's first
@@ -111,9 +110,10 @@ template <int ROWS, bool KS, int NB> struct FFrag {
     }
 };
 
-template <int BM, int BN, bool M_KS, bool N_KS, bool WG, int EPI>
-__global__ __launch_bounds__(F_THREADS, 2) void gemm_f32_kernel(const GemmArgs g) {
-    typedef FTile<BM, BN> TL;
+template <int BM, int BN, int NSTAGE, int BPC, bool M_KS, bool N_KS, bool WG, int EPI>
+__global__ __launch_bounds__(F_THREADS, BPC) void gemm_f32_kernel(const GemmArgs g) {
+    typedef FTile<BM, BN, NSTAGE> TL;
+    constexpr int F_NSTAGE = NSTAGE;
     constexpr int TMW = TL::TMW, TNW = TL::TNW, L = TL::L;
     extern __shared__ __align__(16) char smem[];
     const int lane = threadIdx.x & 63;
@@ -191,6 +191,24 @@ __global__ __launch_bounds__(F_THREADS, 2) void gemm_f32_kernel(const GemmArgs g
 #pragma unroll
             for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
 
+    // Operand sums over the contraction (the bias gradients: sums of go and of t over an expert's rows, torch::sum_out
+    // in MOLE/cpp/core.cpp:399, 408) ride along in the weight-gradient blocks that see the whole operand once: the
+    // first n-tile of every m-tile for the m-side, the first m-tile of every n-tile for the n-side.  The wave row or
+    // column that holds the operand's fragments adds them up as they pass, four partial sums per column.
+    int sum_side = 0;
+    if constexpr (WG) {
+        if (g.colsum != nullptr) {
+            if (g.colsum_side == 1 && nt == 0 && wn == 0) sum_side = 1;
+            if (g.colsum_side == 2 && mt == 0 && wm == 0) sum_side = 2;
+        }
+    }
+    constexpr int SB = TMW > TNW ? TMW : TNW;
+    float psum[4][SB];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int b = 0; b < SB; ++b) psum[j][b] = 0.f;
+
     const int nk = (k_ext + F_BK - 1) / F_BK;
     if (nk > 0) {
         const int kl = k_ext - (nk - 1) * F_BK;     // k-rows of the last stage (a row-ragged product's K is whole stages)
@@ -204,24 +222,25 @@ __global__ __launch_bounds__(F_THREADS, 2) void gemm_f32_kernel(const GemmArgs g
         const long step_m = M_KS ? g.lda * (F_BK * 4) : F_BK * 4;
         const long step_n = N_KS ? g.ldb * (F_BK * 4) : F_BK * 4;
         const uint32_t lds_w = lds_offset_of(smem) + wave * 1024;
-        // the loads of stage s into ring buffer s mod 4; stages are issued in order (the bases advance)
-        auto issue = [&](int s) __attribute__((always_inline)) {
-            const uint32_t dst = lds_w + (s & (F_NSTAGE - 1)) * TL::STAGE;
+        // load j of stage s (the m-side tile's loads come first) into ring buffer s mod NSTAGE; stages are issued in
+        // order, the bases advance after a stage's last load
+        auto issue_one = [&](int s, int j) __attribute__((always_inline)) {
+            const uint32_t dst = lds_w + (s % F_NSTAGE) * TL::STAGE;
             const bool last = WG && s == nk - 1;
-#pragma unroll
-            for (int j = 0; j < TL::LM; ++j) {
+            if (j < TL::LM) {
                 uint32_t o = om.off[j];
                 if constexpr (WG) o = last ? cm.off[j] : o;
                 dma16s(bm, o, dst + j * 4096);
+            } else {
+                uint32_t o = on.off[j - TL::LM];
+                if constexpr (WG) o = last ? cn.off[j - TL::LM] : o;
+                dma16s(bn, o, dst + TL::M_BYTES + (j - TL::LM) * 4096);
             }
+            if (j == L - 1) { bm += step_m; bn += step_n; }
+        };
+        auto issue = [&](int s) __attribute__((always_inline)) {
 #pragma unroll
-            for (int j = 0; j < TL::LN; ++j) {
-                uint32_t o = on.off[j];
-                if constexpr (WG) o = last ? cn.off[j] : o;
-                dma16s(bn, o, dst + TL::M_BYTES + j * 4096);
-            }
-            bm += step_m;
-            bn += step_n;
+            for (int j = 0; j < L; ++j) issue_one(s, j);
         };
         // ragged contraction: zero the k-rows past its end in the last stage (both tiles are [k][rows] there)
         auto zero_tail = [&](int buf) __attribute__((always_inline)) {
@@ -241,38 +260,96 @@ __global__ __launch_bounds__(F_THREADS, 2) void gemm_f32_kernel(const GemmArgs g
 #pragma unroll
         for (int s = 0; s < F_NSTAGE - 1; ++s)
             if (s < nk) issue(s);
-        if (nk >= 3) __builtin_amdgcn_s_waitcnt(waitcnt_vm(2 * L));
-        else if (nk == 2) __builtin_amdgcn_s_waitcnt(waitcnt_vm(L));
+        if (F_NSTAGE == 4 && nk >= 3) __builtin_amdgcn_s_waitcnt(waitcnt_vm(2 * L));
+        else if (nk >= 2) __builtin_amdgcn_s_waitcnt(waitcnt_vm(L));
         else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
         __builtin_amdgcn_s_barrier();
         if (WG && nk == 1 && kl < F_BK) zero_tail(0);
         ma.read(smem, fm0, fm1);
         na.read(smem + TL::M_BYTES, fn0, fn1);
 
-#define MOLE_F32_STAGE(S, MC, NC, MN, NN)                                                                   \
+        // One stage: the MFMAs of stage S on the fragments MC / NC.  With NEXT, first the hand-over to stage S + 1: wait
+        // until this wave's share of it has landed, barrier; then, dealt out between the MFMAs so that the matrix pipe
+        // always has the next one waiting, the loads that refill the buffer stage S - 1 has left and the fragment reads
+        // of stage S + 1 into MN / NN.  (A wave issues in order: eight loads and reads in a row right after the barrier
+        // left the pipe idle for a tenth of a 64 x 128 tile's stage.)  NEXT is a compile-time choice: were the fragment
+        // reads under a run-time condition, the compiler could not tell how many LDS reads are outstanding at the first
+        // MFMA and would wait for all of them, the ones just issued included.
+        // Order of a stage's MFMAs: two waves on a SIMD that each alternate between two accumulators run at 0.85 of the
+        // MFMA rate on this chip (measured with operands held in registers: one, three or four accumulators in turn, or
+        // one wave per SIMD, all reach the full rate), so a wave with two cells runs its eight steps on one cell, then
+        // on the other; with four cells they take turns.
+#define MOLE_F32_STAGE(S, MC, NC, MN, NN, NEXT)                                                             \
         {                                                                                                   \
             const int s_ = (S);                                                                             \
-            if (s_ + 1 < nk) {                                                                              \
-                if (s_ + 2 < nk) __builtin_amdgcn_s_waitcnt(waitcnt_vm(L));                                 \
+            bool refill_ = false;                                                                           \
+            const int nb_ = (s_ + 1) % F_NSTAGE;                                                            \
+            if constexpr (NEXT) {                                                                           \
+                if (F_NSTAGE == 4 && s_ + 2 < nk) __builtin_amdgcn_s_waitcnt(waitcnt_vm(L));                \
                 else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));                                             \
                 __builtin_amdgcn_s_barrier();                                                               \
-                if (s_ + 3 < nk) issue(s_ + 3);                                                             \
-                const int nb_ = (s_ + 1) & (F_NSTAGE - 1);                                                  \
+                refill_ = s_ + F_NSTAGE - 1 < nk;                                                           \
                 if (WG && s_ + 1 == nk - 1 && kl < F_BK) zero_tail(nb_);                                    \
-                MN.read(smem + nb_ * TL::STAGE, fm0, fm1);                                                  \
-                NN.read(smem + nb_ * TL::STAGE + TL::M_BYTES, fn0, fn1);                                    \
             }                                                                                               \
-            _Pragma("unroll") for (int kk = 0; kk < 2; ++kk)                                                \
-            _Pragma("unroll") for (int j = 0; j < 4; ++j)                                                   \
-            _Pragma("unroll") for (int tm = 0; tm < TMW; ++tm)                                              \
-            _Pragma("unroll") for (int tn = 0; tn < TNW; ++tn)                                              \
-                acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(MC.get(tm, kk, j), NC.get(tn, kk, j), acc[tm][tn], 0, 0, 0); \
+            constexpr int CELLS_ = TMW * TNW, NM_ = 8 * CELLS_, G_ = NM_ / 8;                               \
+            _Pragma("unroll") for (int grp = 0; grp < 8; ++grp) {                                           \
+                _Pragma("unroll") for (int u = 0; u < G_; ++u) {                                            \
+                    const int n_ = grp * G_ + u;                                                            \
+                    const int cell_ = CELLS_ == 2 ? n_ / 8 : n_ % CELLS_, step_ = CELLS_ == 2 ? n_ % 8 : n_ / CELLS_; \
+                    const int tm = cell_ / TNW, tn = cell_ % TNW, kk = step_ / 4, j = step_ % 4;            \
+                    acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(MC.get(tm, kk, j), NC.get(tn, kk, j), acc[tm][tn], 0, 0, 0); \
+                }                                                                                           \
+                if constexpr (NEXT) {                                                                       \
+                    if (grp < L && refill_) issue_one(s_ + F_NSTAGE - 1, grp);                              \
+                    if (grp == 0) MN.read(smem + nb_ * TL::STAGE, fm0, fm1);                                \
+                    if (grp == 1) NN.read(smem + nb_ * TL::STAGE + TL::M_BYTES, fn0, fn1);                  \
+                }                                                                                           \
+                __builtin_amdgcn_sched_barrier(0);                                                          \
+            }                                                                                               \
+            if constexpr (WG) {                                                                             \
+                if (sum_side == 1) {                                                                        \
+                    _Pragma("unroll") for (int kk = 0; kk < 2; ++kk)                                        \
+                    _Pragma("unroll") for (int j = 0; j < 4; ++j)                                           \
+                    _Pragma("unroll") for (int b = 0; b < TMW; ++b) psum[j][b] += MC.get(b, kk, j);         \
+                } else if (sum_side == 2) {                                                                 \
+                    _Pragma("unroll") for (int kk = 0; kk < 2; ++kk)                                        \
+                    _Pragma("unroll") for (int j = 0; j < 4; ++j)                                           \
+                    _Pragma("unroll") for (int b = 0; b < TNW; ++b) psum[j][b] += NC.get(b, kk, j);         \
+                }                                                                                           \
+            }                                                                                               \
         }
-        for (int s = 0; s < nk; s += 2) {
-            MOLE_F32_STAGE(s, ma, na, mb, nb)
-            if (s + 1 < nk) MOLE_F32_STAGE(s + 1, mb, nb, ma, na)
+        int s = 0;
+        for (; s + 2 < nk; s += 2) {
+            MOLE_F32_STAGE(s, ma, na, mb, nb, true)
+            MOLE_F32_STAGE(s + 1, mb, nb, ma, na, true)
+        }
+        if (nk - s == 2) {
+            MOLE_F32_STAGE(s, ma, na, mb, nb, true)
+            MOLE_F32_STAGE(s + 1, mb, nb, ma, na, false)
+        } else {
+            MOLE_F32_STAGE(s, ma, na, mb, nb, false)
         }
 #undef MOLE_F32_STAGE
+    }
+
+    if constexpr (WG) {
+        if (sum_side != 0) {
+            // a lane's fragments cover k-rows 8 kk + 4 (lane / 32) + j: the two half waves hold the two halves of the sum
+            const int nbk = sum_side == 1 ? TMW : TNW;
+            const int first = sum_side == 1 ? m0 + wm * 32 * TMW : n0 + wn * 32 * TNW;
+            const int ext = sum_side == 1 ? m_ext : g.N;
+            float *out = (float *)g.colsum + (long)e * ext;
+#pragma unroll
+            for (int b = 0; b < SB; ++b) {
+                float v = (psum[0][b] + psum[1][b]) + (psum[2][b] + psum[3][b]);
+                v += __shfl_xor(v, 32, WAVE);
+                const int c = first + nbk * (lane & 31) + b;
+                if (b < nbk && lane < 32 && c < ext) {
+                    if (g.accumulate) v += out[c];
+                    out[c] = v;
+                }
+            }
+        }
     }
 
     // ---- epilogue.  acc[tm][tn][q] = C[m, n] with i = 8 (q / 4) + 4 (lane / 32) + q % 4 the row inside the m-block and
@@ -338,31 +415,44 @@ __global__ __launch_bounds__(F_THREADS, 2) void gemm_f32_kernel(const GemmArgs g
                 }
             }
             float *dst = Cb + (crow0 + m) * g.ldc;
+            // The weight gradients (which nothing reads before the optimizer) leave with non-temporal stores: -2 us on
+            // 8 x 2048 x 512.  For h, a and t it measured neutral to worse: the launches that follow read them.
+            constexpr bool STREAM = EPI == EPI_WGRAD;
+            auto put = [&](float *p, float x) __attribute__((always_inline)) {
+                if constexpr (STREAM) __builtin_nontemporal_store(x, p); else *p = x;
+            };
+            auto put2 = [&](float *p, float x, float y) __attribute__((always_inline)) {
+                typedef float f32x2 __attribute__((ext_vector_type(2)));
+                if constexpr (STREAM) __builtin_nontemporal_store(f32x2{x, y}, reinterpret_cast<f32x2 *>(p));
+                else *reinterpret_cast<float2 *>(p) = make_float2(x, y);
+            };
             if constexpr (PAIR) {
                 if (ncol[0] < g.N) {
-                    *reinterpret_cast<float2 *>(dst + ncol[0]) = make_float2(v[0], v[1]);
-                    if constexpr (EPI == EPI_BIAS_GELU)
-                        *reinterpret_cast<float2 *>((float *)g.C2 + (crow0 + m) * g.ldc + ncol[0]) = make_float2(v2[0], v2[1]);
+                    put2(dst + ncol[0], v[0], v[1]);
+                    if constexpr (EPI == EPI_BIAS_GELU) put2((float *)g.C2 + (crow0 + m) * g.ldc + ncol[0], v2[0], v2[1]);
                 }
             } else {
 #pragma unroll
                 for (int tn = 0; tn < TNW; ++tn) {
                     if (ncol[tn] >= g.N) continue;
-                    dst[ncol[tn]] = v[tn];
-                    if constexpr (EPI == EPI_BIAS_GELU) ((float *)g.C2)[(crow0 + m) * g.ldc + ncol[tn]] = v2[tn];
+                    put(dst + ncol[tn], v[tn]);
+                    if constexpr (EPI == EPI_BIAS_GELU) put((float *)g.C2 + (crow0 + m) * g.ldc + ncol[tn], v2[tn]);
                 }
             }
         }
     }
 }
 
-template <int BM, int BN, bool M_KS, bool N_KS, bool WG, int EPI>
+template <int BM, int BN, int NSTAGE, int BPC, bool M_KS, bool N_KS, bool WG, int EPI>
 int launch_f32(GemmArgs g, int tiles, hipStream_t st, int kid) {
     if (tiles <= 0) return 0;
     g.n_blocks = tiles;
     const int grid = (tiles + 7) & ~7;
-    auto kern = gemm_f32_kernel<BM, BN, M_KS, N_KS, WG, EPI>;
-    constexpr int lds = FTile<BM, BN>::LDS_BYTES;
+    auto kern = gemm_f32_kernel<BM, BN, NSTAGE, BPC, M_KS, N_KS, WG, EPI>;
+    // the LDS request also caps the blocks a CU takes: with room for more than BPC, the dispatcher fills some CUs
+    // and leaves others short, and the launch lasts as long as the fullest
+    constexpr int lds_min = 160 * 1024 / (BPC + 1) + 1024;
+    constexpr int lds = FTile<BM, BN, NSTAGE>::LDS_BYTES > lds_min ? FTile<BM, BN, NSTAGE>::LDS_BYTES : lds_min;
     static bool attr_done = false;
     if (!attr_done) {
         MOLE_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds));
@@ -373,38 +463,53 @@ int launch_f32(GemmArgs g, int tiles, hipStream_t st, int kid) {
     return 0;
 }
 
-template <int BM>
+template <int BM, int BN, int NSTAGE, int BPC>
 int dispatch_f32(const GemmArgs &g, bool b_ks, bool wg, int epi, int max_rows, hipStream_t st, int kid) {
-    const int n_tiles = ceil_div(g.N, 128);
+    const int n_tiles = ceil_div(g.N, BN);
     if (wg) {
         const int tiles = g.E * ceil_div(g.M, BM) * n_tiles;
-        if (epi == EPI_WGRAD) return launch_f32<BM, 128, true, true, true, EPI_WGRAD>(g, tiles, st, kid);
+        if (epi == EPI_WGRAD) return launch_f32<BM, BN, NSTAGE, BPC, true, true, true, EPI_WGRAD>(g, tiles, st, kid);
         return -100;
     }
     const int rows_bound = g.offsets ? max_rows : g.single_rows;
     const int tiles = (rows_bound / BM + (g.offsets ? g.E : 1)) * n_tiles;     // every expert may end in a partial tile
     if (!b_ks) {
-        if (epi == EPI_BIAS_GELU) return launch_f32<BM, 128, false, false, false, EPI_BIAS_GELU>(g, tiles, st, kid);
-        if (epi == EPI_DGELU) return launch_f32<BM, 128, false, false, false, EPI_DGELU>(g, tiles, st, kid);
+        if (epi == EPI_BIAS_GELU) return launch_f32<BM, BN, NSTAGE, BPC, false, false, false, EPI_BIAS_GELU>(g, tiles, st, kid);
+        if (epi == EPI_DGELU) return launch_f32<BM, BN, NSTAGE, BPC, false, false, false, EPI_DGELU>(g, tiles, st, kid);
     } else {
-        if (epi == EPI_BIAS) return launch_f32<BM, 128, false, true, false, EPI_BIAS>(g, tiles, st, kid);
-        if (epi == EPI_STORE) return launch_f32<BM, 128, false, true, false, EPI_STORE>(g, tiles, st, kid);
+        if (epi == EPI_BIAS) return launch_f32<BM, BN, NSTAGE, BPC, false, true, false, EPI_BIAS>(g, tiles, st, kid);
+        if (epi == EPI_STORE) return launch_f32<BM, BN, NSTAGE, BPC, false, true, false, EPI_STORE>(g, tiles, st, kid);
     }
     return -100;
 }
 
 }  // namespace
 
+// Tile shapes, from same-box sweeps on the reference's configuration (8 experts of about 1000 rows, M 512, F 2048) -
+// durations in us of h = xd.w1^T + b1 | t = (go.w2^T) gelu'(h) | out = a.w2 + b2 | gx = t.w1 | the weight gradients:
+//   128 x 128, 4 stages, 2 blocks per CU    153 | 150 |  -  |  -  | 126   (256 tiles of the two K = F products: one per CU)
+//    64 x 128, 4 stages, 2 blocks per CU     -  |  -  | 127 | 124 | 131
+//    64 x 128, 4 stages, 3 blocks per CU    155 | 145 |  -  |  -  | 131
+//    64 x 128, 3 stages, 4 blocks per CU    144 | 145 |  -  |  -  | 127
+//    64 x  64, 4 stages, 4 blocks per CU     -  |  -  | 128 | 127 |  -
+//   128 x 128, 3 stages, 3 blocks per CU    176 | 171 |  -  |  -  | 125
+// Row-ragged products take 64 x 128 tiles: with enough of them for four blocks per CU the shallower ring, otherwise
+// two blocks per CU with the deeper one; weight gradients take 128 x 128.
+// Whether the weight-gradient launch for g also produces the operand sums asked for in g.colsum.
+bool gemm_f32_sums_operand(const GemmArgs &g) {
+    return !(g.lda % 4 || g.ldb % 4 || g.ldc % 4 || g.N % 4 || g.N < 4 || g.M % 4 || g.M < 4);
+}
+
 int launch_gemm_f32(const GemmArgs &g, bool a_ks, bool b_ks, bool wg, int epi, int max_rows, hipStream_t st, int kid) {
     // what the direct-to-LDS path relies on: 16-byte rows, whole stages of K for row-ragged products
     if (g.lda % 4 || g.ldb % 4 || g.ldc % 4 || g.N % 4 || g.N < 4) return -100;
     if (!wg && (a_ks || g.K <= 0 || g.K % F_BK)) return -100;
     if (wg && (!a_ks || !b_ks || g.M % 4 || g.M < 4)) return -100;
-    // 128 x 128 tiles where they fill the chip with two blocks per CU, 64-row tiles where they would not
-    const int rows = wg ? g.E * g.M : (g.offsets ? max_rows : g.single_rows);
-    const long tiles128 = (long)ceil_div(rows, 128) * ceil_div(g.N, 128);
-    if (tiles128 < 384) return dispatch_f32<64>(g, b_ks, wg, epi, max_rows, st, kid);
-    return dispatch_f32<128>(g, b_ks, wg, epi, max_rows, st, kid);
+    if (wg) return dispatch_f32<128, 128, 4, 2>(g, b_ks, wg, epi, max_rows, st, kid);
+    const int rows = g.offsets ? max_rows : g.single_rows;
+    const long tiles = (long)ceil_div(rows, 64) * ceil_div(g.N, 128);
+    if (tiles >= 4 * 256) return dispatch_f32<64, 128, 3, 4>(g, b_ks, wg, epi, max_rows, st, kid);
+    return dispatch_f32<64, 128, 4, 2>(g, b_ks, wg, epi, max_rows, st, kid);
 }
 
 }  // namespace mole
