@@ -491,7 +491,8 @@ int dispatch_f32(const GemmArgs &g, bool b_ks, bool wg, int epi, int max_rows, h
 //    64 x 128, 4 stages, 2 blocks per CU     -  |  -  | 127 | 124 | 131
 //    64 x 128, 4 stages, 3 blocks per CU    155 | 145 |  -  |  -  | 131
 //    64 x 128, 3 stages, 4 blocks per CU    144 | 145 |  -  |  -  | 127
-//    64 x  64, 4 stages, 4 blocks per CU     -  |  -  | 128 | 127 |  -
+//    64 x  64, 4 stages, 4 blocks per CU    154 | 163 | 128 | 127 |  -
+//    64 x  64, 3 stages, 5 blocks per CU    152 | 159 |  -  |  -  |  -
 //   128 x 128, 3 stages, 3 blocks per CU    176 | 171 |  -  |  -  | 125
 // Row-ragged products take 64 x 128 tiles: with enough of them for four blocks per CU the shallower ring, otherwise
 // two blocks per CU with the deeper one; weight gradients take 128 x 128.

@@ -379,6 +379,16 @@ def measure_layer(name, steps, warmup, with_adam=True):
     else:
         roofline = {"bound": "mfma", "kernel": dom, "achieved": kernels[dom]["tflops"], "peak": peak, "unit": "TFLOP/s",
                     "frac": round(mfma_frac, 4)}
+    # The events attached to a launch put a few microseconds of idle time between the kernels of the event-timed pass,
+    # and a chip that runs its matrix products against its power limit clocks them higher after every pause: the
+    # products measure 7-9 % shorter there than in the back-to-back steps that `value` is taken from (a rocprofv3
+    # trace of both passes shows the same kernels at both durations).  back_to_back = step time / sum of the event-timed
+    # kernel durations says by how much; frac_back_to_back is the dominant kernel's fraction at its duration inside a
+    # step, if all kernels stretch alike.
+    kernel_sum_us = sum(v["avg_us"] * v["launches_per_step"] for v in kernels.values())
+    b2b = ms_per_step * 1e3 / kernel_sum_us if kernel_sum_us > 0 else None
+    roofline.update({"back_to_back": round(b2b, 4) if b2b else None,
+                     "frac_back_to_back": round((hbm_alg_frac if hbm_bound else mfma_frac) / max(b2b, 1.0), 4) if b2b else None})
     roofline.update({"traffic": traffic, "mfma_frac": round(mfma_frac, 4), "hbm_frac_algorithmic_bytes": round(hbm_alg_frac, 4),
                      "hbm_frac_measured_traffic": round(hbm_meas_frac, 4) if hbm_meas_frac is not None else None,
                      "all_ffn_gemms_frac": round(6 * gemm_flop / (gemm_total_us * 1e-6) / 1e12 / peak, 4)})

@@ -105,18 +105,20 @@ def test_gemm_nt_gate_logits(dtype):
         assert rel_err(c, want) < (1e-5 if dtype == torch.float32 else 1e-4)   # fp32 accumulation of exact products
 
 
+@pytest.mark.parametrize("dtype,step", [(torch.bfloat16, 8), (torch.float32, 16), (torch.float32, 4)])
 @pytest.mark.parametrize("seed", range(6))
-def test_ffn_random_shapes_bf16(seed):
-    """Random expert counts, loads and (8-aligned) widths through the bf16 grouped kernels."""
+def test_ffn_random_shapes(seed, dtype, step):
+    """Random expert counts, loads and widths through the grouped kernels: 8-aligned widths for the bf16 direct-to-LDS
+    kernel, 16-aligned ones for the fp32 one (whole stages of K), 4-aligned ones for the mix of the fp32 kernel (weight
+    gradients) and the generic one (row-ragged products whose K is not whole stages)."""
     from mole_amd import hip_ops as H, _lib as L
     rng = np.random.default_rng(100 + seed)
     E = int(rng.integers(1, 40))
-    M = int(rng.integers(1, 40)) * 8
-    Fd = int(rng.integers(1, 80)) * 8
-    rows = [int(r) for r in rng.choice([0, 1, 31, 32, 33, 255, 256, 257, 320, 321, 640, 700], size=E)]
+    M = int(rng.integers(1, 40)) * step
+    Fd = int(rng.integers(1, 80)) * step
+    rows = [int(r) for r in rng.choice([0, 1, 31, 32, 33, 63, 64, 65, 127, 129, 255, 256, 257, 320, 321, 640, 700], size=E)]
     gap = int(rng.integers(0, 3))
-    print(f"ffn random seed={seed} E={E} M={M} F={Fd} rows={rows} gap={gap}", flush=True)
-    dtype = torch.bfloat16
+    print(f"ffn random seed={seed} {dtype} E={E} M={M} F={Fd} rows={rows} gap={gap}", flush=True)
     d = _make(E, M, Fd, rows, dtype, seed=seed, pad_between=gap)
     c = {k: (v.cuda() if torch.is_tensor(v) else v) for k, v in d.items()}
     off = torch.from_numpy(d["off"]).cuda(); n = torch.from_numpy(d["n"]).cuda()
