@@ -37,7 +37,7 @@ PEAK_HBM_GBS = 8000.0
 # hashes of the kernel sources the counters were read from).  A workload whose kernel sources have changed since
 # reports "traffic": null rather than a stale figure.
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
-KERNEL_SOURCES = ("MOLE/cpp/gemm256.hip", "MOLE/cpp/ffn_gemm.hip", "MOLE/cpp/gemm.h")
+KERNEL_SOURCES = ("MOLE/cpp/gemm256.hip", "MOLE/cpp/gemm_f32.hip", "MOLE/cpp/ffn_gemm.hip", "MOLE/cpp/gemm.h", "MOLE/cpp/lds_dma.h")
 # read bytes = FETCH_SIZE x 2 KiB, written bytes = WRITE_SIZE x 1 KiB on this chip (calibrated against a copy of
 # known size in the same runs, see profiles/bench_c2_hbm_traffic.txt)
 FETCH_UNIT_BYTES, WRITE_UNIT_BYTES = 2048.0, 1024.0
@@ -76,7 +76,7 @@ def ingest_counters(args):
         rows = []
         with open(path, newline="") as fh:
             for r in csv.DictReader(fh):
-                mt = re.search(r"mole::gemm(?:256)?_kernel<(.*)>\(", r["Kernel_Name"])
+                mt = re.search(r"mole::(?:\(anonymous namespace\)::)?gemm(?:256|_f32)?_kernel<(.*)>\(", r["Kernel_Name"])
                 if r.get("Counter_Name") == counter and mt:
                     targs = [a.strip() for a in mt.group(1).split(",")]
                     rows.append((int(r["Dispatch_Id"]), targs, int(r["Grid_Size"]), float(r["Counter_Value"])))
@@ -90,7 +90,7 @@ def ingest_counters(args):
             if epi == 2: out["ffn_fwd1"].append(val)
             elif epi == 1: out["ffn_fwd2"].append(val); grid_fwd2 = grid
             elif epi == 3: out["ffn_da"].append(val)
-            elif epi == 4 and "true" in targs[:4]:
+            elif epi == 4 and ("true" in targs[:4] or targs[-2] == "true"):
                 out["ffn_gw2" if n_wg % 2 == 0 else "ffn_gw1"].append(val); n_wg += 1
             elif epi == 0 and grid == grid_fwd2: out["ffn_gx"].append(val)
         return out
@@ -557,7 +557,8 @@ def main():
         # configuration 1 (fp32, the case the CPU baseline runs) on the GPU, beside the headline
         c1 = measure_layer("c1", args.steps, args.warmup, with_adam=False)
         out["c1"] = {"tokens_per_s": c1["value"], "ms_per_step": c1["ms_per_step"], "dtype": c1["dtype"],
-                     "workload": c1["config"]["workload"], "roofline": c1["roofline"], "hbm_permutes": c1["hbm_permutes"]}
+                     "workload": c1["config"]["workload"], "roofline": c1["roofline"], "hbm_permutes": c1["hbm_permutes"],
+                     "kernels_us": {n: v["avg_us"] for n, v in c1["kernels"].items()}}
     if args.workload == "c2" and not args.no_c35:
         # configurations 3 (Zipf loads, 64 experts) and 5 (256 experts, top-8) beside the headline, a few steps each
         for name in ("c3", "c5"):
