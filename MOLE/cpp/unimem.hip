@@ -12,6 +12,7 @@
 // event per slot that the copy stream waits on before overwriting the slot.
 #include "common.h"
 
+#include <algorithm>
 #include <array>
 #include <vector>
 
@@ -99,17 +100,29 @@ static int copy_experts(UniMem *u, const void *const host_src[4], int slot0, con
         std::array<hipEvent_t, 2> *tm;
         if (int rc = next_timer(u, &tm)) return rc;
         MOLE_HIP(hipEventRecord((*tm)[0], u->tran));
-        for (int j = i; j < i + run; ++j) {
+        // Small experts (below 1 MiB) with consecutive ids travel as one copy per parameter kind for up to 16 MiB at a
+        // time: their slots and their host arrays are both contiguous, and four calls per expert cost more than the
+        // bytes they move (hundreds of experts with 8-28 KB biases).  Every slot of a group still gets its own "landed"
+        // event, recorded behind the group's copies.
+        size_t expert_bytes = 0;
+        for (int p = 0; p < 4; ++p) expert_bytes += u->slot_bytes[p];
+        const int group_max = expert_bytes < ((size_t)1 << 20) ? (int)std::max<size_t>(1, ((size_t)16 << 20) / std::max<size_t>(expert_bytes, 1)) : 1;
+        for (int j = i; j < i + run;) {
+            int grp = 1;
+            while (grp < group_max && j + grp < i + run && id_of(j + grp) == id_of(j) + grp) ++grp;
             for (int p = 0; p < 4; ++p) {
                 const size_t sb = u->slot_bytes[p];
                 MOLE_HIP(hipMemcpyAsync(u->pool[p] + (size_t)(slot0 + j) * sb, (const char *)host_src[p] + (size_t)id_of(j) * sb,
-                                        sb, hipMemcpyHostToDevice, u->tran));
-                u->bytes_open += (uint64_t)sb;
+                                        sb * grp, hipMemcpyHostToDevice, u->tran));
+                u->bytes_open += (uint64_t)sb * grp;
             }
-            MOLE_HIP(hipEventRecord(u->landed_event[slot0 + j], u->tran));
-            u->landed_valid[slot0 + j] = 1;
-            u->slot_tag[slot0 + j] = tag;
-            u->slot_src[slot0 + j] = (const char *)host_src[0] + (size_t)id_of(j) * u->slot_bytes[0];
+            for (int q = j; q < j + grp; ++q) {
+                MOLE_HIP(hipEventRecord(u->landed_event[slot0 + q], u->tran));
+                u->landed_valid[slot0 + q] = 1;
+                u->slot_tag[slot0 + q] = tag;
+                u->slot_src[slot0 + q] = (const char *)host_src[0] + (size_t)id_of(q) * u->slot_bytes[0];
+            }
+            j += grp;
         }
         MOLE_HIP(hipEventRecord((*tm)[1], u->tran));
         i += run;
