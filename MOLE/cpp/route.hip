@@ -72,6 +72,62 @@ template <typename T, typename Op> __device__ __forceinline__ T group_reduce(T x
     return x;
 }
 
+// What a block does once the top-k of its BT tokens (BT <= 64) lies in LDS - s_idx / s_graw [k][BT]: expert and raw
+// gate value of every choice, s_col [4][E]: the four waves' column sums of the block's scores: the block's column sums
+// out, gate values and indices out, then each choice's in-block ranks and per-expert histogram.  Four waves.
+__device__ __forceinline__ void topk_block_tail(int BT, int S, int E, int k, int normalize, const int *s_idx,
+                                                const float *s_graw, int *s_hist, const float *s_col,
+                                                int32_t *__restrict__ idx, int32_t *__restrict__ lrank,
+                                                float *__restrict__ gates, int32_t *__restrict__ hist,
+                                                float *__restrict__ colsum, int nb) {
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int b = blockIdx.x, tok0 = b * BT;
+    __syncthreads();
+    for (int e = tid; e < E; e += RT_THREADS)
+        colsum[(size_t)b * E + e] = ((s_col[e] + s_col[E + e]) + s_col[2 * E + e]) + s_col[3 * E + e];
+
+    // ---- gate values and indices out (threads 0..BT-1 = the block's tokens) -------------
+    const int token = tok0 + tid;
+    const bool tv = tid < BT && token < S;
+    if (tv) {
+        float denom = 0.f;
+        for (int j = 0; j < k; ++j) denom += s_graw[j * BT + tid];  // left to right, fp32
+        const float den = denom < FP32_EPS ? FP32_EPS : denom;
+        for (int j = 0; j < k; ++j) {
+            float gv = s_graw[j * BT + tid];
+            if (k > 1 && normalize) gv = gv / den;
+            gates[(size_t)j * S + token] = gv;
+            idx[(size_t)j * S + token] = s_idx[j * BT + tid];
+        }
+    }
+
+    // ---- in-block ranks per choice (lane = token; wave w takes choices w, w + 4, ...) ------
+    // Each wave works on a histogram of its own, so the choices proceed side by side without block barriers
+    // (the loop over distinct experts is a serial chain of ballots: with one wave doing all k choices it was the
+    // longest part of the kernel at top-8).
+    const uint64_t lt_mask = (1ull << lane) - 1ull;
+    int *my_hist = s_hist + w * E;
+    const int ctoken = tok0 + lane;
+    const bool cv = lane < BT && ctoken < S;
+    for (int j = w; j < k; j += RT_THREADS / WAVE) {
+        for (int e = lane; e < E; e += WAVE) my_hist[e] = 0;
+        const int e = cv ? s_idx[j * BT + lane] : -1;
+        int rank = 0;
+        uint64_t remaining = __ballot(cv);
+        while (remaining) {
+            const int leader = __ffsll((unsigned long long)remaining) - 1;
+            const int e0 = __shfl(e, leader, WAVE);
+            const uint64_t m = __ballot(cv && e == e0);
+            if (cv && e == e0) rank = __popcll(m & lt_mask);
+            if (lane == leader) my_hist[e0] = __popcll(m);
+            remaining &= ~m;
+        }
+        if (cv) lrank[(size_t)j * S + ctoken] = rank;
+        // (the histogram is written and read by this wave only: program order is enough)
+        for (int e2 = lane; e2 < E; e2 += WAVE) hist[((size_t)j * E + e2) * nb + b] = my_hist[e2];
+    }
+}
+
 template <int VPL>
 __global__ __launch_bounds__(RT_THREADS) void route_topk_kernel(
     const float *__restrict__ scores, int S, int E, int k, int logG, int normalize,
@@ -148,50 +204,7 @@ __global__ __launch_bounds__(RT_THREADS) void route_topk_kernel(
         const int e = g + (r << logG);
         if (tg == 0 && e < E) s_col[w * E + e] = c;
     }
-    __syncthreads();
-    for (int e = tid; e < E; e += RT_THREADS)
-        colsum[(size_t)b * E + e] = ((s_col[e] + s_col[E + e]) + s_col[2 * E + e]) + s_col[3 * E + e];
-
-    // ---- phase B: gate values and indices out (threads 0..63 = the block's tokens) -------------
-    const int token = tok0 + tid;
-    const bool tv = tid < RT_TOKENS && token < S;
-    if (tv) {
-        float denom = 0.f;
-        for (int j = 0; j < k; ++j) denom += s_graw[j * RT_TOKENS + tid];  // left to right, fp32
-        const float den = denom < FP32_EPS ? FP32_EPS : denom;
-        for (int j = 0; j < k; ++j) {
-            float gv = s_graw[j * RT_TOKENS + tid];
-            if (k > 1 && normalize) gv = gv / den;
-            gates[(size_t)j * S + token] = gv;
-            idx[(size_t)j * S + token] = s_idx[j * RT_TOKENS + tid];
-        }
-    }
-
-    // ---- phase C: in-block ranks per choice (lane = token; wave w takes choices w, w + 4, ...) ------
-    // Each wave works on a histogram of its own, so the choices proceed side by side without block barriers
-    // (the loop over distinct experts is a serial chain of ballots: with one wave doing all k choices it was the
-    // longest part of the kernel at top-8).
-    const uint64_t lt_mask = (1ull << lane) - 1ull;
-    int *my_hist = s_hist + w * E;
-    const int ctoken = tok0 + lane;
-    const bool cv = ctoken < S;
-    for (int j = w; j < k; j += RT_THREADS / WAVE) {
-        for (int e = lane; e < E; e += WAVE) my_hist[e] = 0;
-        const int e = cv ? s_idx[j * RT_TOKENS + lane] : -1;
-        int rank = 0;
-        uint64_t remaining = __ballot(cv);
-        while (remaining) {
-            const int leader = __ffsll((unsigned long long)remaining) - 1;
-            const int e0 = __shfl(e, leader, WAVE);
-            const uint64_t m = __ballot(cv && e == e0);
-            if (cv && e == e0) rank = __popcll(m & lt_mask);
-            if (lane == leader) my_hist[e0] = __popcll(m);
-            remaining &= ~m;
-        }
-        if (cv) lrank[(size_t)j * S + ctoken] = rank;
-        // (the histogram is written and read by this wave only: program order is enough)
-        for (int e2 = lane; e2 < E; e2 += WAVE) hist[((size_t)j * E + e2) * nb + b] = my_hist[e2];
-    }
+    topk_block_tail(RT_TOKENS, S, E, k, normalize, s_idx, s_graw, s_hist, s_col, idx, lrank, gates, hist, colsum, nb);
 }
 
 // one wave per (choice, expert) pair: exclusive prefix over blocks, total into counts
@@ -368,12 +381,13 @@ __global__ __launch_bounds__(FIN_THREADS) void route_finish_kernel(
 __global__ __launch_bounds__(256) void route_finalize_kernel(
     const int32_t *__restrict__ idx, const int32_t *__restrict__ hist, const int32_t *__restrict__ basej,
     const int32_t *__restrict__ offsets, const int32_t *__restrict__ capacity, int S, int E, int k, int nb,
-    int32_t *__restrict__ loc /* in: in-block rank, out: location */, int32_t *__restrict__ row) {
+    int bt /* tokens per histogram block */, int32_t *__restrict__ loc /* in: in-block rank, out: location */,
+    int32_t *__restrict__ row) {
     const size_t p = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (p >= (size_t)k * S) return;
     const int j = (int)(p / S), i = (int)(p % S);
     const int e = idx[p];
-    const int b = i / RT_TOKENS;
+    const int b = i / bt;
     const int l = basej[j * E + e] + hist[((size_t)j * E + e) * nb + b] + loc[p];
     loc[p] = l;
     row[p] = l < capacity[0] ? offsets[e] + l : -1;
@@ -390,6 +404,42 @@ extern "C" size_t mole_route_workspace_bytes(int S, int E, int k) {
     const size_t nb = (size_t)ceil_div(S > 0 ? S : 1, RT_TOKENS);
     return align256(nb * k * E * sizeof(int32_t)) + align256((size_t)k * E * sizeof(int32_t)) +
            align256(nb * E * sizeof(float)) + align256((size_t)COLSUM_SLICES * E * sizeof(float));
+}
+
+// The stages of the routing behind the per-block top-k: scan of the histograms over blocks, counts / capacity /
+// offsets / l_aux, then locations and destination rows.  bt: tokens per histogram block.
+static int route_after_topk(int32_t *hist, int32_t *basej, float *colsum, float *colpart, int nb, int bt, int S, int E, int k,
+                            double capacity_factor, int alignment, int layout, const int32_t *idx, int32_t *loc,
+                            int32_t *row, int32_t *counts, int32_t *kept_rows, int32_t *offsets, int32_t *capacity,
+                            float *l_aux, hipStream_t st) {
+    const int npairs = k * E;
+    const bool scan_in_finish = (long long)npairs * nb <= 8192;    // small enough for one block: saves a launch
+    if (!scan_in_finish) {
+        const int scan_blocks = ceil_div(npairs, 4);
+        hipLaunchKernelGGL(route_scan_kernel, dim3(scan_blocks + COLSUM_SLICES * ceil_div(E, 256)), dim3(256), 0, st, hist,
+                           nb, npairs, counts, scan_blocks, colsum, E, colpart);
+        MOLE_LAUNCH_CHECK();
+    }
+
+    const int spe = (S + E - 1) / E;
+    const int cf_sign = capacity_factor > 0. ? 1 : (capacity_factor < 0. ? -1 : 0);
+    // int(cf * spe) of the Python reference: the product is taken in double precision
+    const double prod = (capacity_factor < 0. ? -capacity_factor : capacity_factor) * (double)spe;
+    const int cap_bound = k * (int)prod;
+    // (when the scan kernel ran, it also folded the column sums: the finish then adds its COLSUM_SLICES rows)
+    hipLaunchKernelGGL(route_finish_kernel, dim3(1), dim3(FIN_THREADS), 0, st, counts,
+                       scan_in_finish ? colsum : colpart, scan_in_finish ? nb : min(nb, COLSUM_SLICES), S, E, k, cf_sign,
+                       cap_bound, alignment, layout, basej, kept_rows, offsets, capacity, l_aux,
+                       scan_in_finish ? hist : (int32_t *)nullptr);
+    MOLE_LAUNCH_CHECK();
+
+    if (S > 0) {
+        const size_t n = (size_t)k * S;
+        hipLaunchKernelGGL(route_finalize_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, idx, hist,
+                           basej, offsets, capacity, S, E, k, nb, bt, loc, row);
+        MOLE_LAUNCH_CHECK();
+    }
+    return 0;
 }
 
 template <int VPL>
@@ -439,34 +489,8 @@ extern "C" int mole_route(const float *scores, int S, int E, int k, double capac
     else launch_topk<16>(scores, S, E, k, logG, normalize_gate, idx, loc, gates, hist, colsum, nb, st);
     MOLE_LAUNCH_CHECK();
 
-    const int npairs = k * E;
-    const bool scan_in_finish = (long long)npairs * nb <= 8192;    // small enough for one block: saves a launch
-    if (!scan_in_finish) {
-        const int scan_blocks = ceil_div(npairs, 4);
-        hipLaunchKernelGGL(route_scan_kernel, dim3(scan_blocks + COLSUM_SLICES * ceil_div(E, 256)), dim3(256), 0, st, hist,
-                           nb, npairs, counts, scan_blocks, colsum, E, colpart);
-        MOLE_LAUNCH_CHECK();
-    }
-
-    const int spe = (S + E - 1) / E;
-    const int cf_sign = capacity_factor > 0. ? 1 : (capacity_factor < 0. ? -1 : 0);
-    // int(cf * spe) of the Python reference: the product is taken in double precision
-    const double prod = (capacity_factor < 0. ? -capacity_factor : capacity_factor) * (double)spe;
-    const int cap_bound = k * (int)prod;
-    // (when the scan kernel ran, it also folded the column sums: the finish then adds its COLSUM_SLICES rows)
-    hipLaunchKernelGGL(route_finish_kernel, dim3(1), dim3(FIN_THREADS), 0, st, counts,
-                       scan_in_finish ? colsum : colpart, scan_in_finish ? nb : min(nb, COLSUM_SLICES), S, E, k, cf_sign,
-                       cap_bound, alignment, layout, basej, kept_rows, offsets, capacity, l_aux,
-                       scan_in_finish ? hist : (int32_t *)nullptr);
-    MOLE_LAUNCH_CHECK();
-
-    if (S > 0) {
-        const size_t n = (size_t)k * S;
-        hipLaunchKernelGGL(route_finalize_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, idx, hist,
-                           basej, offsets, capacity, S, E, k, nb, loc, row);
-        MOLE_LAUNCH_CHECK();
-    }
-    return 0;
+    return route_after_topk(hist, basej, colsum, colpart, nb, RT_TOKENS, S, E, k, capacity_factor, alignment, layout, idx, loc,
+                            row, counts, kept_rows, offsets, capacity, l_aux, st);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -722,10 +746,19 @@ typedef float gate_f32x4 __attribute__((ext_vector_type(4)));
 // the instruction's layout touches 16 rows with 64 bytes each; staged, it fetches 512-byte pieces of two rows (at
 // KSTEPS 8), and the fragments are 16-byte LDS reads (rows 16 bytes longer than their data: the 16 rows of a read
 // fall into distinct banks).  A wave stages and reads its own rows only.
-template <int EG, int KSTEPS, int TG, bool STAGE>   // TG groups of 16 tokens per block: Wg is read once for all of them
+// ROUTE: the block goes on to the first stage of the routing for its 16 TG tokens - top-k, gate values, in-block
+// ranks and per-expert histograms, the block's column sums for l_aux - while a token's scores are still in the 16
+// lanes that formed them (the layout route_topk_kernel works in: lane j of the group holds experts j, 16 + j, ...).
+// The scores are written out as well (the backward needs them) but not read back: one kernel and 4 S E bytes less.
+struct GateRoute {
+    int k, normalize, nb;
+    int32_t *idx, *lrank, *hist;
+    float *gates, *colsum;
+};
+template <int EG, int KSTEPS, int TG, bool STAGE, bool ROUTE = false>   // TG groups of 16 tokens per block: Wg is read once for all of them
 __global__ __launch_bounds__(256) void gate_fwd_kernel(const bf16_t *__restrict__ x, const float *__restrict__ wg,
                                                        const float *__restrict__ bias, int S, int E, int M,
-                                                       float *__restrict__ scores) {
+                                                       float *__restrict__ scores, const GateRoute rt) {
     constexpr int RB = KSTEPS * 64, RS = RB + 16;               // staged row: bytes of data, bytes of stride
     constexpr int LPR = RB / 16, RPI = 64 / LPR;                // lanes per row, rows per load instruction
     constexpr int PART_BYTES = 4 * 16 * TG * (EG * 16 + 1) * 4;
@@ -832,6 +865,15 @@ __global__ __launch_bounds__(256) void gate_fwd_kernel(const bf16_t *__restrict_
             for (int r = 0; r < 4; ++r) part[wave][16 * tg + 4 * kq + r][g * 16 + r16] = acc[tg][g][r];
     __syncthreads();
     const int j = threadIdx.x & 15;               // 16 lanes per token
+    constexpr int BT = 16 * TG;
+    // routing: [k][BT] experts and raw gate values, four histograms, four rows of column sums - behind the staging area
+    int *s_idx = reinterpret_cast<int *>(s_dyn + STAGE_BYTES);
+    float *s_graw = reinterpret_cast<float *>(s_idx + (ROUTE ? rt.k : 0) * BT);
+    int *s_hist = reinterpret_cast<int *>(s_graw + (ROUTE ? rt.k : 0) * BT);
+    float *s_col = reinterpret_cast<float *>(s_hist + 4 * E);
+    float colacc[EG];
+#pragma unroll
+    for (int g = 0; g < EG; ++g) colacc[g] = 0.f;
 #pragma unroll
     for (int tg = 0; tg < TG; ++tg) {
         const int t = 16 * tg + (threadIdx.x >> 4);
@@ -855,8 +897,53 @@ __global__ __launch_bounds__(256) void gate_fwd_kernel(const bf16_t *__restrict_
 #pragma unroll
         for (int g = 0; g < EG; ++g) {
             const int e = g * 16 + j;
-            if (token < S && e < E) scores[(size_t)token * E + e] = v[g] / sum;
+            v[g] = v[g] / sum;
+            if (token < S && e < E) scores[(size_t)token * E + e] = v[g];
         }
+        if constexpr (ROUTE) {
+            // the k rounds of route_topk_kernel on the token's scores (the same keys, the same tie rule)
+            uint32_t key[EG];
+#pragma unroll
+            for (int g = 0; g < EG; ++g) {
+                const bool ok = token < S && g * 16 + j < E;
+                const float sv = __uint_as_float(__float_as_uint(v[g]) & (ok ? 0xffffffffu : 0u));
+                colacc[g] += sv;
+                key[g] = ok ? topk_key(sv) : 0u;
+            }
+            for (int c = 0; c < rt.k; ++c) {
+                uint32_t best = key[0];
+#pragma unroll
+                for (int g = 1; g < EG; ++g) best = max(best, key[g]);
+                const uint32_t top = group_reduce(best, 4, [](uint32_t a, uint32_t b2) { return max(a, b2); });
+                int cand = INT_MAX;
+#pragma unroll
+                for (int g = EG - 1; g >= 0; --g)
+                    if (key[g] == top) cand = j + (g << 4);                // ends on the lane's lowest such expert
+                if (top == 0u) cand = INT_MAX;                             // nothing available (a token past the end)
+                const int bi = group_reduce(cand, 4, [](int a, int b2) { return min(a, b2); });
+                const bool mine = bi != INT_MAX && (bi & 15) == j;
+#pragma unroll
+                for (int g = 0; g < EG; ++g)
+                    if (mine && (bi >> 4) == g) key[g] = 0u;
+                if (j == 0 && token < S) {
+                    s_idx[c * BT + t] = bi;
+                    s_graw[c * BT + t] = topk_unkey(top);
+                }
+            }
+        }
+    }
+    if constexpr (ROUTE) {
+        // column sums of the scores: fold the wave's four token groups, then (in the tail) the four waves
+#pragma unroll
+        for (int g = 0; g < EG; ++g) {
+            float c = colacc[g];
+            c += __shfl_xor(c, 16, WAVE);
+            c += __shfl_xor(c, 32, WAVE);
+            const int e = g * 16 + j;
+            if (lane < 16 && e < E) s_col[wave * E + e] = c;
+        }
+        topk_block_tail(BT, S, E, rt.k, rt.normalize, s_idx, s_graw, s_hist, s_col, rt.idx, rt.lrank, rt.gates, rt.hist,
+                        rt.colsum, rt.nb);
     }
 }
 
@@ -887,6 +974,61 @@ extern "C" int mole_softmax_fwd(const float *logits, const float *logit_bias, in
     return 0;
 }
 
+// dynamic LDS of gate_fwd_kernel<1, 4, 2, true>: the staged token rows (four waves x 32 rows of 4 x 64 + 16 bytes)
+static constexpr unsigned GATE_STAGE_LDS = 4 * 32 * (4 * 64 + 16);
+// tokens per block of the fused gate + routing kernels (TG = 2)
+static constexpr int GATE_ROUTE_TOKENS = 32;
+
+extern "C" size_t mole_gate_route_workspace_bytes(int S, int E, int k) {
+    if (S < 0 || E <= 0 || k <= 0) return 0;
+    const size_t nb = (size_t)ceil_div(S > 0 ? S : 1, GATE_ROUTE_TOKENS);
+    return align256(nb * k * E * sizeof(int32_t)) + align256((size_t)k * E * sizeof(int32_t)) +
+           align256(nb * E * sizeof(float)) + align256((size_t)COLSUM_SLICES * E * sizeof(float));
+}
+
+extern "C" int mole_gate_route(const void *x, int dtype, const float *wg, const float *logit_bias, int S, int E, int M,
+                               int k, double capacity_factor, int normalize_gate, int alignment, int layout, float *scores,
+                               int32_t *idx, int32_t *loc, float *gates, int32_t *row, int32_t *counts,
+                               int32_t *kept_rows, int32_t *offsets, int32_t *capacity, float *l_aux, void *workspace,
+                               size_t workspace_bytes, mole_stream_t stream) {
+    MOLE_REQUIRE(dtype == MOLE_BF16 && S >= 1 && E >= 1 && E <= 32 && M >= 128 && M % 128 == 0,
+                 "mole_gate_route: needs bf16 tokens, M a multiple of 128 and at most 32 experts (S=%d E=%d M=%d dtype=%d); "
+                 "other shapes: mole_gate_fwd (or mole_gemm_nt + mole_softmax_fwd), then mole_route", S, E, M, dtype);
+    MOLE_REQUIRE(k >= 1 && k <= MOLE_MAX_TOPK && k <= E, "mole_gate_route: need 1 <= k <= min(E, %d) (k=%d E=%d)", MOLE_MAX_TOPK, k, E);
+    MOLE_REQUIRE(alignment >= 1, "mole_gate_route: alignment must be >= 1");
+    MOLE_REQUIRE(layout == MOLE_LAYOUT_PADDED || layout == MOLE_LAYOUT_RAGGED, "mole_gate_route: bad layout %d", layout);
+    MOLE_REQUIRE(x && wg && scores && idx && loc && gates && row && counts && kept_rows && offsets && capacity && workspace,
+                 "mole_gate_route: null pointer");
+    MOLE_REQUIRE((long long)S * k < INT_MAX, "mole_gate_route: S*k too large");
+    if (workspace_bytes < mole_gate_route_workspace_bytes(S, E, k)) {
+        set_error("mole_gate_route: workspace of %zu bytes, need %zu", workspace_bytes, mole_gate_route_workspace_bytes(S, E, k));
+        return MOLE_E_WORKSPACE;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    const int nb = ceil_div(S, GATE_ROUTE_TOKENS);
+    char *ws = (char *)workspace;
+    int32_t *hist = (int32_t *)ws;
+    ws += align256((size_t)nb * k * E * sizeof(int32_t));
+    int32_t *basej = (int32_t *)ws;
+    ws += align256((size_t)k * E * sizeof(int32_t));
+    float *colsum = (float *)ws;
+    ws += align256((size_t)nb * E * sizeof(float));
+    float *colpart = (float *)ws;
+    const GateRoute rt{k, normalize_gate, nb, idx, loc, hist, gates, colsum};
+    const unsigned route_lds = (unsigned)((size_t)k * GATE_ROUTE_TOKENS * 8 + (size_t)E * 4 * 4 * 2);
+    const bf16_t *xb = (const bf16_t *)x;
+    if (E <= 16)
+        timed_launch(MOLE_K_GATE_FWD, gate_fwd_kernel<1, 4, 2, true, true>, dim3(nb), dim3(256), GATE_STAGE_LDS + route_lds, st, xb, wg,
+                     logit_bias, S, E, M, scores, rt);
+    else
+        timed_launch(MOLE_K_GATE_FWD, gate_fwd_kernel<2, 4, 2, false, true>, dim3(nb), dim3(256), route_lds, st, xb, wg, logit_bias, S,
+                     E, M, scores, rt);
+    MOLE_LAUNCH_CHECK();
+    ScopedTiming timing(MOLE_K_ROUTE, st);
+    return route_after_topk(hist, basej, colsum, colpart, nb, GATE_ROUTE_TOKENS, S, E, k, capacity_factor, alignment, layout, idx,
+                            loc, row, counts, kept_rows, offsets, capacity, l_aux, st);
+}
+
 extern "C" int mole_gate_fwd(const void *x, int dtype, const float *wg, const float *logit_bias, int S, int E, int M,
                              float *scores, mole_stream_t stream) {
     MOLE_REQUIRE(S >= 0 && E >= 1 &&
@@ -912,11 +1054,12 @@ extern "C" int mole_gate_fwd(const void *x, int dtype, const float *wg, const fl
     const dim3 grid(ceil_div(S, eg <= 2 ? 32 : 16));
     // (16 experts or fewer: staged, 34 KB of LDS; 10.6 against 11.6 us straight from memory at 16384 x 1024, and 11.1
     // with the whole quarter row in one round of eight steps)
-    if (eg == 1) timed_launch(MOLE_K_GATE_FWD, gate_fwd_kernel<1, 4, 2, true>, grid, dim3(256), 4 * 32 * (4 * 64 + 16), st, xb, wg, logit_bias, S, E, M, scores);
-    else if (eg == 2) timed_launch(MOLE_K_GATE_FWD, gate_fwd_kernel<2, 4, 2, false>, grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores);
-    else if (eg <= 4) timed_launch(MOLE_K_GATE_FWD, gate_fwd_kernel<4, 4, 1, false>, grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores);
-    else if (eg <= 8) timed_launch(MOLE_K_GATE_FWD, gate_fwd_kernel<8, 4, 1, false>, grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores);
-    else timed_launch(MOLE_K_GATE_FWD, gate_fwd_kernel<16, 2, 1, false>, grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores);
+    const GateRoute none{};
+    if (eg == 1) timed_launch(MOLE_K_GATE_FWD, gate_fwd_kernel<1, 4, 2, true>, grid, dim3(256), GATE_STAGE_LDS, st, xb, wg, logit_bias, S, E, M, scores, none);
+    else if (eg == 2) timed_launch(MOLE_K_GATE_FWD, gate_fwd_kernel<2, 4, 2, false>, grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores, none);
+    else if (eg <= 4) timed_launch(MOLE_K_GATE_FWD, gate_fwd_kernel<4, 4, 1, false>, grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores, none);
+    else if (eg <= 8) timed_launch(MOLE_K_GATE_FWD, gate_fwd_kernel<8, 4, 1, false>, grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores, none);
+    else timed_launch(MOLE_K_GATE_FWD, gate_fwd_kernel<16, 2, 1, false>, grid, dim3(256), 0, st, xb, wg, logit_bias, S, E, M, scores, none);
     MOLE_LAUNCH_CHECK();
     return 0;
 }

@@ -148,6 +148,20 @@ int mole_route(const float *scores, int S, int E, int k, double capacity_factor,
                int32_t *counts, int32_t *kept_rows, int32_t *offsets, int32_t *capacity,
                float *l_aux, void *workspace, size_t workspace_bytes, mole_stream_t stream);
 
+/* mole_gate_fwd and mole_route in one call for small gates on bf16 tokens (E <= 32, M a multiple of 128, S >= 1): the gate
+ * kernel goes on to the routing's first stage - top-k, gate values, in-block ranks, histograms - while a token's
+ * scores are still in the lanes that formed them, so the routing starts one kernel later and never reads the scores
+ * back (MOLE/utils/Ugate.py:11-14 followed by extract_critical, MOLE/moe/layer.py:442-446).  Arguments and results are
+ * those of the two calls; scores [S,E] is an output here.  Every result equals the two calls' bit for bit except
+ * l_aux, whose column sums are added in another order (32 tokens per block instead of 64).  Other shapes are rejected:
+ * the caller runs the two calls. */
+size_t mole_gate_route_workspace_bytes(int S, int E, int k);
+int mole_gate_route(const void *x, int dtype, const float *wg, const float *logit_bias, int S, int E, int M, int k,
+                    double capacity_factor, int normalize_gate, int alignment, int layout, float *scores,
+                    int32_t *idx, int32_t *loc, float *gates, int32_t *row, int32_t *counts, int32_t *kept_rows,
+                    int32_t *offsets, int32_t *capacity, float *l_aux, void *workspace, size_t workspace_bytes,
+                    mole_stream_t stream);
+
 /* mole_route for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc): the same routing with the same outputs, but without the workspace argument.
  * No counterpart in the reference.  The scratch the routing kernels need (per-block histograms, per-choice bases,

@@ -40,6 +40,9 @@ _SIGNATURES = {
     "mole_route_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "mole_route": (c_int, [_P, c_int, c_int, c_int, c_double, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P,
                            _P, _P, c_size_t, _P]),
+    "mole_gate_route_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "mole_gate_route": (c_int, [_P, c_int, _P, _P, c_int, c_int, c_int, c_int, c_double, c_int, c_int, c_int, _P, _P, _P, _P, _P,
+                                _P, _P, _P, _P, _P, _P, c_size_t, _P]),
     "mole_route_static_max_bytes": (c_size_t, []),
     "mole_route_static": (c_int, [_P, c_int, c_int, c_int, c_double, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P,
                                   _P, _P]),

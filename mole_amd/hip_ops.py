@@ -200,6 +200,44 @@ def route(scores: torch.Tensor, top_k: int, capacity_factor: float = 1.0, normal
     return Route(S, E, k, layout, idx, loc, gates, row, counts, kept, offsets, cap, l_aux, normalize_gate)
 
 
+def gate_route_fused(x: torch.Tensor, wg: torch.Tensor) -> bool:
+    """Whether gate_route() takes (x, wg) in its one-call form."""
+    return (x.dtype == torch.bfloat16 and wg.dtype == torch.float32 and wg.shape[0] <= 32 and x.shape[1] % 128 == 0
+            and x.shape[0] >= 1)
+
+
+def gate_route(x: torch.Tensor, wg: torch.Tensor, logit_bias: Optional[torch.Tensor], top_k: int,
+               capacity_factor: float = 1.0, normalize_gate: bool = True, alignment: int = 1,
+               layout: int = L.LAYOUT_RAGGED):
+    """(scores, Route) = (gate_fwd(x, wg, logit_bias), route(scores, ...)): for small gates on bf16 tokens one call whose
+    gate kernel also does the routing's first stage (mole_gate_route), otherwise the two calls."""
+    _dev(x), _dev(wg)
+    if not gate_route_fused(x, wg):
+        scores = gate_fwd(x, wg, logit_bias)
+        return scores, route(scores, top_k, capacity_factor, normalize_gate, alignment, layout)
+    S, M = x.shape
+    E = wg.shape[0]
+    k = min(int(top_k), E)
+    dev = x.device
+    i32 = dict(dtype=torch.int32, device=dev)
+    scores = torch.empty(S, E, dtype=torch.float32, device=dev)
+    idx, loc, row = (torch.empty(k, S, **i32) for _ in range(3))
+    gates = torch.empty(k, S, dtype=torch.float32, device=dev)
+    meta = torch.empty(k * E + E + (E + 1) + 1, **i32)
+    counts = meta[:k * E].view(k, E)
+    kept = meta[k * E:k * E + E]
+    offsets = meta[k * E + E:k * E + 2 * E + 1]
+    cap = meta[k * E + 2 * E + 1:]
+    l_aux = torch.empty(1, dtype=torch.float32, device=dev)
+    nbytes = L.lib().mole_gate_route_workspace_bytes(S, E, k)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    L.check(L.lib().mole_gate_route(L.ptr(x), L.dtype_code(x.dtype), L.ptr(wg), L.ptr(logit_bias), S, E, M, k,
+                                    float(capacity_factor), int(normalize_gate), int(alignment), int(layout), L.ptr(scores),
+                                    L.ptr(idx), L.ptr(loc), L.ptr(gates), L.ptr(row), L.ptr(counts), L.ptr(kept), L.ptr(offsets),
+                                    L.ptr(cap), L.ptr(l_aux), L.ptr(ws), nbytes, L.stream()), "mole_gate_route")
+    return scores, Route(S, E, k, layout, idx, loc, gates, row, counts, kept, offsets, cap, l_aux, normalize_gate)
+
+
 def dispatch_fwd(x: torch.Tensor, row: torch.Tensor, total_rows: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     _dev(x), _dev(row)
     S, M = x.shape

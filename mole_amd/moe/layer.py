@@ -65,8 +65,7 @@ class _FusedMoE(torch.autograd.Function):
         ctx.set_materialize_grads(False)
         S, M = x.shape
         k = min(m.topk, m.total_experts)
-        scores = Ugate.gate_scores(x, wg, m.gate[0].logit_bias)
-        r = H.route(scores, k, capacity_factor, m.normalize_gate, 1, L.LAYOUT_RAGGED)
+        scores, r = Ugate.gate_scores_route(x, wg, m.gate[0].logit_bias, k, capacity_factor, m.normalize_gate)
         rows = S * k
         if capacity_factor > 0:
             E = m.total_experts

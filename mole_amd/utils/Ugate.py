@@ -34,6 +34,14 @@ def gate_scores(x: torch.Tensor, weight: torch.Tensor, logit_bias=None) -> torch
     return H.gate_fwd(x.detach().contiguous(), weight.detach().contiguous(), logit_bias)
 
 
+def gate_scores_route(x: torch.Tensor, weight: torch.Tensor, logit_bias, top_k: int, capacity_factor: float,
+                      normalize_gate: bool):
+    """(gate_scores(x, weight, logit_bias), the routing of those scores on the ragged layout): what MOLETopk.forward and
+    tutel's extract_critical do between them (MOLE/moe/layer.py:442-446), in one library call where it offers one."""
+    return H.gate_route(x.detach().contiguous(), weight.detach().contiguous(), logit_bias, top_k, capacity_factor,
+                        normalize_gate)
+
+
 class MOLETopk(torch.nn.Module):
     def __init__(self, model_dim, total_experts) -> None:
         super().__init__()

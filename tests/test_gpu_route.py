@@ -194,3 +194,38 @@ def test_route_random_sweep():
         align = int(rng.choice([1, 1, 1, 2, 8]))
         print(f"route sweep {case}: S={S} E={E} k={k} cf={cf} align={align}", flush=True)
         _compare(zipf_scores(S, E, seed=case, ties=(case % 5 == 0)), k, cf, bool(case % 2), normalize=bool(case % 3), alignment=align)
+
+
+@pytest.mark.parametrize("S,E,M,k,cf,bias,normalize,ragged", [
+    (16384, 16, 1024, 1, 1.25, False, True, True), (1000, 8, 256, 2, 1.0, True, True, True),
+    (33, 20, 128, 2, 0.0, False, True, False), (777, 32, 384, 4, 0.5, True, False, True),
+    (64, 3, 128, 3, 1.0, False, True, True), (1, 5, 128, 1, 1.0, False, True, True),
+    (4095, 17, 256, 5, -0.5, True, True, False), (8192, 32, 2048, 2, 0.0, False, True, True),
+])
+def test_gate_and_route_in_one_call(S, E, M, k, cf, bias, normalize, ragged):
+    """mole_gate_route (the gate kernel does the routing's first stage on the scores it has just formed) against
+    mole_gate_fwd followed by mole_route: the same scores and the same routing, bit for bit; l_aux, whose column sums
+    are taken over blocks of 32 instead of 64 tokens, to fp32 rounding.  The two-call path is the one compared with the
+    oracle above; duplicated Wg rows make exact ties in every token's scores."""
+    from mole_amd import hip_ops as H, _lib as L
+    print(f"gate_route S={S} E={E} M={M} k={k} cf={cf} bias={bias}", flush=True)
+    g = torch.Generator().manual_seed(S * 7 + E)
+    x = torch.randn(S, M, generator=g).bfloat16().cuda()
+    wg = torch.randn(E, M, generator=g) * 0.05
+    if E >= 4:
+        wg[E - 1] = wg[0]                      # exact ties: the lower index must win in both paths
+    wg = wg.cuda()
+    lb = (torch.randn(E, generator=g) * 0.5).cuda() if bias else None
+    if bias and E >= 4:
+        lb[E - 1] = lb[0]
+    layout = L.LAYOUT_RAGGED if ragged else L.LAYOUT_PADDED
+    assert H.gate_route_fused(x, wg)
+    scores, r = H.gate_route(x, wg, lb, k, cf, normalize, 1, layout)
+    scores2 = H.gate_fwd(x, wg, lb)
+    r2 = H.route(scores2, k, cf, normalize, 1, layout)
+    assert torch.equal(scores, scores2)
+    a, b = crit_to_numpy(r), crit_to_numpy(r2)
+    for name in ("idx", "loc", "gates", "row", "counts", "kept", "offsets"):
+        np.testing.assert_array_equal(a[name], b[name], err_msg=name)
+    assert a["capacity"] == b["capacity"]
+    assert abs(a["l_aux"] - b["l_aux"]) <= 1e-5 * max(1.0, abs(b["l_aux"]))
