@@ -3,7 +3,7 @@
 
 A step is one forward + backward of one MoE layer (gate, routing, dispatch, grouped expert FFN,
 combine, and all of their gradients) over one batch of synthetic tokens resident in HBM.  The
-default workload is BASELINE.json's configuration 2: Switch-style layer, bf16 with fp32 accumulation,
+default workload is configuration 2 of the benchmark set (the one the headline metric is quoted on): Switch-style layer, bf16 with fp32 accumulation,
 16384 tokens x 1024, 16 experts of 1024 -> 4096 -> 1024, top-1, capacity factor 1.25.
 
 Prints ONE JSON line: the metric (tokens/s), the roofline of the dominant kernel measured with HIP
@@ -155,7 +155,7 @@ def step(m, x, dy, cf):
 
 
 def cpu_baseline(budget_s=12.0):
-    """The CPU oracle's layer (fp32 torch on the host cores), forward + backward, on BASELINE configuration 1
+    """The CPU oracle's layer (fp32 torch on the host cores), forward + backward, on configuration 1 of the benchmark set
     exactly as specified: 4096 tokens x 512 ~N(0,1), gate 512 -> 8 ~N(0,0.02), top-2, experts
     Linear(512 -> 2048) + GELU + Linear(2048 -> 512) ~N(0,0.02), fp32, seed 0, MSE against zero, the reference's
     default capacity factor 1.0.  Three warm-up steps, then at least ten timed ones (until budget_s), median."""
@@ -194,7 +194,7 @@ def cpu_baseline(budget_s=12.0):
 
 
 def bench_offloaded_stack(args):
-    """BASELINE configuration 4: a stack of MoE layers whose experts all live in pinned host memory and
+    """Configuration 4 of the benchmark set: a stack of MoE layers whose experts all live in pinned host memory and
     stream through the device slot pool (32 experts of 4096 -> 14336 -> 4096, bf16: 235 MB per expert,
     7.5 GB per layer; 4096 tokens x 4096, top-2, no drop).  The step is PCIe bound by construction, so
     the figures of interest are the copy stream's host-to-device rate and how much of the step the

@@ -168,7 +168,7 @@ int mole_gate_route(const void *x, int dtype, const float *wg, const float *logi
  * column sums of the scores) lives in a static device array of mole_route_static_max_bytes() = 8 MiB inside the
  * library, one copy per GPU, held until the process ends; the call allocates nothing, on the host side neither.
  * Problem sizes whose mole_route_workspace_bytes(S, E, k) exceeds the array are rejected with MOLE_E_WORKSPACE
- * (the five BASELINE configurations need at most 4.6 MiB).  All calls on one GPU share the array: calls that
+ * (the five configurations of the benchmark set need at most 4.6 MiB).  All calls on one GPU share the array: calls that
  * overlap on one GPU (two streams, two threads) race on it and must be serialised by the caller.  The first
  * call on a device looks up the array's address (hipGetSymbolAddress) and must not run under stream capture. */
 size_t mole_route_static_max_bytes(void);

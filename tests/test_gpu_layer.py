@@ -220,7 +220,7 @@ def test_pool_guards_and_reserve():
 
 
 def test_layer_config1_exact():
-    """BASELINE config 1 as specified: 4096 x 512 fp32, 8 experts, top-2, F = 2048, N(0, 0.02) weights,
+    """Configuration 1 of the benchmark set as specified: 4096 x 512 fp32, 8 experts, top-2, F = 2048, N(0, 0.02) weights,
     MSE against zero, seed 0; with the reference's default capacity factor and without dropping.  Besides the
     max-norm tolerance, every row of y and dx is held to it relative to the row's own largest element."""
     for cf in (1.0, 0.0):
