@@ -661,10 +661,26 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
         const bool single = g.offsets == nullptr;
         auto rows_of = [&](int ee) { return single ? g.single_rows : g.kept[ee]; };
         const int nE = single ? 1 : g.E;
-        // rows and first row of the first 64 experts, fetched together: the lookups below then need no further
-        // dependent loads (the scan itself re-reads rows_of through the cache)
-        const int rows_lane = lane < nE ? rows_of(lane) : 0;
-        const int off_lane = (!single && lane < nE) ? g.offsets[lane] : 0;
+        // rows and first row of the first 256 experts, fetched together (lane l holds experts l, l + 64, l + 128,
+        // l + 192): the lookups below then need no further loads.  Fetched where they were needed, each pass of the
+        // search below and the two lookups after it waited for memory in turn - four to five dependent round trips
+        // per tile for experts past the 64th, half of a tile's fixed cost with 256 experts and a contraction of 1024.
+        // (Beyond 256 experts the rest is read through the cache as before.)
+        constexpr int RC = 4;
+        int rows_c[RC], off_c[RC];
+#pragma unroll
+        for (int c = 0; c < RC; ++c) {
+            const int ee = lane + WAVE * c;
+            rows_c[c] = ee < nE ? rows_of(min(ee, nE - 1)) : 0;
+            off_c[c] = (!single && ee < nE) ? g.offsets[min(ee, nE - 1)] : 0;
+        }
+        auto rows_at = [&](int ee) {            // rows of expert ee = base + lane of the caller's pass (ee uniform in ee / 64)
+            int r = 0;
+#pragma unroll
+            for (int c = 0; c < RC; ++c)
+                if ((ee >> 6) == c) r = rows_c[c];
+            return (ee >> 6) < RC ? r : (ee < nE ? rows_of(ee) : 0);
+        };
         // An expert's m-tiles are heavy (more than half a tile of rows) or light: the full tiles and, of the
         // remainder scheme, a remainder above half a tile; with the even split all tiles of an expert alike.
         // Heavy tiles are numbered before light ones, each class in expert order and each XCD taking a contiguous
@@ -683,7 +699,7 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
         };
         int n_h = 0, n_l = 0;
         for (int ee = lane; ee < nE; ee += WAVE) {
-            const int r = ee < WAVE ? rows_lane : rows_of(ee);
+            const int r = rows_at(ee);
             const int hv = heavy_of(r);
             n_h += hv;
             n_l += tiles_of(r) - hv;
@@ -709,7 +725,7 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
         int run = 0, found = -1, before = 0, cnt_found = 1;
         for (int base = 0; base < nE && found < 0; base += WAVE) {
             const int ee = base + lane;
-            const int r = base == 0 ? rows_lane : (ee < nE ? rows_of(ee) : 0);
+            const int r = rows_at(ee);
             const int hv = heavy_of(r);
             const int cnt = (heavy ? hv : tiles_of(r) - hv) * unit;
             int incl = cnt;
@@ -728,7 +744,14 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
         }
         if (found < 0) return;
         e = found;
-        m_ext = found < WAVE ? __shfl(rows_lane, found, WAVE) : rows_of(e);
+        // (found is the same in every lane: the expert's chunk register, then the lane that holds it)
+        {
+            int mv = 0;
+#pragma unroll
+            for (int c = 0; c < RC; ++c)
+                if ((found >> 6) == c) mv = __shfl(rows_c[c], found & 63, WAVE);
+            m_ext = (found >> 6) < RC ? mv : rows_of(e);
+        }
         int mt_class = target - before;
         if (mf) {
             // groups of G n-tiles, an expert's m-tiles of the class inside a group, the group's n-tiles innermost
@@ -745,7 +768,13 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
         mt = mt_class + (heavy ? 0 : heavy_of(m_ext));   // an expert's light tiles follow its heavy ones
         const int t_e = (m_ext + Q_BM - 1) / Q_BM;
         tile_h = TMB == 10 ? ((((m_ext + t_e - 1) / t_e) + 31) & ~31) : Q_BM;
-        row0 = single ? 0 : (found < WAVE ? __shfl(off_lane, found, WAVE) : g.offsets[e]);
+        {
+            int ov = 0;
+#pragma unroll
+            for (int c = 0; c < RC; ++c)
+                if ((found >> 6) == c) ov = __shfl(off_c[c], found & 63, WAVE);
+            row0 = single ? 0 : ((found >> 6) < RC ? ov : g.offsets[e]);
+        }
         k_ext = g.K;
     } else {
         // The contraction length differs from expert to expert, so experts are not handed to XCDs in
