@@ -19,6 +19,7 @@
 #include <math.h>
 
 #include <mutex>
+#include <stdlib.h>
 
 namespace mole {
 
@@ -406,6 +407,18 @@ extern "C" size_t mole_route_workspace_bytes(int S, int E, int k) {
            align256(nb * E * sizeof(float)) + align256((size_t)COLSUM_SLICES * E * sizeof(float));
 }
 
+// Lanes per token (as a power of two) of the kernels that give a group of lanes a token's E values, each lane holding
+// E / lanes of them: 16 lanes at most, more only where a lane would otherwise hold more than 16 values.  A group's
+// reductions act on all the wave's groups at once, so in the top-k, whose rounds are chains of reductions, small groups
+// with many values per lane cost fewer instructions per token than the whole wave on one token (top-8 of 256 scores for 32768 tokens: 106 us with 64 lanes per token,
+// 83 with 32, 72 with 16; top-2 of 64 for 8192: 33.6 / 29.5 / 25.8 us).
+static int lane_group_log2(int E) {
+    int logG = 0;
+    while ((1 << logG) < E && logG < 4) ++logG;
+    while (ceil_div(E, 1 << logG) > 16 && logG < 6) ++logG;
+    return logG;
+}
+
 // The stages of the routing behind the per-block top-k: scan of the histograms over blocks, counts / capacity /
 // offsets / l_aux, then locations and destination rows.  bt: tokens per histogram block.
 static int route_after_topk(int32_t *hist, int32_t *basej, float *colsum, float *colpart, int nb, int bt, int S, int E, int k,
@@ -479,8 +492,7 @@ extern "C" int mole_route(const float *scores, int S, int E, int k, double capac
     ws += align256((size_t)nb * E * sizeof(float));
     float *colpart = (float *)ws;
 
-    int logG = 0;
-    while ((1 << logG) < E && logG < 6) ++logG;
+    const int logG = lane_group_log2(E);
     const int vpl = ceil_div(E, 1 << logG);
     if (vpl <= 1) launch_topk<1>(scores, S, E, k, logG, normalize_gate, idx, loc, gates, hist, colsum, nb, st);
     else if (vpl <= 2) launch_topk<2>(scores, S, E, k, logG, normalize_gate, idx, loc, gates, hist, colsum, nb, st);
@@ -964,7 +976,7 @@ extern "C" int mole_softmax_fwd(const float *logits, const float *logit_bias, in
     if (S == 0) return 0;
     MOLE_REQUIRE(logits && scores, "mole_softmax_fwd: null pointer");
     int logG = 0;
-    while ((1 << logG) < E && logG < 6) ++logG;
+    while ((1 << logG) < E && logG < 6) ++logG;       // (16-lane groups as in the top-k: 18.1 against 17.1 us at 256 experts)
     const int vpl = ceil_div(E, 1 << logG);
     const int tpw = 64 >> logG;
     const dim3 grid(ceil_div(S, 4 * tpw));
