@@ -100,8 +100,8 @@ int mole_softmax_bwd(const float *dscores, const float *scores, int S, int E, fl
 /* The whole of MOLETopk.forward (MOLE/utils/Ugate.py:11-14) in one kernel:
  * scores[S,E] = softmax(x[S,M] . wg[E,M]^T + logit_bias), wg fp32, logit_bias [E] or NULL.
  * bf16 tokens: M a multiple of 128, E <= 256; wg is rounded to bf16 for the products, fp32 accumulation.  Every
- * block of 16 tokens reads all of wg, so beyond a few dozen experts the two-kernel path is the faster one (the
- * Python host side switches at E = 32).
+ * block of 16-64 tokens reads all of wg, so beyond 64 experts the two-kernel path is the faster one (the Python
+ * host side switches there).
  * fp32 tokens: M a multiple of 4, E <= 32, x and wg 16-byte aligned; fp32 FMAs throughout.
  * Other cases use mole_gemm_nt + mole_softmax_fwd. */
 int mole_gate_fwd(const void *x, int dtype, const float *wg, const float *logit_bias, int S, int E, int M,
@@ -148,7 +148,7 @@ int mole_route(const float *scores, int S, int E, int k, double capacity_factor,
                int32_t *counts, int32_t *kept_rows, int32_t *offsets, int32_t *capacity,
                float *l_aux, void *workspace, size_t workspace_bytes, mole_stream_t stream);
 
-/* mole_gate_fwd and mole_route in one call for small gates on bf16 tokens (E <= 32, M a multiple of 128, S >= 1): the gate
+/* mole_gate_fwd and mole_route in one call for small gates on bf16 tokens (E <= 64, M a multiple of 128, S >= 1): the gate
  * kernel goes on to the routing's first stage - top-k, gate values, in-block ranks, histograms - while a token's
  * scores are still in the lanes that formed them, so the routing starts one kernel later and never reads the scores
  * back (MOLE/utils/Ugate.py:11-14 followed by extract_critical, MOLE/moe/layer.py:442-446).  Arguments and results are

@@ -48,16 +48,16 @@ def softmax_fwd(logits: torch.Tensor, logit_bias: Optional[torch.Tensor] = None)
 
 def gate_fwd(x: torch.Tensor, wg: torch.Tensor, logit_bias: Optional[torch.Tensor] = None,
              fused: Optional[bool] = None) -> torch.Tensor:
-    """scores [S,E] fp32 = softmax(x @ wg.T + logit_bias): one fused kernel for small gates (E <= 32; bf16 tokens
-    with M % 128 == 0, where a block of 16 tokens re-reads all of wg, which only pays while wg is small, or fp32
-    tokens with M % 4 == 0), the NT GEMM followed by the softmax kernel otherwise.  fused=True asks for the
+    """scores [S,E] fp32 = softmax(x @ wg.T + logit_bias): one fused kernel for small gates (bf16 tokens with
+    M % 128 == 0 and E <= 64, where a block of 16-64 tokens re-reads all of wg, which only pays while wg is small, or
+    fp32 tokens with M % 4 == 0 and E <= 32), the NT GEMM followed by the softmax kernel otherwise.  fused=True asks for the
     one-kernel path where the kernel allows it (bf16: any E <= 256)."""
     _dev(x), _dev(wg)
     S, M = x.shape
     E = wg.shape[0]
     if fused is None:
-        fused = wg.dtype == torch.float32 and E <= 32 and (
-            (x.dtype == torch.bfloat16 and M % 128 == 0) or (x.dtype == torch.float32 and M % 4 == 0))
+        fused = wg.dtype == torch.float32 and (
+            (x.dtype == torch.bfloat16 and M % 128 == 0 and E <= 64) or (x.dtype == torch.float32 and M % 4 == 0 and E <= 32))
     if fused:
         scores = torch.empty(S, E, dtype=torch.float32, device=x.device)
         L.check(L.lib().mole_gate_fwd(L.ptr(x), L.dtype_code(x.dtype), L.ptr(wg), L.ptr(logit_bias), S, E, M, L.ptr(scores),
@@ -202,7 +202,7 @@ def route(scores: torch.Tensor, top_k: int, capacity_factor: float = 1.0, normal
 
 def gate_route_fused(x: torch.Tensor, wg: torch.Tensor) -> bool:
     """Whether gate_route() takes (x, wg) in its one-call form."""
-    return (x.dtype == torch.bfloat16 and wg.dtype == torch.float32 and wg.shape[0] <= 32 and x.shape[1] % 128 == 0
+    return (x.dtype == torch.bfloat16 and wg.dtype == torch.float32 and wg.shape[0] <= 64 and x.shape[1] % 128 == 0
             and x.shape[0] >= 1)
 
 

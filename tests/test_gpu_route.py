@@ -201,6 +201,7 @@ def test_route_random_sweep():
     (33, 20, 128, 2, 0.0, False, True, False), (777, 32, 384, 4, 0.5, True, False, True),
     (64, 3, 128, 3, 1.0, False, True, True), (1, 5, 128, 1, 1.0, False, True, True),
     (4095, 17, 256, 5, -0.5, True, True, False), (8192, 32, 2048, 2, 0.0, False, True, True),
+    (8192, 64, 2048, 2, 1.0, False, True, True), (16500, 48, 1024, 3, 1.25, True, True, True), (301, 33, 128, 8, 0.5, True, False, False),
 ])
 def test_gate_and_route_in_one_call(S, E, M, k, cf, bias, normalize, ragged):
     """mole_gate_route (the gate kernel does the routing's first stage on the scores it has just formed) against
