@@ -85,6 +85,7 @@ struct GemmArgs {
     void *colsum;           // weight gradients, direct-to-LDS kernels: [E][M] (side 1) or [E][N] (side 2) sums of an operand
     int colsum_side;        //   over the expert's rows: 1 = the m-side operand (A), 2 = the n-side operand (B)
     int wg_expert_major;    // weight gradients, 256-wide kernel: all (m-tile, n-tile) blocks of an expert on one XCD
+    int m_fastest_from;     //   ... for experts with at least this many m-tiles (of the class); the others n-tile first
     int m_fastest;          // row-ragged products, 256-wide kernel: number an expert's tiles m-tile first (see gemm256.hip)
 };
 

@@ -716,7 +716,13 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
         // run side by side on an XCD are then a few m-tiles times all n-tiles, i.e. they stream the expert's whole
         // weight matrix through the L2 once per group of m-tiles.  m-tile first (m_fastest): an expert's tiles are
         // numbered n-tile by n-tile, all its m-tiles of the class inside; the blocks side by side are then all
-        // m-tiles of the expert times a few n-tiles, and every weight panel is fetched once.
+        // m-tiles of the expert times a few n-tiles, and every weight panel is fetched once.  In between (m_fastest =
+        // G > 1): groups of G n-tiles with the expert's m-tiles inside, so that the 32 blocks of an XCD are about
+        // 32 / G m-tiles times G n-tiles and fetch 32 / G + G panels between them instead of 1 + 32.  The two products
+        // with a contraction over M and wide results (h = xd.w1^T + b1, t = (go.w2^T) gelu'(h)) use G = 8 for experts
+        // of at least m_fastest_from = 8 m-tiles (8192 tokens, 64 experts of 2048 -> 8192, top-2, skewed loads: 798 ->
+        // 766 and 777 -> 752 us); for experts of four or five m-tiles it is the slower order (16 experts of about 1024
+        // rows, 1024 -> 4096: +6 and +3 us), so those keep n-tile first.
         const bool mf = g.m_fastest != 0;
         const int unit = mf ? n_tiles : 1;       // tiles per counted m-tile
         const int target = mf ? t : t / n_tiles;
@@ -753,7 +759,11 @@ __global__ __launch_bounds__((Tile<TMB, WM>::THREADS), (Tile<TMB, WM>::BLOCKS_PE
             m_ext = (found >> 6) < RC ? mv : rows_of(e);
         }
         int mt_class = target - before;
-        if (mf) {
+        if (mf && cnt_found / n_tiles < g.m_fastest_from) {
+            // an expert with few m-tiles keeps the n-tile-first order (its tiles are counted one by one here)
+            nt = mt_class % n_tiles;
+            mt_class /= n_tiles;
+        } else if (mf) {
             // groups of G n-tiles, an expert's m-tiles of the class inside a group, the group's n-tiles innermost
             // (G = 1: m-tile first; the last group may be short)
             const int c_e = cnt_found / n_tiles;      // the expert's m-tiles of this class
@@ -925,21 +935,23 @@ static int launch256(GemmArgs g, int tiles, hipStream_t st, int kid) {
     return 0;
 }
 
-// Launch options that were measured and are off by default; a -DMOLE_TUNING build reads them from the environment
-// (MOLE_MFAST: bit mask of the products that number an XCD's tiles m-tile first, MOLE_MFAST_G: n-tiles per group of
-// that order, MOLE_WG_EMAJOR: expert count from which a weight gradient keeps an expert's blocks on one XCD,
+// Launch options and their defaults; a -DMOLE_TUNING build reads them from the environment
+// (MOLE_MFAST: bit mask of the products that number an expert's tiles m-tile first within groups of MOLE_MFAST_G
+// n-tiles, MOLE_MFAST_FROM: m-tiles an expert needs for that order, MOLE_WG_EMAJOR: expert count from which a weight gradient keeps an expert's blocks on one XCD,
 // MOLE_TMB: 4 | 8 = four-wave tiles of 128 | 256 rows, 16 = the 256-row eight-wave tile for every product,
 // MOLE_NO_SUMS: bias gradients from their own kernel).
 #ifdef MOLE_TUNING
 static int env_int(const char *name, int dflt) { const char *v = getenv(name); return v ? atoi(v) : dflt; }
-static int m_fastest_mask() { static const int v = env_int("MOLE_MFAST", 0); return v; }
-static int m_fastest_group() { static const int v = env_int("MOLE_MFAST_G", 1); return v > 0 ? v : 1; }
+static int m_fastest_mask() { static const int v = env_int("MOLE_MFAST", 9); return v; }
+static int m_fastest_group() { static const int v = env_int("MOLE_MFAST_G", 8); return v > 0 ? v : 1; }
+static int m_fastest_from() { static const int v = env_int("MOLE_MFAST_FROM", 8); return v; }
 static int wg_emajor_from() { static const int v = env_int("MOLE_WG_EMAJOR", 128); return v; }
 static int forced_tile() { static const int v = env_int("MOLE_TMB", 0); return v; }
 static bool sums_off() { static const bool v = getenv("MOLE_NO_SUMS") != nullptr; return v; }
 #else
-static int m_fastest_mask() { return 0; }
-static int m_fastest_group() { return 1; }
+static int m_fastest_mask() { return 9; }        // h = xd.w1^T + b1 and t = (go.w2^T) gelu'(h)
+static int m_fastest_group() { return 8; }
+static int m_fastest_from() { return 8; }
 static int wg_emajor_from() { return 128; }
 static int forced_tile() { return 0; }
 static bool sums_off() { return false; }
@@ -964,6 +976,7 @@ static int dispatch256(const GemmArgs &g, bool b_ks, bool wg, int epi, int max_r
     const int rows_bound = g.offsets ? max_rows : g.single_rows;
     GemmArgs gg = g;
     gg.m_fastest = ((m_fastest_mask() >> kid) & 1) ? m_fastest_group() : 0;
+    gg.m_fastest_from = m_fastest_from();
     // (+ 16: the heavy and the light tiles of an XCD are rounded up to whole slots separately)
     const int tiles = (((rows_bound / BM + (g.offsets ? g.E : 1)) * n_tiles + 7) & ~7) + 16;
     if (wg) return -100;
