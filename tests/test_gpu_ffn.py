@@ -54,6 +54,10 @@ CASES = [
     (3, 264, 520, [1500, 3, 321], 5),
     # more than 16 rounds of tiles (the grouped kernel then numbers them in plain expert order)
     (150, 64, 4096, [257 + (11 * e) % 90 for e in range(150)], 0),
+    # experts of eight or more m-tiles (their tiles are numbered in groups of 8 n-tiles, the last group short: 9 and
+    # 11 n-tiles here) beside experts that keep the plain order, one of them with a remainder tile of its own class
+    (4, 64, 2304, [2100, 300, 0, 2600], 0),
+    (3, 128, 2816, [2049, 1793, 2305], 8),
 ]
 
 
