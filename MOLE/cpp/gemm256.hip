@@ -272,7 +272,7 @@ template <int TMB, int WM, bool M_KS, bool N_KS, bool WG, int TMC> struct Feeder
     }
     // loads [J0, J1) of stage s (the m-side tile's loads come first) into ring buffer buf
     template <int J0, int J1> __device__ __forceinline__ void issue(int s, int buf) {
-        const uint32_t dst = lds_w + buf * SG::BYTES;
+        const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_w + buf * SG::BYTES);
         const bool clamp_k = WG && ragged_k && s >= nk - 1;
 #pragma unroll
         for (int j = J0; j < J1; ++j) {
@@ -301,6 +301,22 @@ __device__ __forceinline__ void unpack4(uint2 u, float *f) {
     f[3] = __uint_as_float(u.y & 0xffff0000u);
 }
 
+// Waits until at most `behind` whole stages of L loads each (behind <= B; below 0 counts as 0), and X more loads if
+// `extra`, are in flight (the instruction takes its count as an immediate, hence the chain).
+template <int B, int L, int X> __device__ __forceinline__ void wait_stages_behind(int behind, bool extra) {
+    if constexpr (B <= 0) {
+        if (extra) __builtin_amdgcn_s_waitcnt(waitcnt_vm(X));
+        else __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));
+    } else {
+        if (behind >= B) {
+            if (extra) __builtin_amdgcn_s_waitcnt(waitcnt_vm(B * L + X));
+            else __builtin_amdgcn_s_waitcnt(waitcnt_vm(B * L));
+        } else {
+            wait_stages_behind<B - 1, L, X>(behind, extra);
+        }
+    }
+}
+
 // The K loop.  Stage s (32 of K) lives in ring buffer s mod NSTAGE and is fetched NSTAGE-1 stages ahead.
 // A wave cannot issue MFMAs while one of its loads waits for the memory pipeline to take it, so the loads
 // of a stage are not issued in one burst: each half of an iteration is cut into parts, and a part issues
@@ -323,7 +339,7 @@ __device__ __forceinline__ void main_loop(const bf16_t *Mp, long ldm, int m0, in
     constexpr int AHEAD = SG::NSTAGE - 1, NP = 4;
     typedef Feeder<TMB, WM, M_KS, N_KS, WG, TMC> FD;
     constexpr int L = FD::L, LH = L / 2;      // loads per wave per stage; the halves are LH and L - LH
-    const int nk = (k_ext + Q_BK - 1) / Q_BK;
+    const int nk = __builtin_amdgcn_readfirstlane((k_ext + Q_BK - 1) / Q_BK);
     if (nk == 0) return;
     FD fd;
     fd.init(Mp, ldm, m0, m_ext, Np, ldn, n0, n_ext, k_ext, smem, wave);
@@ -339,12 +355,23 @@ __device__ __forceinline__ void main_loop(const bf16_t *Mp, long ldm, int m0, in
     // of look-ahead is lost for the later half); with two, all of them go into the half after the barrier.
     constexpr bool SPLIT = AHEAD >= 3;
     constexpr bool NO_LOADS = PART == 1 || PART == 4, NO_READS = PART == 2 || PART == 4, NO_BARRIERS = PART == 3 || PART == 4;
+    // Only stages that exist are fetched (but for one part of a stage, see below): the prologue stops at the
+    // contraction's last stage, the last iterations issue nothing, and the waits count what is really in flight.
+    // Fetching AHEAD stages past the end, as a loop with one kind of iteration does, costs a tile of K = 1024 a tenth
+    // more loads, a one-stage tile of a nearly empty expert four times its loads, and the epilogue a wait for loads
+    // that nothing reads.  The iterations without loads are a second copy of the loop body, compiled without them: the
+    // same body with the loads under a (wave-uniform) condition ran 3-10 % slower, and a third copy for the one
+    // iteration in between made the register allocator spill.
+    constexpr int LX = SPLIT ? LH : L;        // loads of stage AHEAD - 1 that the prologue issues
     if constexpr (!NO_LOADS) {
 #pragma unroll
-        for (int s = 0; s < AHEAD - 1; ++s) fd.template issue<0, L>(s, s);
-        fd.template issue<0, SPLIT ? LH : L>(AHEAD - 1, AHEAD - 1);
+        for (int s = 0; s < AHEAD - 1; ++s)
+            if (s < nk) fd.template issue<0, L>(s, s);
+        if (AHEAD - 1 < nk) fd.template issue<0, LX>(AHEAD - 1, AHEAD - 1);
     }
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm((AHEAD - 2) * L + (SPLIT ? LH : L)));
+    // stage 0 has landed when no more is in flight than what was issued after it
+    if (nk >= AHEAD) __builtin_amdgcn_s_waitcnt(waitcnt_vm((AHEAD - 2) * L + LX));
+    else wait_stages_behind<AHEAD - 2, L, 0>(nk - 1, false);
     __builtin_amdgcn_s_barrier();
     if constexpr (BIAS) {
 #pragma unroll
@@ -362,32 +389,43 @@ __device__ __forceinline__ void main_loop(const bf16_t *Mp, long ldm, int m0, in
     f0.read(smem, wm, wn, 0);
     if constexpr (NO_READS) f1.read(smem, wm, wn, 1);
     int cur_b = 0;                    // ring buffer of stage s
-    for (int s = 0; s < nk; ++s) {
-        const int nxt_b = cur_b + 1 == SG::NSTAGE ? 0 : cur_b + 1;
-        const int free_b = cur_b == 0 ? SG::NSTAGE - 1 : cur_b - 1;     // held stage s-1, takes stage s+AHEAD
-        const int fill_b = free_b == 0 ? SG::NSTAGE - 1 : free_b - 1;   // takes the rest of stage s+AHEAD-1
-        const char *cur = smem + cur_b * SG::BYTES;
-        const char *nxt = smem + nxt_b * SG::BYTES;
-#define MOLE_HALF(P, J0, N, S_LOAD, BUF, FR, STAGE_PTR, KK, FM)                                           \
-        if constexpr (!NO_LOADS) fd.template issue<(J0) + part_lo<P, NP, (N)>(), (J0) + part_lo<P + 1, NP, (N)>()>(S_LOAD, BUF); \
+#define MOLE_HALF(ISSUE, P, J0, N, S_LOAD, BUF, FR, STAGE_PTR, KK, FM)                                    \
+        if constexpr (!NO_LOADS && (ISSUE)) fd.template issue<(J0) + part_lo<P, NP, (N)>(), (J0) + part_lo<P + 1, NP, (N)>()>(S_LOAD, BUF); \
         if constexpr (!NO_READS) FR.template read_part<P, NP>(STAGE_PTR, wm, wn, KK);                       \
         FM.template mma_part<P, NP, SUM>(acc, sums, wm, wn);                                              \
         __builtin_amdgcn_sched_barrier(0);
-        MOLE_HALF(0, SPLIT ? LH : 0, SPLIT ? L - LH : 0, s + AHEAD - 1, fill_b, f1, cur, 1, f0)
-        MOLE_HALF(1, SPLIT ? LH : 0, SPLIT ? L - LH : 0, s + AHEAD - 1, fill_b, f1, cur, 1, f0)
-        MOLE_HALF(2, SPLIT ? LH : 0, SPLIT ? L - LH : 0, s + AHEAD - 1, fill_b, f1, cur, 1, f0)
-        MOLE_HALF(3, SPLIT ? LH : 0, SPLIT ? L - LH : 0, s + AHEAD - 1, fill_b, f1, cur, 1, f0)
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm((AHEAD - 2) * L));
-        if constexpr (!NO_BARRIERS) __builtin_amdgcn_s_barrier();
-        __builtin_amdgcn_sched_barrier(0);
-        fix_tail(s + 1, nxt_b);
-        MOLE_HALF(0, 0, SPLIT ? LH : L, s + AHEAD, free_b, f0, nxt, 0, f1)
-        MOLE_HALF(1, 0, SPLIT ? LH : L, s + AHEAD, free_b, f0, nxt, 0, f1)
-        MOLE_HALF(2, 0, SPLIT ? LH : L, s + AHEAD, free_b, f0, nxt, 0, f1)
-        MOLE_HALF(3, 0, SPLIT ? LH : L, s + AHEAD, free_b, f0, nxt, 0, f1)
-#undef MOLE_HALF
-        cur_b = nxt_b;
+    // One iteration (stage s).  ISSUE: the first half issues the rest of stage s + AHEAD - 1, the second the first
+    // loads of stage s + AHEAD; WAIT: the wait for stage s + 1.
+#define MOLE_ITER(ISSUE, WAIT)                                                                            \
+    {                                                                                                     \
+        const int nxt_b = cur_b + 1 == SG::NSTAGE ? 0 : cur_b + 1;                                        \
+        const int free_b = cur_b == 0 ? SG::NSTAGE - 1 : cur_b - 1;     /* held stage s-1, takes stage s+AHEAD */ \
+        const int fill_b = free_b == 0 ? SG::NSTAGE - 1 : free_b - 1;   /* takes the rest of stage s+AHEAD-1 */   \
+        const char *cur = smem + cur_b * SG::BYTES;                                                       \
+        const char *nxt = smem + nxt_b * SG::BYTES;                                                       \
+        MOLE_HALF(ISSUE, 0, SPLIT ? LH : 0, SPLIT ? L - LH : 0, s + AHEAD - 1, fill_b, f1, cur, 1, f0)    \
+        MOLE_HALF(ISSUE, 1, SPLIT ? LH : 0, SPLIT ? L - LH : 0, s + AHEAD - 1, fill_b, f1, cur, 1, f0)    \
+        MOLE_HALF(ISSUE, 2, SPLIT ? LH : 0, SPLIT ? L - LH : 0, s + AHEAD - 1, fill_b, f1, cur, 1, f0)    \
+        MOLE_HALF(ISSUE, 3, SPLIT ? LH : 0, SPLIT ? L - LH : 0, s + AHEAD - 1, fill_b, f1, cur, 1, f0)    \
+        WAIT;                                                                                             \
+        if constexpr (!NO_BARRIERS) __builtin_amdgcn_s_barrier();                                         \
+        __builtin_amdgcn_sched_barrier(0);                                                                \
+        fix_tail(s + 1, nxt_b);                                                                           \
+        MOLE_HALF(ISSUE, 0, 0, SPLIT ? LH : L, s + AHEAD, free_b, f0, nxt, 0, f1)                         \
+        MOLE_HALF(ISSUE, 1, 0, SPLIT ? LH : L, s + AHEAD, free_b, f0, nxt, 0, f1)                         \
+        MOLE_HALF(ISSUE, 2, 0, SPLIT ? LH : L, s + AHEAD, free_b, f0, nxt, 0, f1)                         \
+        MOLE_HALF(ISSUE, 3, 0, SPLIT ? LH : L, s + AHEAD, free_b, f0, nxt, 0, f1)                         \
+        cur_b = nxt_b;                                                                                    \
     }
+    int s = 0;
+    // while stage s + AHEAD - 1 exists: its rest is issued, then the first loads of stage s + AHEAD (in the last of
+    // these iterations that stage does not exist: LX loads that nothing reads, the only ones of a tile)
+    for (; s + AHEAD - 1 < nk; ++s) MOLE_ITER(true, __builtin_amdgcn_s_waitcnt(waitcnt_vm((AHEAD - 2) * L)))
+    // the last AHEAD - 1 iterations issue nothing; in flight behind stage s + 1: the stages after it and those LX loads
+    const bool extra = nk >= AHEAD;
+    for (; s < nk; ++s) MOLE_ITER(false, (wait_stages_behind<AHEAD - 2, L, LX>(nk - 2 - s, extra)))
+#undef MOLE_ITER
+#undef MOLE_HALF
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(0));   // nothing may still be writing LDS when the block retires
 }
 
